@@ -1,0 +1,162 @@
+/*
+ * sparse_mlp_amd.h — C ABI of the MI355X (gfx950) sparse-MLP decode path.
+ *
+ * Plain pointers and sizes only: every `const void*` / `void*` below is a
+ * DEVICE pointer unless its comment says "host"; `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream).  All entry points return
+ * ST_OK (0) or a negative st_status; st_last_error() gives a message for the
+ * calling thread.  No entry point except st_cache_create/st_cache_destroy
+ * (host memory only) and st_cache_sync_state (one small device-to-host copy)
+ * allocates or synchronises: work is enqueued on `stream` and ordered with
+ * whatever else the caller enqueues there.
+ *
+ * Each entry point names the interface of NimbleEdge/sparse_transformers it
+ * replaces (paths relative to that repository).
+ */
+#ifndef SPARSE_MLP_AMD_H
+#define SPARSE_MLP_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum st_status {
+    ST_OK = 0,
+    ST_ERR_ARG = -1,       /* bad shape / alignment / null pointer / unsupported size */
+    ST_ERR_NO_ACTIVE = -2, /* update left the cache empty: the reference's "No active weights" */
+    ST_ERR_HIP = -3,       /* a HIP runtime call failed */
+    ST_ERR_INVALID = -4    /* cache has no valid contents yet: the reference's "Cache is not valid" */
+} st_status;
+
+typedef enum st_dtype { ST_F32 = 0, ST_F16 = 1, ST_BF16 = 2 } st_dtype;
+
+typedef enum st_act {
+    ST_ACT_RELU = 0,      /* what sparse_mlp_op.cpp:157,183 computes */
+    ST_ACT_SILU = 1,      /* ACT2FN["silu"], src/modeling_skip.py:65,116 */
+    ST_ACT_GELU_TANH = 2, /* "gelu_pytorch_tanh" (gemma3n) */
+    ST_ACT_SIGMOID = 3,   /* what sparse_mlp_cuda.cu:83 computes */
+    ST_ACT_IDENTITY = 4
+} st_act;
+
+int st_version(void);
+/* host; message of the last failing call made by this thread ("" if none) */
+const char *st_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * Sparse MLP forward.
+ * Replaces sparse_mlp_forward / sparse_mlp_forward_cpu
+ * (sparse_transformers/csrc/sparse_mlp_op.cpp:53-76,79-192), the Python path
+ * SkipMLP._forward_sparse_weight_cache (src/modeling_skip.py:114-117) and the
+ * ungated OPTSkipMLP variant (src/models/opt/modelling_opt_skip.py:116-119).
+ *
+ *   x          [B,H]   activations, dtype `dtype`
+ *   gate_rows  [n,H]   active gate rows (NULL when !has_gate): concat_weight[:n]
+ *   up_rows    [n,H]   active up rows: concat_weight[n:2n] (concat_weight when ungated)
+ *   down_rows  [n,H]   active down columns, packed one per row: the memory
+ *                      behind active_down_weight ([H,n], strides (1,H))
+ *   n                  host-side active count; rows >= n are never read
+ *   n_dev              optional device int32: when non-NULL the kernels use
+ *                      min(*n_dev, n) instead, so a cache update and the
+ *                      forward can be enqueued back to back with no host read
+ *   out        [B,H]   dtype `dtype`   (the reference's down_proj_buffer)
+ *   combined   [B,ldc] dtype `dtype`, optional (NULL = skip): receives
+ *                      act(gate)*up in columns [0,n) and, when gated, the raw
+ *                      up projection in [n,2n) — what the in-place operator
+ *                      leaves in combined_proj_buffer
+ *   workspace          float scratch of st_mlp_workspace_bytes(B,H) bytes
+ * All rows must be 16-byte aligned (H*sizeof(dtype) % 16 == 0). B <= 4096.
+ * ------------------------------------------------------------------------ */
+int64_t st_mlp_workspace_bytes(int64_t B, int64_t H);
+int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
+                   const void *down_rows, int64_t n, const int32_t *n_dev, void *out, void *combined, int64_t ldc,
+                   void *workspace, int64_t workspace_bytes, int act, int dtype, int has_gate, void *stream);
+
+/* ------------------------------------------------------------------------
+ * LoRA predictor -> threshold mask -> union over rows, on the device.
+ * Replaces FastLoRAProjection.forward (src/modeling_skip.py:52-53) and the
+ * "naive" branch plus any(dim=0) of SkipDecoderLayer._compute_binary_mask
+ * (src/modeling_skip.py:204-207,214), generalised from 0 to a scalar
+ * threshold.
+ *
+ *   x [B,H], A [r,H] (down.weight), Bm [I,r] (up.weight), all dtype `dtype`
+ *   t_ws    float [B,r] scratch (the rank-r intermediate, kept in fp32)
+ *   scores  optional float [B,I] (NULL = not written)
+ *   mask    uint8 [I]: mask[i] = any_b(score[b,i] >= thr)  (cmp_ge != 0)
+ *                               any_b(score[b,i] >  thr)  (cmp_ge == 0)
+ * H*sizeof(dtype) and r*sizeof(dtype) must be multiples of 16. B <= 64.
+ * ------------------------------------------------------------------------ */
+int st_predictor_mask(const void *x, int64_t B, int64_t H, const void *A, int64_t r, const void *Bm, int64_t I,
+                      int dtype, float thr, int cmp_ge, float *t_ws, float *scores, uint8_t *mask, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Differential weight cache, resident in HBM.
+ * Replaces class WeightCache (sparse_transformers/csrc/weight_cache.h:13-381)
+ * as registered in sparse_mlp_op.cpp:198-202.  The caller owns every device
+ * buffer (so a torch allocator, or plain hipMalloc, can provide them); the
+ * handle only holds host-side bookkeeping.
+ * ------------------------------------------------------------------------ */
+typedef struct st_cache_buffers {
+    /* pools: all rows, never modified after st_cache_load_weights */
+    void *gate_pool;   /* [I,H] (NULL when !has_gate) */
+    void *up_pool;     /* [I,H] */
+    void *downT_pool;  /* [I,H]: row i = column i of the [H,I] down matrix */
+    /* packed active rows, capacity I rows each; first n_active rows valid */
+    void *gate_active; /* [I,H] (NULL when !has_gate) */
+    void *up_active;   /* [I,H] */
+    void *down_active; /* [I,H] */
+    int32_t *indices;  /* [I] ordered active list (the reference's active_indices) */
+    uint8_t *cur_mask; /* [I] the reference's current_mask */
+    int32_t *state;    /* [ST_STATE_WORDS] see st_state_word */
+    int32_t *scratch;  /* [2*I] work lists of one update */
+} st_cache_buffers;
+
+enum st_state_word {
+    ST_STATE_N_ACTIVE = 0,  /* number of valid rows in the active buffers */
+    ST_STATE_N_CHANGED = 1, /* rows rewritten by the last update */
+    ST_STATE_STATUS = 2,    /* 0 ok, ST_ERR_NO_ACTIVE after an update that emptied the cache */
+    ST_STATE_VALID = 3,     /* the reference's cache_valid */
+    ST_STATE_N_ADDED = 4,   /* |new & ~old| of the last update */
+    ST_STATE_N_REMOVED = 5, /* |old & ~new| of the last update */
+    ST_STATE_SERIAL = 6,    /* updates that changed something */
+    ST_STATE_WORDS = 8
+};
+
+typedef struct st_cache st_cache;
+
+/* Largest intermediate size the update kernel supports (its index maps live in LDS). */
+int64_t st_cache_max_intermediate(void);
+
+/* host only.  weight_cache.h:148-194 (allocation is the caller's). */
+st_cache *st_cache_create(const st_cache_buffers *bufs, int64_t I, int64_t H, int dtype, int has_gate);
+void st_cache_destroy(st_cache *c);
+
+/* Fill the pools (down [H,I] is transposed on the device) and reset the
+ * bookkeeping to "nothing active, current_mask = 0": weight_cache.h:199-223.
+ * gate/up [I,H], down [H,I], dtype of the cache; gate may be NULL when ungated. */
+int st_cache_load_weights(st_cache *c, const void *gate, const void *up, const void *down, void *stream);
+
+/* update_active_weights(mask): weight_cache.h:229-359 (diff :84-110, pairing
+ * :248-277, append :280-307, swap-with-last :310-353).  mask: uint8/bool [I]
+ * on the device.  Enqueues a plan kernel and a row-copy kernel; returns
+ * without waiting.  An update that empties the cache sets
+ * state[ST_STATE_STATUS] = ST_ERR_NO_ACTIVE and, like the reference, leaves
+ * cur_mask unchanged. */
+int st_cache_update_async(st_cache *c, const uint8_t *mask, void *stream);
+
+/* Copies the state words to the host (waits for `stream`).  Returns
+ * ST_ERR_NO_ACTIVE if the last update emptied the cache, else ST_OK.
+ * state_out: host int32[ST_STATE_WORDS], may be NULL. */
+int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream);
+
+/* get_concat_weight(): weight_cache.h:113-145,362-366.  Writes the contiguous
+ * [2n,H] (gate rows then up rows; [n,H] when ungated) tensor into dst, for
+ * callers that need the reference's tensor; n is the host's count from the
+ * last st_cache_sync_state. */
+int st_cache_materialize_concat(st_cache *c, void *dst, int64_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPARSE_MLP_AMD_H */

@@ -1,0 +1,21 @@
+"""MI355X-native sparse-MLP decode path (LoRA predictor -> mask -> differential weight cache ->
+fused gate/up/activation/down) behind the operator API of NimbleEdge/sparse_transformers.
+
+Unlike the reference's ``sparse_transformers/__init__.py`` nothing global is changed at import
+(no thread-count or JIT settings).  The HIP library is loaded on first use and there is no CPU
+fallback: without the built library, or without a GPU tensor, calls raise.
+"""
+from .ops import predictor_mask, predictor_scores, sparse_mlp_forward
+from .skip_mlp import FastLoRAProjection, SkipMLP, SparseDecodeLayer, SparseMLPStack
+from .weight_cache import WeightCache
+
+__all__ = [
+    "sparse_mlp_forward",
+    "WeightCache",
+    "predictor_mask",
+    "predictor_scores",
+    "FastLoRAProjection",
+    "SkipMLP",
+    "SparseDecodeLayer",
+    "SparseMLPStack",
+]

@@ -1,0 +1,53 @@
+"""Compile the HIP sources under csrc/ into libsparse_mlp_amd.so (gfx950 only).
+
+Usage:  python -m sparse_transformers_amd.build
+The library is built in-tree, next to this file, so that it travels with the
+source tree; nothing is installed.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_NAME = "libsparse_mlp_amd.so"
+LIB_PATH = os.path.join(HERE, LIB_NAME)
+SOURCES = ["capi.hip", "mlp_decode.hip", "mlp_prefill.hip", "predictor.hip", "cache.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _compile(src: str, obj: str) -> None:
+    subprocess.run([HIPCC, *FLAGS, "-c", src, "-o", obj], check=True)
+
+
+def build(verbose: bool = True) -> str:
+    build_dir = os.path.join(HERE, "build")
+    os.makedirs(build_dir, exist_ok=True)
+    srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    objs = [os.path.join(build_dir, s.replace(".hip", ".o")) for s in srcs]
+    if verbose:
+        print(f"[build] hipcc gfx950: {', '.join(srcs)}", flush=True)
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
+        list(ex.map(lambda so: _compile(os.path.join(CSRC, so[0]), so[1]), zip(srcs, objs)))
+    subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs], check=True)
+    if verbose:
+        print(f"[build] wrote {LIB_PATH}", flush=True)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

@@ -1,0 +1,394 @@
+// Differential weight cache resident in HBM.
+//
+// update = one "plan" kernel (a single 1024-thread workgroup doing only
+// integer bookkeeping in LDS) + one "copy" kernel (16-byte row copies).
+//
+// The plan kernel replays WeightCache::update_active_weights
+// (sparse_transformers/csrc/weight_cache.h:229-359) exactly:
+//   diff      ascending added / removed lists     (weight_cache.h:84-110)
+//   phase 1   i-th removed position <- i-th added  (:248-277)   parallel
+//   phase 2   surplus additions appended           (:280-307)   parallel
+//   phase 3   surplus removals, swap-with-last     (:310-353)   one lane,
+//             because each step depends on the list the previous one left
+// It only decides WHICH index ends up at WHICH position.  Because every active
+// row is a bit-copy of a pool row, the data movement never has to follow the
+// sequential order: the copy kernel rewrites each position whose index
+// changed straight from the pool (no reads of the active buffers, hence no
+// hazards between copies).
+#include "st_common.h"
+
+#include <new>
+
+namespace st {
+
+constexpr int kPlanThreads = 1024;
+constexpr int kPlanWaves = kPlanThreads / kWave;
+constexpr uint16_t kNone = 0xffffu;
+// LDS per intermediate element: pos(2) + idx(2) + removed list(2) + flags(1) + dirty(1/8)
+constexpr int64_t kPlanMaxI = 22000;
+
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane)
+{
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const uint32_t o = __shfl_up(v, off, kWave);
+        if (lane >= off) v += o;
+    }
+    return v;
+}
+
+// Exclusive scan of one uint32 per thread over the block; *total receives the sum.
+__device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wave_tot, uint32_t *total)
+{
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const uint32_t incl = wave_incl_scan(v, lane);
+    __syncthreads();  // protect wave_tot from the previous use
+    if (lane == kWave - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    uint32_t prefix = 0, tot = 0;
+    for (int w = 0; w < kPlanWaves; ++w) {
+        const uint32_t t = wave_tot[w];
+        if (w < wave) prefix += t;
+        tot += t;
+    }
+    *total = tot;
+    return prefix + incl - v;
+}
+
+__global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t *__restrict__ new_mask,
+                                                                  uint8_t *__restrict__ cur_mask,
+                                                                  int32_t *__restrict__ indices,
+                                                                  int32_t *__restrict__ state,
+                                                                  int32_t *__restrict__ scratch, int I)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);  // index -> position
+    uint16_t *idx_l = pos_l + I;                           // position -> index
+    uint16_t *rem_l = idx_l + I;                           // ascending removed indices
+    uint32_t *dirty = reinterpret_cast<uint32_t *>(rem_l + I + (I & 1));  // bit per position
+    const int dirty_words = (I + 31) >> 5;
+    uint8_t *flag_l = reinterpret_cast<uint8_t *>(dirty + dirty_words);   // bit0 new, bit1 old
+    __shared__ uint32_t wave_tot[kPlanWaves];
+    __shared__ int n_new_s;
+
+    int32_t *added_g = scratch;        // [I] ascending added indices
+    int32_t *changed_g = scratch + I;  // [I] positions to rewrite
+
+    const int tid = threadIdx.x;
+    const int n = state[ST_STATE_N_ACTIVE];
+
+    for (int i = tid; i < I; i += kPlanThreads) {
+        pos_l[i] = kNone;
+        flag_l[i] = (new_mask[i] ? 1 : 0) | (cur_mask[i] ? 2 : 0);
+    }
+    for (int w = tid; w < dirty_words; w += kPlanThreads) dirty[w] = 0u;
+    __syncthreads();
+    for (int p = tid; p < n; p += kPlanThreads) {
+        const int idx = indices[p];
+        idx_l[p] = (uint16_t)idx;
+        pos_l[idx] = (uint16_t)p;
+    }
+
+    // ---- diff: contiguous element range per thread keeps the lists ascending
+    const int E = (I + kPlanThreads - 1) / kPlanThreads;
+    const int e0 = tid * E < I ? tid * E : I, e1 = e0 + E < I ? e0 + E : I;
+    uint32_t cnt = 0;  // added in the low half, removed in the high half
+    for (int i = e0; i < e1; ++i) {
+        const uint8_t f = flag_l[i];
+        cnt += (f == 1) ? 1u : 0u;
+        cnt += (f == 2) ? 0x10000u : 0u;
+    }
+    uint32_t total;
+    const uint32_t off = block_excl_scan(cnt, wave_tot, &total);  // contains __syncthreads
+    const int na = (int)(total & 0xffffu), nr = (int)(total >> 16);
+    if (na == 0 && nr == 0) {  // unchanged mask: nothing is touched (weight_cache.h:237-240)
+        if (tid == 0) {
+            state[ST_STATE_N_CHANGED] = 0;
+            state[ST_STATE_N_ADDED] = 0;
+            state[ST_STATE_N_REMOVED] = 0;
+        }
+        return;
+    }
+    {
+        int oa = (int)(off & 0xffffu), orr = (int)(off >> 16);
+        for (int i = e0; i < e1; ++i) {
+            const uint8_t f = flag_l[i];
+            if (f == 1) added_g[oa++] = i;
+            if (f == 2) rem_l[orr++] = (uint16_t)i;
+        }
+    }
+    __syncthreads();
+
+    const int pairs = na < nr ? na : nr;
+    // ---- phase 1: paired replacement
+    for (int i = tid; i < pairs; i += kPlanThreads) {
+        const int e = rem_l[i];
+        const uint16_t p = pos_l[e];
+        if (p != kNone) {
+            const int a = added_g[i];
+            idx_l[p] = (uint16_t)a;
+            pos_l[a] = p;
+            pos_l[e] = kNone;
+            atomicOr(&dirty[p >> 5], 1u << (p & 31));
+        }
+    }
+    // ---- phase 2: append surplus additions
+    for (int i = pairs + tid; i < na; i += kPlanThreads) {
+        const int p = n + (i - pairs);
+        if (p < I) {
+            const int a = added_g[i];
+            idx_l[p] = (uint16_t)a;
+            pos_l[a] = (uint16_t)p;
+            atomicOr(&dirty[p >> 5], 1u << (p & 31));
+        }
+    }
+    __syncthreads();
+
+    // ---- phase 3: surplus removals, sequential by construction
+    if (tid == 0) {
+        int m = n + (na - pairs);
+        if (m > I) m = I;
+        for (int k = pairs; k < nr; ++k) {
+            const int e = rem_l[k];
+            const uint16_t p = pos_l[e];
+            if (p == kNone) continue;
+            if (m <= 0) break;
+            const int last = m - 1;
+            if ((int)p != last) {
+                const uint16_t li = idx_l[last];
+                idx_l[p] = li;
+                pos_l[li] = p;
+                dirty[p >> 5] |= 1u << (p & 31);
+            }
+            --m;
+            pos_l[e] = kNone;
+        }
+        n_new_s = m;
+    }
+    __syncthreads();
+    const int n_new = n_new_s;
+
+    // ---- compact the dirty positions below n_new into the copy list
+    uint32_t word = 0;
+    if (tid < dirty_words) {
+        word = dirty[tid];
+        const int lo = tid << 5;
+        if (lo >= n_new) word = 0;
+        else if (lo + 32 > n_new) word &= (1u << (n_new - lo)) - 1u;
+    }
+    uint32_t n_changed;
+    uint32_t coff = block_excl_scan((uint32_t)__popc(word), wave_tot, &n_changed);
+    while (word) {
+        const int bit = __ffs(word) - 1;
+        word &= word - 1;
+        const int p = (tid << 5) + bit;
+        changed_g[coff++] = p;
+        indices[p] = idx_l[p];
+    }
+
+    if (n_new > 0) {  // the reference stores the mask only when the rebuild did not throw
+        for (int i = tid; i < I; i += kPlanThreads) cur_mask[i] = flag_l[i] & 1;
+    }
+    if (tid == 0) {
+        state[ST_STATE_N_ACTIVE] = n_new;
+        state[ST_STATE_N_CHANGED] = (int)n_changed;
+        state[ST_STATE_N_ADDED] = na;
+        state[ST_STATE_N_REMOVED] = nr;
+        state[ST_STATE_SERIAL] += 1;
+        if (n_new > 0) {
+            state[ST_STATE_STATUS] = 0;
+            state[ST_STATE_VALID] = 1;
+        } else {
+            state[ST_STATE_STATUS] = ST_ERR_NO_ACTIVE;
+        }
+    }
+}
+
+struct CopyPlan {
+    const unsigned char *pool[3];
+    unsigned char *active[3];
+    int nmat;
+    int row_bytes;
+};
+
+// One block per (changed position, matrix): active[m][p] <- pool[m][indices[p]].
+__global__ __launch_bounds__(256) void cache_copy_kernel(CopyPlan cp, const int32_t *__restrict__ state,
+                                                         const int32_t *__restrict__ changed,
+                                                         const int32_t *__restrict__ indices)
+{
+    const int work = state[ST_STATE_N_CHANGED] * cp.nmat;
+    for (int w = blockIdx.x; w < work; w += gridDim.x) {
+        const int j = w / cp.nmat, m = w - j * cp.nmat;
+        const int p = changed[j];
+        const int idx = indices[p];
+        const unsigned char *src = cp.pool[m] + (size_t)idx * cp.row_bytes;
+        unsigned char *dst = cp.active[m] + (size_t)p * cp.row_bytes;
+        for (int o = threadIdx.x * 16; o < cp.row_bytes; o += 256 * 16) st16(dst + o, ld16(src + o));
+    }
+}
+
+// in [R,C] -> out [C,R], 64x64 tiles through LDS.
+template <typename E>
+__global__ __launch_bounds__(256) void transpose_kernel(const E *__restrict__ in, E *__restrict__ out, int R, int C)
+{
+    __shared__ E tile[64][65];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+    for (int k = ty; k < 64; k += 4) {
+        const int r = r0 + k, c = c0 + tx;
+        if (r < R && c < C) tile[k][tx] = in[(size_t)r * C + c];
+    }
+    __syncthreads();
+    for (int k = ty; k < 64; k += 4) {
+        const int c = c0 + k, r = r0 + tx;
+        if (r < R && c < C) out[(size_t)c * R + r] = tile[tx][k];
+    }
+}
+
+__global__ void cache_reset_kernel(uint8_t *cur_mask, int32_t *indices, int32_t *state, int I)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < I) {
+        cur_mask[i] = 0;
+        indices[i] = -1;
+    }
+    if (i < ST_STATE_WORDS) state[i] = 0;
+}
+
+}  // namespace st
+
+struct st_cache {
+    st_cache_buffers b;
+    int64_t I, H;
+    int dtype, has_gate;
+    int esz;
+    int32_t *host_state;  // pinned
+};
+
+extern "C" int64_t st_cache_max_intermediate(void) { return st::kPlanMaxI; }
+
+extern "C" st_cache *st_cache_create(const st_cache_buffers *bufs, int64_t I, int64_t H, int dtype, int has_gate)
+{
+    using namespace st;
+    auto fail = [](const char *m) -> st_cache * { set_error("st_cache_create: %s", m); return nullptr; };
+    if (!bufs) return fail("null buffers");
+    if (dtype < ST_F32 || dtype > ST_BF16) return fail("unknown dtype");
+    const int esz = dtype == ST_F32 ? 4 : 2;
+    if (I < 1 || I > kPlanMaxI) return fail("intermediate size out of range (see st_cache_max_intermediate)");
+    if (H < 1 || (H * esz) % 16 != 0) return fail("rows are not 16-byte multiples");
+    if (!bufs->up_pool || !bufs->downT_pool || !bufs->up_active || !bufs->down_active || !bufs->indices ||
+        !bufs->cur_mask || !bufs->state || !bufs->scratch)
+        return fail("null device buffer");
+    if (has_gate && (!bufs->gate_pool || !bufs->gate_active)) return fail("has_gate set but gate buffers are null");
+    const uintptr_t align = (uintptr_t)bufs->gate_pool | (uintptr_t)bufs->up_pool | (uintptr_t)bufs->downT_pool |
+                            (uintptr_t)bufs->gate_active | (uintptr_t)bufs->up_active | (uintptr_t)bufs->down_active;
+    if (align & 15) return fail("weight buffers must be 16-byte aligned");
+    st_cache *c = new (std::nothrow) st_cache;
+    if (!c) return fail("out of host memory");
+    c->b = *bufs;
+    c->I = I; c->H = H; c->dtype = dtype; c->has_gate = has_gate ? 1 : 0; c->esz = esz;
+    c->host_state = nullptr;
+    if (hipHostMalloc(reinterpret_cast<void **>(&c->host_state), ST_STATE_WORDS * sizeof(int32_t), hipHostMallocDefault) !=
+        hipSuccess) {
+        delete c;
+        return fail("hipHostMalloc failed");
+    }
+    return c;
+}
+
+extern "C" void st_cache_destroy(st_cache *c)
+{
+    if (!c) return;
+    if (c->host_state) (void)hipHostFree(c->host_state);
+    delete c;
+}
+
+extern "C" int st_cache_load_weights(st_cache *c, const void *gate, const void *up, const void *down, void *stream)
+{
+    using namespace st;
+    ST_REQUIRE(c && up && down, "st_cache_load_weights: null pointer");
+    ST_REQUIRE(!c->has_gate || gate, "st_cache_load_weights: gated cache needs gate weights");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t bytes = (size_t)c->I * c->H * c->esz;
+    ST_HIP(hipMemcpyAsync(c->b.up_pool, up, bytes, hipMemcpyDeviceToDevice, s));
+    if (c->has_gate) ST_HIP(hipMemcpyAsync(c->b.gate_pool, gate, bytes, hipMemcpyDeviceToDevice, s));
+    const dim3 grid((unsigned)((c->I + 63) / 64), (unsigned)((c->H + 63) / 64));
+    if (c->esz == 4)
+        hipLaunchKernelGGL(transpose_kernel<uint32_t>, grid, dim3(256), 0, s, static_cast<const uint32_t *>(down),
+                           static_cast<uint32_t *>(c->b.downT_pool), (int)c->H, (int)c->I);
+    else
+        hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, s, static_cast<const uint16_t *>(down),
+                           static_cast<uint16_t *>(c->b.downT_pool), (int)c->H, (int)c->I);
+    ST_HIP(hipGetLastError());
+    hipLaunchKernelGGL(cache_reset_kernel, dim3((unsigned)((c->I + 255) / 256)), dim3(256), 0, s, c->b.cur_mask,
+                       c->b.indices, c->b.state, (int)c->I);
+    ST_HIP(hipGetLastError());
+    return ST_OK;
+}
+
+extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *stream)
+{
+    using namespace st;
+    ST_REQUIRE(c && mask, "st_cache_update_async: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int I = (int)c->I;
+    const size_t lds = (size_t)I * 6 + (I & 1) * 2 + (size_t)((I + 31) >> 5) * 4 + (size_t)I + 16;
+    static bool attr_set = false;
+    if (!attr_set) {
+        ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(cache_plan_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(cache_plan_kernel, dim3(1), dim3(kPlanThreads), lds, s, mask, c->b.cur_mask, c->b.indices,
+                       c->b.state, c->b.scratch, I);
+    ST_HIP(hipGetLastError());
+    CopyPlan cp;
+    cp.nmat = 0;
+    if (c->has_gate) {
+        cp.pool[cp.nmat] = static_cast<const unsigned char *>(c->b.gate_pool);
+        cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.gate_active);
+    }
+    cp.pool[cp.nmat] = static_cast<const unsigned char *>(c->b.up_pool);
+    cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.up_active);
+    cp.pool[cp.nmat] = static_cast<const unsigned char *>(c->b.downT_pool);
+    cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.down_active);
+    for (int k = cp.nmat; k < 3; ++k) { cp.pool[k] = nullptr; cp.active[k] = nullptr; }
+    cp.row_bytes = (int)(c->H * c->esz);
+    const int grid = 8 * device_cu_count();
+    hipLaunchKernelGGL(cache_copy_kernel, dim3(grid), dim3(256), 0, s, cp, c->b.state, c->b.scratch + c->I,
+                       c->b.indices);
+    ST_HIP(hipGetLastError());
+    return ST_OK;
+}
+
+extern "C" int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream)
+{
+    using namespace st;
+    ST_REQUIRE(c, "st_cache_sync_state: null handle");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    ST_HIP(hipMemcpyAsync(c->host_state, c->b.state, ST_STATE_WORDS * sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    ST_HIP(hipStreamSynchronize(s));
+    if (state_out)
+        for (int i = 0; i < ST_STATE_WORDS; ++i) state_out[i] = c->host_state[i];
+    if (c->host_state[ST_STATE_STATUS] == ST_ERR_NO_ACTIVE) {
+        set_error("No active weights");
+        return ST_ERR_NO_ACTIVE;
+    }
+    return ST_OK;
+}
+
+extern "C" int st_cache_materialize_concat(st_cache *c, void *dst, int64_t n, void *stream)
+{
+    using namespace st;
+    ST_REQUIRE(c && dst, "st_cache_materialize_concat: null pointer");
+    ST_REQUIRE(n >= 1 && n <= c->I, "st_cache_materialize_concat: n=%lld out of range", (long long)n);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t blk = (size_t)n * c->H * c->esz;
+    unsigned char *d = static_cast<unsigned char *>(dst);
+    if (c->has_gate) {
+        ST_HIP(hipMemcpyAsync(d, c->b.gate_active, blk, hipMemcpyDeviceToDevice, s));
+        d += blk;
+    }
+    ST_HIP(hipMemcpyAsync(d, c->b.up_active, blk, hipMemcpyDeviceToDevice, s));
+    return ST_OK;
+}

@@ -1,0 +1,373 @@
+// Fused sparse-MLP decode kernel for gfx950 (small batch, HBM-bound).
+//
+// One launch streams the three packed active matrices exactly once.  A block
+// (one per CU, 512 threads, so each thread may hold up to 256 VGPRs) owns a
+// contiguous range of active rows.  Every thread owns one 16-byte column chunk
+// of the hidden dimension (two when the row has more than 512 chunks) and, for
+// each row of its group, issues the gate, up AND down loads of that chunk up
+// front, so a whole batch of rows is in flight before any arithmetic:
+//   phase 1  per-thread partial products <gate[j],x>, <up[j],x> on the chunk,
+//            DPP wave reduction, cross-wave sum through LDS,
+//            h[j] = act(g) * u  left in LDS
+//   phase 2  acc[chunk] += h[j] * down[j, chunk]   from the registers that
+//            were loaded before phase 1
+// Each block writes one fp32 partial row; a second small kernel sums the
+// partials in a fixed order (deterministic) and converts to the output type.
+//
+// Replaces sparse_mlp_forward_cpu (sparse_transformers/csrc/sparse_mlp_op.cpp:79-192)
+// and SkipMLP._forward_sparse_weight_cache (src/modeling_skip.py:114-117).
+#include "st_common.h"
+
+namespace st {
+
+constexpr int kMlpThreads = 512;
+constexpr int kMlpWaves = kMlpThreads / kWave;
+constexpr int kMlpMaxGroups = kMlpThreads / kWave;
+
+// T: storage type; NB: x rows per launch; RB: rows per group kept in flight;
+// CPT: 16-byte chunks per thread (2 only when one group spans the block).
+template <typename T, int NB, int RB, int CPT>
+__global__ __launch_bounds__(kMlpThreads) void mlp_decode_kernel(
+    const T *__restrict__ x, int B, int H, const T *__restrict__ gate, const T *__restrict__ up,
+    const T *__restrict__ down, int n_host, const int *__restrict__ n_dev, T *__restrict__ combined, long ldc,
+    float *__restrict__ partials, int act, int has_gate, int gs_log2)
+{
+    constexpr int VEC = Elem<T>::kVec;
+    extern __shared__ __align__(16) unsigned char region[];  // group combine buffer
+    __shared__ float red[kMlpWaves][RB][NB][2];               // per-wave partial (g,u)
+    __shared__ float hs[kMlpMaxGroups][RB][NB];               // h of the rows in flight
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int G = gridDim.x, blk = blockIdx.x;
+    int n = n_host;
+    if (n_dev) {
+        const int nd = *n_dev;
+        n = nd < n ? nd : n;
+        if (n < 0) n = 0;
+    }
+    const int r0 = (int)(((long)blk * n) / G), r1 = (int)(((long)(blk + 1) * n) / G);
+    const int chunks = H / VEC;
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+
+    // groups of 2^gs_log2 threads each cover all chunks of a row
+    const int GS = 1 << gs_log2, ngrp = kMlpThreads >> gs_log2, wpg = GS >> 6;
+    const int grp = tid >> gs_log2, cc = tid & (GS - 1);
+    bool valid[CPT];
+    size_t coff[CPT];
+#pragma unroll
+    for (int q = 0; q < CPT; ++q) {
+        valid[q] = cc + q * GS < chunks;
+        coff[q] = (size_t)(cc + q * GS) * VEC;
+    }
+
+    uint4 xr[NB][CPT];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int q = 0; q < CPT; ++q) xr[b][q] = (valid[q] && b < B) ? ld16(x + (size_t)b * H + coff[q]) : zero4;
+
+    float acc[NB][CPT][VEC];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int q = 0; q < CPT; ++q)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[b][q][e] = 0.f;
+
+    const int rpg = (r1 - r0 + ngrp - 1) / ngrp;  // rows per group, uniform over the block
+    const int nbat = (rpg + RB - 1) / RB;
+    for (int bat = 0; bat < nbat; ++bat) {
+        const int base = r0 + grp + bat * RB * ngrp;
+        uint4 wg[RB][CPT], wu[RB][CPT], wd[RB][CPT];
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+            const int row = base + k * ngrp;
+#pragma unroll
+            for (int q = 0; q < CPT; ++q) {
+                const bool ok = valid[q] && row < r1;
+                const size_t o = (size_t)row * H + coff[q];
+                wg[k][q] = (ok && has_gate) ? ld16(gate + o) : zero4;
+                wu[k][q] = ok ? ld16(up + o) : zero4;
+                wd[k][q] = ok ? ld16(down + o) : zero4;
+            }
+        }
+        // ---- phase 1: partial dot products on this thread's chunk(s)
+        float pg[RB][NB], pu[RB][NB];
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) pg[k][b] = pu[k][b] = 0.f;
+#pragma unroll
+            for (int q = 0; q < CPT; ++q) {
+                float fg[VEC], fu[VEC];
+                unpack<T>(wg[k][q], fg);
+                unpack<T>(wu[k][q], fu);
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    float fx[VEC];
+                    unpack<T>(xr[b][q], fx);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        pg[k][b] = fmaf(fg[e], fx[e], pg[k][b]);
+                        pu[k][b] = fmaf(fu[e], fx[e], pu[k][b]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < RB; ++k)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const float sg = wave_sum_dpp(pg[k][b]);
+                const float su = wave_sum_dpp(pu[k][b]);
+                if (lane == 0) {
+                    red[wave][k][b][0] = sg;
+                    red[wave][k][b][1] = su;
+                }
+            }
+        __syncthreads();
+        if (tid < ngrp * RB * NB) {
+            const int g_ = tid / (RB * NB), rem = tid - g_ * (RB * NB);
+            const int k_ = rem / NB, b_ = rem - k_ * NB;
+            const int row = r0 + g_ + (bat * RB + k_) * ngrp;
+            float sg = 0.f, su = 0.f;
+            for (int w = g_ * wpg; w < (g_ + 1) * wpg; ++w) {
+                sg += red[w][k_][b_][0];
+                su += red[w][k_][b_][1];
+            }
+            const float hv = has_gate ? activate(sg, act) * su : activate(su, act);
+            const bool ok = row < r1;
+            hs[g_][k_][b_] = ok ? hv : 0.f;
+            if (ok && combined && b_ < B) {
+                combined[(size_t)b_ * ldc + row] = from_float<T>(hv);
+                if (has_gate) combined[(size_t)b_ * ldc + n + row] = from_float<T>(su);
+            }
+        }
+        __syncthreads();
+        // ---- phase 2: down projection from the rows already in registers
+#pragma unroll
+        for (int k = 0; k < RB; ++k)
+#pragma unroll
+            for (int q = 0; q < CPT; ++q) {
+                float fw[VEC];
+                unpack<T>(wd[k][q], fw);
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    const float hv = hs[grp][k][b];
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[b][q][e] = fmaf(hv, fw[e], acc[b][q][e]);
+                }
+            }
+    }
+
+    // ---- combine the thread groups through LDS (CPT == 1 whenever ngrp > 1)
+    if (ngrp > 1) {
+        float *redc = reinterpret_cast<float *>(region);  // [ngrp-1][NB][H]
+        if (grp > 0 && valid[0]) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int e = 0; e < VEC; e += 4)
+                    *reinterpret_cast<float4 *>(redc + ((size_t)(grp - 1) * NB + b) * H + coff[0] + e) =
+                        make_float4(acc[b][0][e], acc[b][0][e + 1], acc[b][0][e + 2], acc[b][0][e + 3]);
+        }
+        __syncthreads();
+        if (grp == 0 && valid[0]) {
+            for (int gq = 1; gq < ngrp; ++gq)
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+#pragma unroll
+                    for (int e = 0; e < VEC; e += 4) {
+                        const float4 v =
+                            *reinterpret_cast<const float4 *>(redc + ((size_t)(gq - 1) * NB + b) * H + coff[0] + e);
+                        acc[b][0][e] += v.x; acc[b][0][e + 1] += v.y; acc[b][0][e + 2] += v.z; acc[b][0][e + 3] += v.w;
+                    }
+        }
+    }
+    if (grp == 0) {
+#pragma unroll
+        for (int q = 0; q < CPT; ++q) {
+            if (!valid[q]) continue;
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int e = 0; e < VEC; e += 4)
+                    *reinterpret_cast<float4 *>(partials + ((size_t)blk * NB + b) * H + coff[q] + e) =
+                        make_float4(acc[b][q][e], acc[b][q][e + 1], acc[b][q][e + 2], acc[b][q][e + 3]);
+        }
+    }
+}
+
+// out[b, c] = sum over blocks of partials[blk][b][c], fixed order.
+template <typename T>
+__global__ __launch_bounds__(256) void mlp_reduce_kernel(const float *__restrict__ partials, int G, int NB, int B,
+                                                         int H, T *__restrict__ out)
+{
+    __shared__ float4 red[16][16];
+    const int tid = threadIdx.x, q = tid & 15, rg = tid >> 4;
+    const int b = blockIdx.y;
+    const int col = blockIdx.x * 64 + q * 4;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (col < H) {
+        for (int blk = rg; blk < G; blk += 16) {
+            const float4 v = *reinterpret_cast<const float4 *>(partials + ((size_t)blk * NB + b) * H + col);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+    }
+    red[rg][q] = s;
+    __syncthreads();
+    if (rg == 0 && col < H) {
+        for (int k = 1; k < 16; ++k) {
+            const float4 v = red[k][q];
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        T *o = out + (size_t)b * H + col;
+        o[0] = from_float<T>(s.x); o[1] = from_float<T>(s.y);
+        o[2] = from_float<T>(s.z); o[3] = from_float<T>(s.w);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+constexpr int kMaxLds = 160 * 1024;
+
+struct MlpLaunch {
+    const void *x; int B; int H;
+    const void *gate, *up, *down;
+    int n; const int *n_dev;
+    void *out; void *combined; long ldc;
+    float *partials;
+    int act, has_gate;
+    hipStream_t stream;
+    int G;
+};
+
+template <typename T, int NB, int RB, int CPT> static int launch_inst(const MlpLaunch &a, int b0, int bcount, int gs_log2)
+{
+    const int ngrp = kMlpThreads >> gs_log2;
+    const size_t lds = (size_t)(ngrp - 1) * NB * a.H * 4;
+    ST_REQUIRE(lds <= (size_t)kMaxLds - 8192, "st_mlp_forward: H=%d needs %zu bytes of LDS", a.H, lds);
+    auto kern = mlp_decode_kernel<T, NB, RB, CPT>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   kMaxLds - 8192));
+        attr_set = true;
+    }
+    const T *x = static_cast<const T *>(a.x) + (size_t)b0 * a.H;
+    T *comb = a.combined ? static_cast<T *>(a.combined) + (size_t)b0 * a.ldc : nullptr;
+    hipLaunchKernelGGL(kern, dim3(a.G), dim3(kMlpThreads), lds, a.stream, x, bcount, a.H,
+                       static_cast<const T *>(a.gate), static_cast<const T *>(a.up), static_cast<const T *>(a.down),
+                       a.n, a.n_dev, comb, a.ldc, a.partials, a.act, a.has_gate, gs_log2);
+    ST_HIP(hipGetLastError());
+    T *out = static_cast<T *>(a.out) + (size_t)b0 * a.H;
+    hipLaunchKernelGGL(mlp_reduce_kernel<T>, dim3((a.H + 63) / 64, bcount), dim3(256), 0, a.stream, a.partials, a.G,
+                       NB, bcount, a.H, out);
+    ST_HIP(hipGetLastError());
+    return ST_OK;
+}
+
+// Picks the rows-in-flight depth: the smallest instantiated RB that covers the
+// rows a group owns, so the common case is a single batch with every load of
+// the block issued before any arithmetic.
+template <typename T, int NB> static int launch_one(const MlpLaunch &a, int b0, int bcount)
+{
+    const int chunks = a.H / Elem<T>::kVec;
+    ST_REQUIRE(chunks <= 2 * kMlpThreads, "st_mlp_forward: hidden size %d too large for this dtype (max %d)", a.H,
+               2 * kMlpThreads * Elem<T>::kVec);
+    if (chunks > kMlpThreads) {
+        const int rows = (a.n + a.G - 1) / a.G;
+        if constexpr (NB == 1) {
+            if (rows <= 4) return launch_inst<T, NB, 4, 2>(a, b0, bcount, 9);
+            return launch_inst<T, NB, 7, 2>(a, b0, bcount, 9);
+        } else {
+            return launch_inst<T, NB, 2, 2>(a, b0, bcount, 9);
+        }
+    }
+    int gs_log2 = 6;
+    while ((1 << gs_log2) < chunks) ++gs_log2;
+    const int ngrp = kMlpThreads >> gs_log2;
+    const int rows = ((a.n + a.G - 1) / a.G + ngrp - 1) / ngrp;
+    if constexpr (NB == 1) {
+        if (rows <= 4) return launch_inst<T, NB, 4, 1>(a, b0, bcount, gs_log2);
+        if (rows <= 8) return launch_inst<T, NB, 8, 1>(a, b0, bcount, gs_log2);
+        if (rows <= 12) return launch_inst<T, NB, 12, 1>(a, b0, bcount, gs_log2);
+        return launch_inst<T, NB, 15, 1>(a, b0, bcount, gs_log2);
+    } else if constexpr (NB == 2) {
+        if (rows <= 4) return launch_inst<T, NB, 4, 1>(a, b0, bcount, gs_log2);
+        return launch_inst<T, NB, 8, 1>(a, b0, bcount, gs_log2);
+    } else {
+        return launch_inst<T, NB, 4, 1>(a, b0, bcount, gs_log2);
+    }
+}
+
+template <typename T> static int launch_nb(const MlpLaunch &a)
+{
+    int b0 = 0;
+    while (b0 < a.B) {
+        const int left = a.B - b0;
+        int rc;
+        if (left >= 3) {
+            rc = launch_one<T, 4>(a, b0, left < 4 ? left : 4);
+            b0 += 4;
+        } else if (left == 2) {
+            rc = launch_one<T, 2>(a, b0, 2);
+            b0 += 2;
+        } else {
+            rc = launch_one<T, 1>(a, b0, 1);
+            b0 += 1;
+        }
+        if (rc != ST_OK) return rc;
+    }
+    return ST_OK;
+}
+
+constexpr int kMlpMaxBatchPerLaunch = 4;
+
+}  // namespace st
+
+extern "C" int64_t st_mlp_workspace_bytes(int64_t B, int64_t H)
+{
+    (void)B;
+    const int64_t G = st::device_cu_count();
+    return G * st::kMlpMaxBatchPerLaunch * H * 4;
+}
+
+extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
+                              const void *down_rows, int64_t n, const int32_t *n_dev, void *out, void *combined,
+                              int64_t ldc, void *workspace, int64_t workspace_bytes, int act, int dtype, int has_gate,
+                              void *stream)
+{
+    using namespace st;
+    ST_REQUIRE(x && up_rows && down_rows && out && workspace, "st_mlp_forward: null pointer");
+    ST_REQUIRE(!has_gate || gate_rows, "st_mlp_forward: has_gate set but gate_rows is null");
+    ST_REQUIRE(B >= 1 && B <= 4096, "st_mlp_forward: B=%lld out of range [1,4096]", (long long)B);
+    ST_REQUIRE(n >= 0 && n <= (1 << 24), "st_mlp_forward: n=%lld out of range", (long long)n);
+    ST_REQUIRE(act >= ST_ACT_RELU && act <= ST_ACT_IDENTITY, "st_mlp_forward: unknown activation %d", act);
+    ST_REQUIRE(dtype >= ST_F32 && dtype <= ST_BF16, "st_mlp_forward: unknown dtype %d", dtype);
+    const int esz = dtype == ST_F32 ? 4 : 2;
+    ST_REQUIRE(H >= 1 && (H * esz) % 16 == 0, "st_mlp_forward: H=%lld rows are not 16-byte multiples", (long long)H);
+    ST_REQUIRE(workspace_bytes >= st_mlp_workspace_bytes(B, H), "st_mlp_forward: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)st_mlp_workspace_bytes(B, H));
+    ST_REQUIRE(!combined || ldc >= (has_gate ? 2 * n : n), "st_mlp_forward: ldc=%lld too small for n=%lld",
+               (long long)ldc, (long long)n);
+    const uintptr_t align = (uintptr_t)x | (uintptr_t)gate_rows | (uintptr_t)up_rows | (uintptr_t)down_rows |
+                            (uintptr_t)workspace;
+    ST_REQUIRE((align & 15) == 0, "st_mlp_forward: pointers must be 16-byte aligned");
+
+    MlpLaunch a;
+    a.x = x; a.B = (int)B; a.H = (int)H;
+    a.gate = gate_rows; a.up = up_rows; a.down = down_rows;
+    a.n = (int)n; a.n_dev = n_dev;
+    a.out = out; a.combined = combined; a.ldc = (long)ldc;
+    a.partials = static_cast<float *>(workspace);
+    a.act = act; a.has_gate = has_gate ? 1 : 0;
+    a.stream = static_cast<hipStream_t>(stream);
+    a.G = device_cu_count();
+    switch (dtype) {
+    case ST_F32: return launch_nb<float>(a);
+    case ST_F16: return launch_nb<f16_t>(a);
+    default: return launch_nb<bf16_t>(a);
+    }
+}

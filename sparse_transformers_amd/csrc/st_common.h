@@ -1,0 +1,148 @@
+// Shared device helpers for the gfx950 sparse-MLP kernels: 16-byte vector
+// loads, element unpacking for fp32 / fp16 / bf16, wave64 reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/sparse_mlp_amd.h"
+
+namespace st {
+
+constexpr int kWave = 64;
+
+struct f16_t { uint16_t bits; };   // tag types: storage is 2 bytes, maths is fp32
+struct bf16_t { uint16_t bits; };
+
+template <typename T> struct Elem;
+template <> struct Elem<float>  { static constexpr int kVec = 4; static constexpr int kBytes = 4; };
+template <> struct Elem<f16_t>  { static constexpr int kVec = 8; static constexpr int kBytes = 2; };
+template <> struct Elem<bf16_t> { static constexpr int kVec = 8; static constexpr int kBytes = 2; };
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+// One 16-byte chunk of a row -> kVec floats.
+template <typename T> __device__ __forceinline__ void unpack(const uint4 &v, float *f);
+
+template <> __device__ __forceinline__ void unpack<float>(const uint4 &v, float *f)
+{
+    f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y);
+    f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+}
+template <> __device__ __forceinline__ void unpack<f16_t>(const uint4 &v, float *f)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        half2_t h = __builtin_bit_cast(half2_t, w[i]);
+        f[2 * i] = (float)h.x;
+        f[2 * i + 1] = (float)h.y;
+    }
+}
+template <> __device__ __forceinline__ void unpack<bf16_t>(const uint4 &v, float *f)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = __uint_as_float(w[i] << 16);
+        f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+
+// float -> storage element (round to nearest even).
+template <typename T> __device__ __forceinline__ T from_float(float f);
+template <> __device__ __forceinline__ float from_float<float>(float f) { return f; }
+template <> __device__ __forceinline__ f16_t from_float<f16_t>(float f)
+{
+    _Float16 h = (_Float16)f;
+    f16_t r; r.bits = __builtin_bit_cast(uint16_t, h);
+    return r;
+}
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    bf16_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) { r.bits = (uint16_t)((u >> 16) | 0x40u); return r; }  // NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    r.bits = (uint16_t)(u >> 16);
+    return r;
+}
+
+template <typename T> __device__ __forceinline__ float to_float(T v);
+template <> __device__ __forceinline__ float to_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_float<f16_t>(f16_t v) { return (float)__builtin_bit_cast(_Float16, v.bits); }
+template <> __device__ __forceinline__ float to_float<bf16_t>(bf16_t v) { return __uint_as_float((uint32_t)v.bits << 16); }
+
+__device__ __forceinline__ uint4 ld16(const void *p) { return *reinterpret_cast<const uint4 *>(p); }
+__device__ __forceinline__ void st16(void *p, const uint4 &v) { *reinterpret_cast<uint4 *>(p) = v; }
+
+// Sum over the 64 lanes of a wave; every lane receives the total.
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+// Same sum with DPP row operations (no LDS traffic): four steps reduce each
+// row of 16 lanes, the four row totals are then read through scalar registers.
+template <int CTRL> __device__ __forceinline__ float dpp_add(float v)
+{
+    const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+    return v + __int_as_float(t);
+}
+__device__ __forceinline__ float wave_sum_dpp(float v)
+{
+    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);  // row_half_mirror
+    v = dpp_add<0x140>(v);  // row_mirror
+    const int iv = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(iv, 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(iv, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(iv, 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(iv, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// Sum over aligned groups of `width` lanes (power of two <= 64).
+__device__ __forceinline__ float group_sum(float v, int width)
+{
+    for (int off = width >> 1; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+__device__ __forceinline__ float activate(float v, int act)
+{
+    switch (act) {
+    case ST_ACT_RELU: return v > 0.f ? v : 0.f;
+    case ST_ACT_SILU: return v / (1.f + expf(-v));
+    case ST_ACT_GELU_TANH: {
+        const float k = 0.7978845608028654f;  // sqrt(2/pi)
+        return 0.5f * v * (1.f + tanhf(k * (v + 0.044715f * v * v * v)));
+    }
+    case ST_ACT_SIGMOID: return 1.f / (1.f + expf(-v));
+    default: return v;
+    }
+}
+
+// Host-side error plumbing shared by the C-ABI translation units.
+void set_error(const char *fmt, ...);
+int hip_fail(hipError_t e, const char *what);
+
+#define ST_HIP(call)                                              \
+    do {                                                          \
+        hipError_t e__ = (call);                                  \
+        if (e__ != hipSuccess) return ::st::hip_fail(e__, #call); \
+    } while (0)
+
+#define ST_REQUIRE(cond, ...)             \
+    do {                                  \
+        if (!(cond)) {                    \
+            ::st::set_error(__VA_ARGS__); \
+            return ST_ERR_ARG;            \
+        }                                 \
+    } while (0)
+
+int device_cu_count();
+
+}  // namespace st

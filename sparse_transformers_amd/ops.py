@@ -1,0 +1,174 @@
+"""Operator-level host API: sparse_mlp_forward and the LoRA predictor mask.
+
+Mirrors the operator surface of NimbleEdge/sparse_transformers:
+  * ``sparse_mlp_forward(x, concat_weight, active_down_weight, down_proj_buffer,
+    combined_proj_buffer, act, has_gate=True)`` — sparse_transformers/csrc/sparse_mlp_op.cpp:53-76,
+    README.md:108-116 (six-argument call).
+  * ``predictor_mask`` / ``predictor_scores`` — FastLoRAProjection.forward and
+    SkipDecoderLayer._compute_binary_mask, src/modeling_skip.py:52-53,204-214.
+
+torch is used for device memory and the current stream only; all arithmetic is
+done by the HIP kernels behind the C ABI.
+"""
+from __future__ import annotations
+
+import warnings
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.ST_F32, torch.float16: _lib.ST_F16, torch.bfloat16: _lib.ST_BF16}
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}; expected float32, float16 or bfloat16") from None
+
+
+def require_gpu(*tensors: torch.Tensor) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "sparse_transformers_amd runs on an AMD GPU only: got a tensor on "
+                f"{t.device} (there is no CPU fallback)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def current_stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+_workspaces: dict = {}
+
+
+def mlp_workspace(device: torch.device, B: int, H: int) -> torch.Tensor:
+    need = int(_lib.lib().st_mlp_workspace_bytes(B, H))
+    key = (device.index if device.index is not None else torch.cuda.current_device())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def mlp_forward_rows(x2: torch.Tensor, gate_rows: Optional[torch.Tensor], up_rows: torch.Tensor,
+                     down_rows: torch.Tensor, n: int, n_dev: Optional[torch.Tensor], out: torch.Tensor,
+                     combined: Optional[torch.Tensor], act: str, has_gate: bool) -> None:
+    """Raw launch on packed rows: gate/up/down are [>=n, H] row-major, x2/out are [B, H]."""
+    dev = require_gpu(x2, gate_rows, up_rows, down_rows, out, combined, n_dev)
+    B, H = x2.shape
+    ws = mlp_workspace(dev, B, H)
+    if act not in _lib.ACT_CODES:
+        raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
+    rc = _lib.lib().st_mlp_forward(
+        x2.data_ptr(), B, H, gate_rows.data_ptr() if has_gate else None, up_rows.data_ptr(), down_rows.data_ptr(),
+        int(n), n_dev.data_ptr() if n_dev is not None else None, out.data_ptr(),
+        combined.data_ptr() if combined is not None else None, combined.stride(0) if combined is not None else 0,
+        ws.data_ptr(), ws.numel(), _lib.ACT_CODES[act], dtype_code(x2), int(bool(has_gate)), current_stream_ptr(dev))
+    _lib.check(rc, "st_mlp_forward")
+
+
+_warned_layout = False
+
+
+def sparse_mlp_forward(x: torch.Tensor, concat_weight: torch.Tensor, active_down_weight: torch.Tensor,
+                       down_proj_buffer: torch.Tensor, combined_proj_buffer: torch.Tensor, act: str = "silu",
+                       has_gate: bool = True) -> torch.Tensor:
+    """out = (act(x @ Wg^T) * (x @ Wu^T)) @ Wd^T on the active rows.
+
+    x: [..., H]; concat_weight: [2n, H] (gate rows then up rows; [n, H] when ``has_gate`` is False);
+    active_down_weight: [H, n], normally the cache's transposed view with strides (1, H).
+    ``down_proj_buffer`` is resized in place to [B, H] and returned viewed to x's shape (it aliases the
+    result, as in the reference); ``combined_proj_buffer`` is resized to [B, concat_weight.size(0)] and
+    left holding act(gate)*up in its first n columns.  Unlike sparse_mlp_op.cpp:157, ``act`` is honoured:
+    "relu" reproduces that operator, "silu" reproduces src/modeling_skip.py:114-117.
+    """
+    global _warned_layout
+    dev = require_gpu(x, concat_weight, active_down_weight, down_proj_buffer, combined_proj_buffer)
+    H = x.shape[-1]
+    rows = concat_weight.size(0)
+    if has_gate and rows % 2:
+        raise ValueError("concat_weight must hold gate rows followed by as many up rows")
+    n = rows // 2 if has_gate else rows
+    if concat_weight.dim() != 2 or concat_weight.size(1) != H:
+        raise ValueError(f"concat_weight must be [rows, {H}], got {tuple(concat_weight.shape)}")
+    if tuple(active_down_weight.shape) != (H, n):
+        raise ValueError(f"active_down_weight must be [{H}, {n}], got {tuple(active_down_weight.shape)}")
+    for name, t in (("concat_weight", concat_weight), ("active_down_weight", active_down_weight),
+                    ("down_proj_buffer", down_proj_buffer), ("combined_proj_buffer", combined_proj_buffer)):
+        if t.dtype != x.dtype:
+            raise TypeError(f"{name} has dtype {t.dtype}, expected {x.dtype}")
+    x2 = x.reshape(-1, H)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    if not concat_weight.is_contiguous():
+        concat_weight = concat_weight.contiguous()
+    B = x2.size(0)
+    # [H, n] with strides (1, H) is a packed [n, H] buffer underneath
+    if n > 0 and active_down_weight.stride() == (1, H):
+        down_rows = active_down_weight.t()
+    else:
+        if not _warned_layout:
+            warnings.warn("active_down_weight is not the cache's transposed [n,H] view; repacking it "
+                          "(one extra device copy per call)")
+            _warned_layout = True
+        down_rows = active_down_weight.t().contiguous()
+    if down_proj_buffer.dim() != 2 or down_proj_buffer.size(0) != B or down_proj_buffer.size(1) != H:
+        down_proj_buffer.resize_(B, H)
+    if combined_proj_buffer.dim() != 2 or combined_proj_buffer.size(0) != B or combined_proj_buffer.size(1) != rows:
+        combined_proj_buffer.resize_(B, rows)
+    gate_rows = concat_weight[:n] if has_gate else None
+    up_rows = concat_weight[n:] if has_gate else concat_weight
+    mlp_forward_rows(x2, gate_rows, up_rows, down_rows, n, None, down_proj_buffer, combined_proj_buffer, act,
+                     has_gate)
+    return down_proj_buffer.view(x.shape) if x.dim() != 2 else down_proj_buffer
+
+
+def predictor_mask(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.Tensor, thr: float = 0.0,
+                   ge: bool = True, return_scores: bool = False, out: Optional[torch.Tensor] = None):
+    """mask[i] = any over rows b of ((x @ down^T) @ up^T)[b, i] >= thr  (``>`` when ``ge`` is False).
+
+    x: [..., H]; down_weight: [r, H] (FastLoRAProjection.down.weight); up_weight: [I, r].
+    Returns a bool[I] tensor (and the fp32 scores [B, I] when ``return_scores``).
+    thr = 0, ge = True is the reference's "naive" method (src/modeling_skip.py:206-207).
+    """
+    dev = require_gpu(x, down_weight, up_weight, out)
+    H = x.shape[-1]
+    x2 = x.reshape(-1, H)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    B = x2.size(0)
+    r, I = down_weight.size(0), up_weight.size(0)
+    if tuple(down_weight.shape) != (r, H) or tuple(up_weight.shape) != (I, r):
+        raise ValueError(f"predictor weights must be [r,{H}] and [I,r]; got {tuple(down_weight.shape)}, "
+                         f"{tuple(up_weight.shape)}")
+    if down_weight.dtype != x.dtype or up_weight.dtype != x.dtype:
+        raise TypeError("predictor weights and x must share one dtype")
+    down_weight = down_weight if down_weight.is_contiguous() else down_weight.contiguous()
+    up_weight = up_weight if up_weight.is_contiguous() else up_weight.contiguous()
+    t_ws = torch.empty(B, r, dtype=torch.float32, device=dev)
+    scores = torch.empty(B, I, dtype=torch.float32, device=dev) if return_scores else None
+    mask = out if out is not None else torch.empty(I, dtype=torch.bool, device=dev)
+    if mask.dtype != torch.bool or mask.numel() != I or not mask.is_contiguous():
+        raise ValueError("out must be a contiguous bool[I] tensor")
+    rc = _lib.lib().st_predictor_mask(
+        x2.data_ptr(), B, H, down_weight.data_ptr(), r, up_weight.data_ptr(), I, dtype_code(x2), float(thr), int(ge),
+        t_ws.data_ptr(), scores.data_ptr() if scores is not None else None, mask.data_ptr(), current_stream_ptr(dev))
+    _lib.check(rc, "st_predictor_mask")
+    return (mask, scores) if return_scores else mask
+
+
+def predictor_scores(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.Tensor) -> torch.Tensor:
+    """fp32 scores [B, I] of the LoRA predictor (FastLoRAProjection.forward)."""
+    return predictor_mask(x, down_weight, up_weight, 0.0, True, return_scores=True)[1]

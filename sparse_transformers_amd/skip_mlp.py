@@ -1,0 +1,137 @@
+"""Host-side mirror of the reference's callers of the sparse-MLP path.
+
+  * ``FastLoRAProjection`` — src/modeling_skip.py:32-53 (the importance predictor's two bias-free maps)
+  * ``SkipMLP``            — src/modeling_skip.py:55-128 (buffers, ``initialize_weight_cache``, sparse forward)
+  * ``SparseDecodeLayer`` / ``SparseMLPStack`` — the per-layer order of SkipDecoderLayer.forward
+    (src/modeling_skip.py:204-219,234-261): predictor -> mask -> union -> cache update -> sparse MLP,
+    without attention or normalisation, which are outside this path.
+
+No HuggingFace dependency; parameters are plain tensors on the GPU.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import torch
+
+from .ops import predictor_mask, predictor_scores, sparse_mlp_forward
+from .weight_cache import WeightCache
+
+
+class FastLoRAProjection:
+    """scores = (x @ down.weight^T) @ up.weight^T with down.weight [r,H], up.weight [I,r]."""
+
+    def __init__(self, down_weight: torch.Tensor, up_weight: torch.Tensor):
+        self.down_weight = down_weight.contiguous()
+        self.up_weight = up_weight.contiguous()
+        self.lora_size, self.hidden_size = self.down_weight.shape
+        self.intermediate_size = self.up_weight.size(0)
+
+    @classmethod
+    def from_state_dict(cls, sd: dict, device=None, dtype=None) -> "FastLoRAProjection":
+        """Accepts the reference's predictor checkpoints: keys ``down.weight`` and ``up.weight``
+        (src/trainer.py:570-585)."""
+        d, u = sd["down.weight"], sd["up.weight"]
+        return cls(d.to(device=device, dtype=dtype), u.to(device=device, dtype=dtype))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return predictor_scores(x, self.down_weight, self.up_weight)
+
+    __call__ = forward
+
+    def mask(self, x: torch.Tensor, method: str = "naive", thr: float = 0.0, ge: bool = True, k: int = 0,
+             std_multiplier: float = 0.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Union-over-rows boolean mask, src/modeling_skip.py:204-214.
+
+        ``naive`` (score >= 0) and ``threshold`` (score >= thr, or > thr) are fused into the predictor
+        kernel.  ``topk`` and ``statistical_topk`` take the kernel's fp32 scores and finish with torch
+        reductions on the device.
+        """
+        if method == "naive":
+            return predictor_mask(x, self.down_weight, self.up_weight, 0.0, True, out=out)
+        if method == "threshold":
+            return predictor_mask(x, self.down_weight, self.up_weight, thr, ge, out=out)
+        scores = self.forward(x)
+        if method == "topk":
+            idx = scores.topk(k, sorted=False)[1]
+            m = torch.zeros_like(scores, dtype=torch.bool)
+            m.scatter_(-1, idx, True)
+        elif method == "statistical_topk":
+            mean = scores.mean(dim=-1, keepdim=True)
+            std = scores.std(dim=-1, keepdim=True, unbiased=False)
+            m = scores > (mean + std * std_multiplier)
+        else:
+            raise ValueError(f"unknown sparsity method {method!r}")
+        m = m.any(dim=0)
+        if out is not None:
+            out.copy_(m)
+            return out
+        return m
+
+
+class SkipMLP:
+    """Gated (or ungated) MLP whose decode path runs on the differential weight cache."""
+
+    def __init__(self, gate_weight: Optional[torch.Tensor], up_weight: torch.Tensor, down_weight: torch.Tensor,
+                 sparsity: float = 0.5, act_fn: str = "silu", has_gate: bool = True):
+        self.gate_weight, self.up_weight, self.down_weight = gate_weight, up_weight, down_weight
+        self.intermediate_size, self.hidden_size = up_weight.shape
+        self.sparsity = sparsity
+        self.act_fn_name = act_fn
+        self.has_gate = has_gate
+        dev, dt = up_weight.device, up_weight.dtype
+        self.init_mask = torch.ones(self.intermediate_size, dtype=torch.bool, device=dev)
+        self.weight_cache: Optional[WeightCache] = None
+        cols = (2 if has_gate else 1) * int(self.intermediate_size * sparsity)
+        self.down_proj_buffer = torch.zeros(1, self.hidden_size, dtype=dt, device=dev)
+        self.combined_proj_buffer = torch.zeros(1, max(cols, 1), dtype=dt, device=dev)
+
+    def initialize_weight_cache(self) -> None:
+        if self.weight_cache is None:
+            self.weight_cache = WeightCache(self.init_mask, self.hidden_size, self.gate_weight, self.up_weight,
+                                            self.down_weight, self.has_gate)
+
+    def forward(self, x: torch.Tensor, use_sparse: bool = True) -> torch.Tensor:
+        if not use_sparse:
+            raise NotImplementedError("the dense (prefill) MLP is outside this package's path")
+        wc = self.weight_cache
+        if wc is None:
+            raise RuntimeError("call initialize_weight_cache() first")
+        return sparse_mlp_forward(x, wc.get_concat_weight(), wc.get_active_down_weight(), self.down_proj_buffer,
+                                  self.combined_proj_buffer, self.act_fn_name, self.has_gate)
+
+    __call__ = forward
+
+
+class SparseDecodeLayer:
+    """predictor -> mask -> cache update -> sparse MLP for one layer, all stream-ordered."""
+
+    def __init__(self, predictor: FastLoRAProjection, cache: WeightCache, act: str = "silu", thr: float = 0.0,
+                 ge: bool = True):
+        self.predictor, self.cache, self.act, self.thr, self.ge = predictor, cache, act, thr, ge
+        self.mask = torch.zeros(cache.intermediate_size, dtype=torch.bool, device=cache.device)
+
+    def compute_mask_and_update(self, x_pred: torch.Tensor, mask_override: Optional[torch.Tensor] = None) -> None:
+        self.predictor.mask(x_pred, "threshold", self.thr, self.ge, out=self.mask)
+        self.cache.update_active_weights_async(self.mask if mask_override is None else mask_override)
+
+    def mlp(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return self.cache.forward(x, self.act, out=out)
+
+
+class SparseMLPStack:
+    """A stack of sparse layers stepped one token at a time (the decode loop of the reference,
+    src/modeling_skip.py:383-402, restricted to the sparse-MLP path)."""
+
+    def __init__(self, layers: Sequence[SparseDecodeLayer]):
+        self.layers: List[SparseDecodeLayer] = list(layers)
+
+    def decode_step(self, x: torch.Tensor, x_pred: Optional[Sequence[torch.Tensor]] = None,
+                    mask_override: Optional[Sequence[torch.Tensor]] = None) -> torch.Tensor:
+        """x: [B,H].  Layer l's predictor sees ``x_pred[l]`` (default: the layer's own input), its MLP
+        sees the previous layer's output."""
+        for l, layer in enumerate(self.layers):
+            xp = x if x_pred is None else x_pred[l]
+            layer.compute_mask_and_update(xp, None if mask_override is None else mask_override[l])
+            x = layer.mlp(x)
+        return x

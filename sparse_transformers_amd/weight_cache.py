@@ -1,0 +1,172 @@
+"""HBM-resident differential weight cache with the reference's class surface.
+
+Mirrors ``torch.classes.sparse_mlp.WeightCache`` (sparse_transformers/csrc/weight_cache.h:13-381,
+registered in sparse_mlp_op.cpp:198-202): same six constructor arguments, ``update_active_weights``,
+``get_concat_weight``, ``get_active_down_weight``.  All storage is device memory owned by torch
+tensors; the bookkeeping (ordered active list, mask diff, pairing, swap-with-last) runs in HIP kernels.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .ops import current_stream_ptr, dtype_code, mlp_forward_rows, require_gpu
+
+
+class WeightCache:
+    """Drop-in for the reference WeightCache, plus a zero-copy fast path.
+
+    Reference-compatible calls (each may read a few state words back from the device):
+      ``update_active_weights(mask)``, ``get_concat_weight()``, ``get_active_down_weight()``.
+    Fast path (nothing is read back, everything is stream-ordered):
+      ``update_active_weights_async(mask)`` then ``forward(x, act, ...)``; the kernels take the active
+      count from device memory.
+    """
+
+    def __init__(self, init_mask: torch.Tensor, hidden_size: int, gate_weight: Optional[torch.Tensor],
+                 up_weight: torch.Tensor, down_weight: torch.Tensor, has_gate: bool = True):
+        self.has_gate = bool(has_gate)
+        if self.has_gate and gate_weight is None:
+            raise ValueError("has_gate=True needs gate_weight")
+        dev = require_gpu(up_weight, down_weight, gate_weight if self.has_gate else None)
+        self.device = dev
+        self.dtype = up_weight.dtype
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(up_weight.size(0))
+        I, H = self.intermediate_size, self.hidden_size
+        if tuple(up_weight.shape) != (I, H) or tuple(down_weight.shape) != (H, I):
+            raise ValueError(f"up must be [I,H] and down [H,I]; got {tuple(up_weight.shape)}, {tuple(down_weight.shape)}")
+        if self.has_gate and tuple(gate_weight.shape) != (I, H):
+            raise ValueError(f"gate must be [{I},{H}], got {tuple(gate_weight.shape)}")
+        if down_weight.dtype != self.dtype or (self.has_gate and gate_weight.dtype != self.dtype):
+            raise TypeError("gate, up and down weights must share one dtype")
+        code = dtype_code(up_weight)
+        L = _lib.lib()
+        if I > L.st_cache_max_intermediate():
+            raise ValueError(f"intermediate size {I} exceeds the supported maximum {L.st_cache_max_intermediate()}")
+
+        def wbuf():
+            return torch.empty(I, H, dtype=self.dtype, device=dev)
+
+        self.gate_pool = wbuf() if self.has_gate else None
+        self.up_pool = wbuf()
+        self.downT_pool = wbuf()
+        self.gate_active = wbuf() if self.has_gate else None
+        self.up_active = wbuf()
+        self.down_active = wbuf()
+        self.indices = torch.empty(I, dtype=torch.int32, device=dev)
+        self.cur_mask = torch.empty(I, dtype=torch.uint8, device=dev)
+        self.state = torch.empty(_lib.STATE_WORDS, dtype=torch.int32, device=dev)
+        self.scratch = torch.empty(2 * I, dtype=torch.int32, device=dev)
+        self.n_active_dev = self.state[_lib.STATE_N_ACTIVE:_lib.STATE_N_ACTIVE + 1]
+
+        bufs = _lib.CacheBuffers(
+            self.gate_pool.data_ptr() if self.has_gate else None, self.up_pool.data_ptr(), self.downT_pool.data_ptr(),
+            self.gate_active.data_ptr() if self.has_gate else None, self.up_active.data_ptr(),
+            self.down_active.data_ptr(), self.indices.data_ptr(), self.cur_mask.data_ptr(), self.state.data_ptr(),
+            self.scratch.data_ptr())
+        self._h = L.st_cache_create(C.byref(bufs), I, H, code, int(self.has_gate))
+        if not self._h:
+            raise RuntimeError(f"st_cache_create: {_lib.last_error()}")
+
+        up_c = up_weight.detach().contiguous()
+        down_c = down_weight.detach().contiguous()
+        gate_c = gate_weight.detach().contiguous() if self.has_gate else None
+        rc = L.st_cache_load_weights(self._h, gate_c.data_ptr() if self.has_gate else None, up_c.data_ptr(),
+                                     down_c.data_ptr(), current_stream_ptr(dev))
+        _lib.check(rc, "st_cache_load_weights")
+        self._host_state = (C.c_int32 * _lib.STATE_WORDS)()
+        self._host_serial = -1      # serial the host copy of the state belongs to
+        self._dirty = True          # updates enqueued since the last read-back
+        self._concat: Optional[torch.Tensor] = None
+        self._concat_serial = -1
+        # weight_cache.h:226: the constructor ends with update_active_weights(init_mask)
+        self.update_active_weights(init_mask)
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h and _lib._lib is not None:
+            _lib._lib.st_cache_destroy(h)
+
+    # ------------------------------------------------------------------ updates
+    def _mask_arg(self, mask: torch.Tensor) -> torch.Tensor:
+        if mask.device != self.device:
+            mask = mask.to(self.device)
+        if mask.dtype not in (torch.bool, torch.uint8):
+            mask = mask != 0
+        if mask.numel() != self.intermediate_size:
+            raise ValueError(f"mask must have {self.intermediate_size} elements, got {mask.numel()}")
+        return mask if mask.is_contiguous() else mask.contiguous()
+
+    def update_active_weights_async(self, mask: torch.Tensor) -> None:
+        """Enqueue the differential update on the current stream; never waits for the device."""
+        m = self._mask_arg(mask)
+        rc = _lib.lib().st_cache_update_async(self._h, m.data_ptr(), current_stream_ptr(self.device))
+        _lib.check(rc, "st_cache_update_async")
+        self._dirty = True
+
+    def update_active_weights(self, mask: torch.Tensor) -> None:
+        """weight_cache.h:229: raises RuntimeError("No active weights") when the mask empties the cache."""
+        self.update_active_weights_async(mask)
+        self.sync_state()
+
+    def sync_state(self) -> dict:
+        """Read the state words back (waits for the current stream)."""
+        if self._dirty:
+            rc = _lib.lib().st_cache_sync_state(self._h, self._host_state, current_stream_ptr(self.device))
+            self._dirty = False
+            _lib.check(rc, "st_cache_sync_state")
+        s = self._host_state
+        return {"n_active": s[_lib.STATE_N_ACTIVE], "n_changed": s[_lib.STATE_N_CHANGED],
+                "status": s[_lib.STATE_STATUS], "valid": s[_lib.STATE_VALID], "n_added": s[_lib.STATE_N_ADDED],
+                "n_removed": s[_lib.STATE_N_REMOVED], "serial": s[_lib.STATE_SERIAL]}
+
+    # ------------------------------------------------------------------ getters
+    def get_num_active(self) -> int:
+        return int(self.sync_state()["n_active"])
+
+    def get_active_indices(self) -> torch.Tensor:
+        """Ordered active list (the reference's ``active_indices``) as int64[n]."""
+        n = self.get_num_active()
+        return self.indices[:n].to(torch.int64)
+
+    def _require_valid(self) -> dict:
+        st = self.sync_state()
+        if not st["valid"]:
+            raise RuntimeError("Cache is not valid")
+        return st
+
+    def get_concat_weight(self) -> torch.Tensor:
+        """Contiguous [2n,H] (gate rows then up rows; [n,H] when ungated), valid until the next update."""
+        st = self._require_valid()
+        n = int(st["n_active"])
+        if self._concat is None or self._concat_serial != st["serial"]:
+            rows = (2 if self.has_gate else 1) * n
+            buf = torch.empty(rows, self.hidden_size, dtype=self.dtype, device=self.device)
+            if n > 0:
+                rc = _lib.lib().st_cache_materialize_concat(self._h, buf.data_ptr(), n, current_stream_ptr(self.device))
+                _lib.check(rc, "st_cache_materialize_concat")
+            self._concat, self._concat_serial = buf, st["serial"]
+        return self._concat
+
+    def get_active_down_weight(self) -> torch.Tensor:
+        """[H,n] view with strides (1,H) over the packed down rows (zero-copy)."""
+        st = self._require_valid()
+        return self.down_active[: int(st["n_active"])].t()
+
+    # ---------------------------------------------------------------- fast path
+    def forward(self, x: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor] = None,
+                combined: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Sparse MLP on the cache's packed rows; the active count is read on the device."""
+        H = self.hidden_size
+        x2 = x.reshape(-1, H)
+        if not x2.is_contiguous():
+            x2 = x2.contiguous()
+        if out is None:
+            out = torch.empty_like(x2)
+        mlp_forward_rows(x2, self.gate_active, self.up_active, self.down_active, self.intermediate_size,
+                         self.n_active_dev, out, combined, act, self.has_gate)
+        return out.view(x.shape)
