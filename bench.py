@@ -1,0 +1,253 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-MLP decode path on one MI355X.
+
+A "step" is one decoded token through the whole stack of the chosen workload: per layer the LoRA
+predictor + threshold mask, the differential weight-cache update (driven by a pre-generated mask trace
+with the workload's active fraction and per-step churn) and the fused sparse MLP.  All inputs (weights,
+predictor inputs, mask trace) are resident in HBM before the timed region starts.
+
+Prints ONE JSON line (see README / DESIGN.md for the fields).  `roofline` is for the dominant kernel
+(the fused decode MLP): algorithmic bytes 3*n*H*s per launch over its mean duration, measured with HIP
+events recorded on the launch stream in a second pass over the same workload.  `cpu_baseline` times the
+same path on the host cores on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="llama3b_stack_fp16")
+    ap.add_argument("--layers", type=int, default=0, help="override the number of layers (debug)")
+    ap.add_argument("--batch", type=int, default=0, help="override the decode batch (rows of x)")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="run predictor/cache update on the same stream as the MLP instead of a side stream")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-layers", type=int, default=2)
+    ap.add_argument("--cpu-steps", type=int, default=24)
+    ap.add_argument("--profile-steps", type=int, default=32)
+    ap.add_argument("--seed", type=int, default=1236)
+    return ap.parse_args()
+
+
+def build_stack(wl, layers, batch, seed, torch, st):
+    """Random-init weights of the workload's shape on the GPU, caches, predictors, thresholds."""
+    dev = torch.device("cuda:0")
+    dt = getattr(torch, wl.dtype)
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+
+    def nrm(*shape):
+        return (torch.randn(*shape, generator=g, device=dev, dtype=torch.float32) * 0.02).to(dt)
+
+    H, I, r = wl.hidden, wl.intermediate, wl.rank
+    init_mask = torch.ones(I, dtype=torch.bool, device=dev)
+    stack_layers = []
+    for _ in range(layers):
+        gate = nrm(I, H) if wl.has_gate else None
+        up, down = nrm(I, H), nrm(H, I)
+        A, Bm = nrm(r, H), nrm(I, r)
+        cache = st.WeightCache(init_mask, H, gate, up, down, wl.has_gate)
+        del gate, up, down
+        pred = st.FastLoRAProjection(A, Bm)
+        # threshold: the (1 - active_frac) quantile of this layer's scores on a probe input
+        probe = torch.randn(1, H, generator=g, device=dev, dtype=torch.float32).to(dt)
+        s = pred(probe).float().flatten()
+        thr = float(torch.quantile(s, 1.0 - wl.active_frac))
+        stack_layers.append(st.SparseDecodeLayer(pred, cache, wl.act, thr, True))
+    return st.SparseMLPStack(stack_layers), g
+
+
+def cpu_baseline(wl, layers, steps, seed, torch):
+    """The same path on the host: the reference's own C++ WeightCache (compiled into oracle/_ref) when
+    it loads, else the C oracle; predictor and MLP as the torch-CPU calls of src/modeling_skip.py
+    (fp32, as the reference cache is fp32 only).  Returns tok/s scaled to the full stack depth."""
+    import oracle
+    from sparse_transformers_amd import synthetic as syn
+
+    ref = oracle.load_reference()
+    kind = "reference" if ref else "port"
+    H, I, r = wl.hidden, wl.intermediate, wl.rank
+    rng = np.random.default_rng(seed)
+    trace = syn.mask_trace(seed + 1, layers, I, wl.n_active, steps + 4, wl.churn_lo, wl.churn_hi)
+    act = {"silu": torch.nn.functional.silu, "relu": torch.relu}[wl.act]
+    built = []
+    for l in range(layers):
+        w = syn.layer_weights(rng, H, I, r, has_gate=wl.has_gate)
+        up, down = torch.from_numpy(w["up"]), torch.from_numpy(w["down"])
+        gate = torch.from_numpy(w["gate"]) if wl.has_gate else None
+        A, Bm = torch.from_numpy(w["A"]), torch.from_numpy(w["Bm"])
+        m0 = torch.from_numpy(trace[0, l])
+        if ref:
+            cache = ref[0](m0, H, gate, up, down, wl.has_gate)
+        else:
+            cache = oracle.OracleWeightCache(trace[0, l], H, w["gate"], w["up"], w["down"], wl.has_gate)
+        built.append((cache, A, Bm))
+    x = torch.randn(wl.batch, H)
+    times = []
+    for t in range(1, steps + 4):
+        t0 = time.perf_counter()
+        for l, (cache, A, Bm) in enumerate(built):
+            scores = (x @ A.t()) @ Bm.t()
+            _ = (scores >= 0).any(dim=0)                    # predictor + naive mask + union
+            m = trace[t, l]
+            if ref:
+                cache.update_active_weights(torch.from_numpy(m))
+                cw, dw = cache.get_concat_weight(), cache.get_active_down_weight()
+            else:
+                cache.update_active_weights(m)
+                cw, dw = torch.from_numpy(cache.get_concat_weight()), torch.from_numpy(cache.get_active_down_weight())
+            if wl.has_gate:
+                gt, u = x.matmul(cw.t()).chunk(2, dim=-1)
+                y = (act(gt) * u).matmul(dw.t())
+            else:
+                y = act(x.matmul(cw.t())).matmul(dw.t())
+        times.append(time.perf_counter() - t0)
+    per_layer_step = float(np.median(times[4:])) / layers
+    tok_s = wl.batch / (per_layer_step * wl.layers)
+    return {
+        "value": round(tok_s, 3), "unit": "tok/s", "cores": int(torch.get_num_threads()), "kind": kind,
+        "sample": f"{layers} of {wl.layers} layers x {steps} steps, fp32, median per-layer time scaled to "
+                  f"{wl.layers} layers; cache update = "
+                  + ("reference WeightCache compiled from its own sources" if ref else "C restatement")
+                  + ", predictor/MLP = torch CPU matmul path",
+        "ms_per_layer_step": round(per_layer_step * 1e3, 3),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (every box has one); --gpus {args.gpus} is not supported. "
+              "The path shards along the intermediate dimension (see DESIGN.md) but no multi-GPU code exists.",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    import sparse_transformers_amd as st
+    from sparse_transformers_amd import _lib, synthetic as syn
+
+    wl = syn.WORKLOADS[args.workload]
+    layers = args.layers or wl.layers
+    B = args.batch or wl.batch
+    dev = torch.device("cuda:0")
+    dt = getattr(torch, wl.dtype)
+    esz = 4 if wl.dtype == "float32" else 2
+    H, I, n = wl.hidden, wl.intermediate, wl.n_active
+    K, W, P = args.steps, args.warmup, args.profile_steps
+
+    stack, g = build_stack(wl, layers, B, args.seed, torch, st)
+    T = W + K + 1
+    trace = torch.from_numpy(syn.mask_trace(args.seed + 7, layers, I, n, T, wl.churn_lo, wl.churn_hi)).to(dev)
+    # predictor inputs per layer and step, MLP input of the first layer per step
+    x_pred = torch.randn(T, layers, B, H, generator=g, device=dev, dtype=torch.float32).to(dt)
+    x_in = torch.randn(T, B, H, generator=g, device=dev, dtype=torch.float32).to(dt)
+
+    # bring every cache to the first mask of the trace (the big one-off shrink from all-ones)
+    for l, layer in enumerate(stack.layers):
+        layer.cache.update_active_weights(trace[0, l])
+        assert layer.cache.get_num_active() == n
+
+    use_graph = not args.no_graph
+    stack.prepare(B, overlap=not args.no_overlap)
+    if use_graph:
+        stack.step_staged(x_in[0], x_pred[0], trace[0])     # first launches outside capture
+        torch.cuda.synchronize()
+        stack.capture()
+
+    def run(t):
+        stack.step_staged(x_in[t], x_pred[t], trace[t], replay=use_graph)
+
+    for t in range(1, W + 1):
+        run(t)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t_host0 = time.perf_counter()
+    e0.record()
+    for t in range(W + 1, W + K + 1):
+        run(t)
+    e1.record()
+    torch.cuda.synchronize()
+    host_s = time.perf_counter() - t_host0
+    ms_per_step = e0.elapsed_time(e1) / K
+    tok_s = B * 1000.0 / ms_per_step
+
+    # ---- second pass over the same masks (backwards, so every transition has the same churn) with
+    # ---- per-kernel HIP events recorded on the launch stream
+    L = _lib.lib()
+    cap = P * layers * 8
+    _lib.check(L.st_profile_enable(cap), "st_profile_enable")
+    for t in range(W + K - 1, W + K - 1 - P, -1):
+        stack.step_staged(x_in[t], x_pred[t], trace[t], replay=False)
+    torch.cuda.synchronize()
+    kinds = (C.c_int * cap)()
+    ms = (C.c_float * cap)()
+    cnt = L.st_profile_collect(kinds, ms, cap)
+    L.st_profile_disable()
+    kinds_np, ms_np = np.frombuffer(kinds, dtype=np.int32)[:cnt], np.frombuffer(ms, dtype=np.float32)[:cnt]
+    per_kernel = {}
+    for k, name in enumerate(_lib.KERNEL_KINDS):
+        sel = ms_np[kinds_np == k]
+        if sel.size:
+            per_kernel[name] = {"launches": int(sel.size), "mean_us": round(float(sel.mean()) * 1e3, 3),
+                                "median_us": round(float(np.median(sel)) * 1e3, 3),
+                                "p10_us": round(float(np.percentile(sel, 10)) * 1e3, 3),
+                                "p90_us": round(float(np.percentile(sel, 90)) * 1e3, 3)}
+    mats = 3 if wl.has_gate else 2
+    alg_bytes = mats * n * H * esz                      # active-weight bytes one launch streams
+    mlp_us = per_kernel["mlp_decode"]["mean_us"]
+    achieved = alg_bytes / (mlp_us * 1e-6) / 1e9
+    upd_us = per_kernel["cache_plan"]["mean_us"] + per_kernel["cache_copy"]["mean_us"]
+
+    churn_mean = 0.5 * (wl.churn_lo + wl.churn_hi)
+    result = {
+        "metric": "sparse-MLP decode tok/s", "value": round(tok_s, 2), "unit": "tok/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[wl.dtype], "data": "synthetic",
+        "config": {"workload": wl.name, "layers": layers, "hidden": H, "intermediate": I, "predictor_rank": wl.rank,
+                   "batch": B, "act": wl.act, "has_gate": wl.has_gate, "n_active": n,
+                   "churn": [wl.churn_lo, wl.churn_hi], "mask_source": "trace",
+                   "launch": "hip_graph" if use_graph else "eager",
+                   "streams": 1 if args.no_overlap else 2},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "mlp_decode_kernel",
+                     "bytes_per_launch": alg_bytes, "mean_us": mlp_us},
+        "cache_update_us_per_layer": round(upd_us, 3),
+        "stack_hbm_gbps": round(layers * alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+        "host_wall_ms_per_step": round(host_s * 1e3 / K, 5),
+        "kernels_us": per_kernel,
+        "churn_mean": churn_mean,
+    }
+    if not args.no_cpu_baseline:
+        try:
+            result["cpu_baseline"] = cpu_baseline(wl, max(1, min(args.cpu_layers, layers)), args.cpu_steps,
+                                                  args.seed, torch)
+        except Exception as exc:  # the baseline is reported, never required for the GPU numbers
+            result["cpu_baseline"] = {"value": None, "unit": "tok/s", "cores": 0, "kind": "port",
+                                      "sample": f"failed: {exc!r}"}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -60,6 +60,11 @@ const char *st_last_error(void);
  *   n_dev              optional device int32: when non-NULL the kernels use
  *                      min(*n_dev, n) instead, so a cache update and the
  *                      forward can be enqueued back to back with no host read
+ *                      (rows in [*n_dev, n) may be read but are ignored, so
+ *                      the buffers must really hold n rows)
+ *   n_hint             only with n_dev: the count the host expects (0 = no
+ *                      idea).  Rows below it are requested before *n_dev has
+ *                      arrived; a wrong hint costs time, never correctness
  *   out        [B,H]   dtype `dtype`   (the reference's down_proj_buffer)
  *   combined   [B,ldc] dtype `dtype`, optional (NULL = skip): receives
  *                      act(gate)*up in columns [0,n) and, when gated, the raw
@@ -70,8 +75,9 @@ const char *st_last_error(void);
  * ------------------------------------------------------------------------ */
 int64_t st_mlp_workspace_bytes(int64_t B, int64_t H);
 int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
-                   const void *down_rows, int64_t n, const int32_t *n_dev, void *out, void *combined, int64_t ldc,
-                   void *workspace, int64_t workspace_bytes, int act, int dtype, int has_gate, void *stream);
+                   const void *down_rows, int64_t n, const int32_t *n_dev, int64_t n_hint, void *out, void *combined,
+                   int64_t ldc, void *workspace, int64_t workspace_bytes, int act, int dtype, int has_gate,
+                   void *stream);
 
 /* ------------------------------------------------------------------------
  * LoRA predictor -> threshold mask -> union over rows, on the device.
@@ -155,6 +161,33 @@ int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream);
  * callers that need the reference's tensor; n is the host's count from the
  * last st_cache_sync_state. */
 int st_cache_materialize_concat(st_cache *c, void *dst, int64_t n, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Per-kernel timing with HIP events, for benchmarks (no counterpart in the
+ * reference, whose benchmark.py:149-156 times whole generations from the
+ * host).  While enabled, every kernel launched by this library is bracketed
+ * by a pair of events recorded on the launch stream; st_profile_collect waits
+ * for them and returns one (kind, milliseconds) sample per launch.  Recording
+ * costs a few microseconds per launch, so throughput is measured with
+ * profiling off.
+ * ------------------------------------------------------------------------ */
+typedef enum st_kernel_kind {
+    ST_K_MLP_DECODE = 0,
+    ST_K_MLP_REDUCE = 1,
+    ST_K_CACHE_PLAN = 2,
+    ST_K_CACHE_COPY = 3,
+    ST_K_PRED_DOWN = 4,
+    ST_K_PRED_UP_MASK = 5,
+    ST_K_MLP_PREFILL_GATEUP = 6,
+    ST_K_MLP_PREFILL_DOWN = 7,
+    ST_K_KINDS = 8
+} st_kernel_kind;
+
+int st_profile_enable(int max_samples); /* host; allocates the event pool */
+int st_profile_disable(void);
+/* host; kinds/ms: arrays of `cap` entries; returns the number of samples
+ * written (or a negative st_status) and clears the sample list */
+int st_profile_collect(int *kinds, float *ms, int cap);
 
 #ifdef __cplusplus
 }

@@ -38,7 +38,8 @@ SIGNATURES = {
     "st_version": (_ci, []),
     "st_last_error": (C.c_char_p, []),
     "st_mlp_workspace_bytes": (_i64, [_i64, _i64]),
-    "st_mlp_forward": (_ci, [_vp, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _ci, _ci, _ci, _vp]),
+    "st_mlp_forward": (_ci, [_vp, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _ci, _ci, _ci,
+                             _vp]),
     "st_predictor_mask": (_ci, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _ci, _f, _ci, _vp, _vp, _vp, _vp]),
     "st_cache_max_intermediate": (_i64, []),
     "st_cache_create": (_vp, [C.POINTER(CacheBuffers), _i64, _i64, _ci, _ci]),
@@ -47,7 +48,13 @@ SIGNATURES = {
     "st_cache_update_async": (_ci, [_vp, _vp, _vp]),
     "st_cache_sync_state": (_ci, [_vp, _vp, _vp]),
     "st_cache_materialize_concat": (_ci, [_vp, _vp, _i64, _vp]),
+    "st_profile_enable": (_ci, [_ci]),
+    "st_profile_disable": (_ci, []),
+    "st_profile_collect": (_ci, [_vp, _vp, _ci]),
 }
+
+KERNEL_KINDS = ["mlp_decode", "mlp_reduce", "cache_plan", "cache_copy", "pred_down", "pred_up_mask",
+                "mlp_prefill_gateup", "mlp_prefill_down"]
 
 _lib = None
 

@@ -24,7 +24,7 @@ namespace st {
 constexpr int kPlanThreads = 1024;
 constexpr int kPlanWaves = kPlanThreads / kWave;
 constexpr uint16_t kNone = 0xffffu;
-// LDS per intermediate element: pos(2) + idx(2) + removed list(2) + flags(1) + dirty(1/8)
+// LDS per intermediate element: pos(2) + idx(2) + added/removed lists(2) + flags(1) + dirty(1/8)
 constexpr int64_t kPlanMaxI = 22000;
 
 __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane)
@@ -64,30 +64,30 @@ __global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t 
     extern __shared__ __align__(16) unsigned char smem[];
     uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);  // index -> position
     uint16_t *idx_l = pos_l + I;                           // position -> index
-    uint16_t *rem_l = idx_l + I;                           // ascending removed indices
-    uint32_t *dirty = reinterpret_cast<uint32_t *>(rem_l + I + (I & 1));  // bit per position
+    // added indices ascending from the front, removed indices ascending from the
+    // back (k-th removed at lists[I-1-k]); the two never meet: na + nr <= I
+    uint16_t *lists = idx_l + I;
+    uint32_t *dirty = reinterpret_cast<uint32_t *>(lists + I + (I & 1));  // bit per position
     const int dirty_words = (I + 31) >> 5;
     uint8_t *flag_l = reinterpret_cast<uint8_t *>(dirty + dirty_words);   // bit0 new, bit1 old
     __shared__ uint32_t wave_tot[kPlanWaves];
     __shared__ int n_new_s;
 
-    int32_t *added_g = scratch;        // [I] ascending added indices
-    int32_t *changed_g = scratch + I;  // [I] positions to rewrite
+    int32_t *changed_g = scratch;      // [I] positions to rewrite
+    int32_t *source_g = scratch + I;   // [I] pool row for each of them
 
     const int tid = threadIdx.x;
+    // Everything the plan needs from global memory is requested in one go:
+    // the count, both masks and the whole index list (entries >= n are ignored).
     const int n = state[ST_STATE_N_ACTIVE];
-
     for (int i = tid; i < I; i += kPlanThreads) {
         pos_l[i] = kNone;
         flag_l[i] = (new_mask[i] ? 1 : 0) | (cur_mask[i] ? 2 : 0);
+        idx_l[i] = (uint16_t)indices[i];
     }
     for (int w = tid; w < dirty_words; w += kPlanThreads) dirty[w] = 0u;
     __syncthreads();
-    for (int p = tid; p < n; p += kPlanThreads) {
-        const int idx = indices[p];
-        idx_l[p] = (uint16_t)idx;
-        pos_l[idx] = (uint16_t)p;
-    }
+    for (int p = tid; p < n; p += kPlanThreads) pos_l[idx_l[p]] = (uint16_t)p;
 
     // ---- diff: contiguous element range per thread keeps the lists ascending
     const int E = (I + kPlanThreads - 1) / kPlanThreads;
@@ -113,8 +113,8 @@ __global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t 
         int oa = (int)(off & 0xffffu), orr = (int)(off >> 16);
         for (int i = e0; i < e1; ++i) {
             const uint8_t f = flag_l[i];
-            if (f == 1) added_g[oa++] = i;
-            if (f == 2) rem_l[orr++] = (uint16_t)i;
+            if (f == 1) lists[oa++] = (uint16_t)i;
+            if (f == 2) lists[I - 1 - (orr++)] = (uint16_t)i;
         }
     }
     __syncthreads();
@@ -122,10 +122,10 @@ __global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t 
     const int pairs = na < nr ? na : nr;
     // ---- phase 1: paired replacement
     for (int i = tid; i < pairs; i += kPlanThreads) {
-        const int e = rem_l[i];
+        const int e = lists[I - 1 - i];
         const uint16_t p = pos_l[e];
         if (p != kNone) {
-            const int a = added_g[i];
+            const int a = lists[i];
             idx_l[p] = (uint16_t)a;
             pos_l[a] = p;
             pos_l[e] = kNone;
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t 
     for (int i = pairs + tid; i < na; i += kPlanThreads) {
         const int p = n + (i - pairs);
         if (p < I) {
-            const int a = added_g[i];
+            const int a = lists[i];
             idx_l[p] = (uint16_t)a;
             pos_l[a] = (uint16_t)p;
             atomicOr(&dirty[p >> 5], 1u << (p & 31));
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t 
         int m = n + (na - pairs);
         if (m > I) m = I;
         for (int k = pairs; k < nr; ++k) {
-            const int e = rem_l[k];
+            const int e = lists[I - 1 - k];
             const uint16_t p = pos_l[e];
             if (p == kNone) continue;
             if (m <= 0) break;
@@ -182,8 +182,11 @@ __global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t 
         const int bit = __ffs(word) - 1;
         word &= word - 1;
         const int p = (tid << 5) + bit;
-        changed_g[coff++] = p;
-        indices[p] = idx_l[p];
+        const int idx = idx_l[p];
+        changed_g[coff] = p;
+        source_g[coff] = idx;
+        ++coff;
+        indices[p] = idx;
     }
 
     if (n_new > 0) {  // the reference stores the mask only when the rebuild did not throw
@@ -211,19 +214,45 @@ struct CopyPlan {
     int row_bytes;
 };
 
-// One block per (changed position, matrix): active[m][p] <- pool[m][indices[p]].
-__global__ __launch_bounds__(256) void cache_copy_kernel(CopyPlan cp, const int32_t *__restrict__ state,
-                                                         const int32_t *__restrict__ changed,
-                                                         const int32_t *__restrict__ indices)
+constexpr int kCopyThreads = 256;
+constexpr int kCopyUnroll = 4;  // 16-byte chunks per thread issued together
+
+// One block per (changed position, matrix): active[m][p] <- pool[m][source].
+// The work item is read speculatively together with the count, so a block
+// needs two memory round trips: (count, position, source), then the row.
+__global__ __launch_bounds__(kCopyThreads) void cache_copy_kernel(CopyPlan cp, const int32_t *__restrict__ state,
+                                                                  const int32_t *__restrict__ changed,
+                                                                  const int32_t *__restrict__ source, int I)
 {
-    const int work = state[ST_STATE_N_CHANGED] * cp.nmat;
-    for (int w = blockIdx.x; w < work; w += gridDim.x) {
-        const int j = w / cp.nmat, m = w - j * cp.nmat;
-        const int p = changed[j];
-        const int idx = indices[p];
+    const int nmat = cp.nmat;
+    const int cap = I * nmat;
+    int w = blockIdx.x;
+    if (w >= cap) return;
+    // the lists have I entries, so reading entry w / nmat is safe before the count is known
+    int p = changed[w / nmat];
+    int idx = source[w / nmat];
+    const int work = state[ST_STATE_N_CHANGED] * nmat;
+    for (; w < work; w += gridDim.x) {
+        const int j = w / nmat, m = w - j * nmat;
+        if (w != (int)blockIdx.x) {
+            p = changed[j];
+            idx = source[j];
+        }
         const unsigned char *src = cp.pool[m] + (size_t)idx * cp.row_bytes;
         unsigned char *dst = cp.active[m] + (size_t)p * cp.row_bytes;
-        for (int o = threadIdx.x * 16; o < cp.row_bytes; o += 256 * 16) st16(dst + o, ld16(src + o));
+        for (int o0 = 0; o0 < cp.row_bytes; o0 += kCopyThreads * kCopyUnroll * 16) {
+            uint4 v[kCopyUnroll];
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u) {
+                const int o = o0 + (u * kCopyThreads + (int)threadIdx.x) * 16;
+                if (o < cp.row_bytes) v[u] = ld16(src + o);
+            }
+#pragma unroll
+            for (int u = 0; u < kCopyUnroll; ++u) {
+                const int o = o0 + (u * kCopyThreads + (int)threadIdx.x) * 16;
+                if (o < cp.row_bytes) st16(dst + o, v[u]);
+            }
+        }
     }
 }
 
@@ -339,8 +368,11 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
         attr_set = true;
     }
-    hipLaunchKernelGGL(cache_plan_kernel, dim3(1), dim3(kPlanThreads), lds, s, mask, c->b.cur_mask, c->b.indices,
-                       c->b.state, c->b.scratch, I);
+    {
+        ProfScope ps(ST_K_CACHE_PLAN, s);
+        hipLaunchKernelGGL(cache_plan_kernel, dim3(1), dim3(kPlanThreads), lds, s, mask, c->b.cur_mask, c->b.indices,
+                           c->b.state, c->b.scratch, I);
+    }
     ST_HIP(hipGetLastError());
     CopyPlan cp;
     cp.nmat = 0;
@@ -355,8 +387,11 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     for (int k = cp.nmat; k < 3; ++k) { cp.pool[k] = nullptr; cp.active[k] = nullptr; }
     cp.row_bytes = (int)(c->H * c->esz);
     const int grid = 8 * device_cu_count();
-    hipLaunchKernelGGL(cache_copy_kernel, dim3(grid), dim3(256), 0, s, cp, c->b.state, c->b.scratch + c->I,
-                       c->b.indices);
+    {
+        ProfScope ps(ST_K_CACHE_COPY, s);
+        hipLaunchKernelGGL(cache_copy_kernel, dim3(grid), dim3(kCopyThreads), 0, s, cp, c->b.state, c->b.scratch,
+                           c->b.scratch + c->I, (int)c->I);
+    }
     ST_HIP(hipGetLastError());
     return ST_OK;
 }

@@ -3,6 +3,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <vector>
 
 namespace st {
 
@@ -35,7 +36,69 @@ int device_cu_count()
     return cached[dev];
 }
 
+// ---- per-kernel event timing ------------------------------------------------
+struct ProfState {
+    bool on = false;
+    int cap = 0, used = 0;
+    std::vector<hipEvent_t> start, stop;
+    std::vector<int> kind;
+};
+static ProfState g_prof;
+
+ProfScope::ProfScope(int kind, hipStream_t s) : slot(-1), stream(s)
+{
+    if (!g_prof.on || g_prof.used >= g_prof.cap) return;
+    slot = g_prof.used++;
+    g_prof.kind[slot] = kind;
+    (void)hipEventRecord(g_prof.start[slot], stream);
+}
+ProfScope::~ProfScope()
+{
+    if (slot >= 0) (void)hipEventRecord(g_prof.stop[slot], stream);
+}
+
 }  // namespace st
+
+extern "C" int st_profile_enable(int max_samples)
+{
+    using namespace st;
+    ST_REQUIRE(max_samples > 0 && max_samples <= (1 << 20), "st_profile_enable: max_samples out of range");
+    while ((int)g_prof.start.size() < max_samples) {
+        hipEvent_t a, b;
+        ST_HIP(hipEventCreate(&a));
+        ST_HIP(hipEventCreate(&b));
+        g_prof.start.push_back(a);
+        g_prof.stop.push_back(b);
+    }
+    g_prof.kind.assign(max_samples, 0);
+    g_prof.cap = max_samples;
+    g_prof.used = 0;
+    g_prof.on = true;
+    return ST_OK;
+}
+
+extern "C" int st_profile_disable(void)
+{
+    st::g_prof.on = false;
+    return ST_OK;
+}
+
+extern "C" int st_profile_collect(int *kinds, float *ms, int cap)
+{
+    using namespace st;
+    ST_REQUIRE(kinds && ms && cap >= 0, "st_profile_collect: bad arguments");
+    int nout = 0;
+    for (int i = 0; i < g_prof.used && nout < cap; ++i) {
+        ST_HIP(hipEventSynchronize(g_prof.stop[i]));
+        float t = 0.f;
+        ST_HIP(hipEventElapsedTime(&t, g_prof.start[i], g_prof.stop[i]));
+        kinds[nout] = g_prof.kind[i];
+        ms[nout] = t;
+        ++nout;
+    }
+    g_prof.used = 0;
+    return nout;
+}
 
 extern "C" int st_version(void) { return 1; }
 extern "C" const char *st_last_error(void) { return st::g_err; }

@@ -18,34 +18,42 @@
 // and SkipMLP._forward_sparse_weight_cache (src/modeling_skip.py:114-117).
 #include "st_common.h"
 
+#include <cstdlib>
+
+// Timeline hook: a build that defines ST_TL(i) before including this file can
+// record a timestamp at stage i of the decode kernel; the library build leaves
+// it empty.
+#ifndef ST_TL
+#define ST_TL(i)
+#endif
+
 namespace st {
 
-constexpr int kMlpThreads = 512;
-constexpr int kMlpWaves = kMlpThreads / kWave;
-constexpr int kMlpMaxGroups = kMlpThreads / kWave;
-
 // T: storage type; NB: x rows per launch; RB: rows per group kept in flight;
-// CPT: 16-byte chunks per thread (2 only when one group spans the block).
-template <typename T, int NB, int RB, int CPT>
-__global__ __launch_bounds__(kMlpThreads) void mlp_decode_kernel(
+// CPT: 16-byte chunks per thread (2 only when one group spans the block);
+// TPB: threads per block (512 leaves 256 VGPRs per thread, 1024 leaves 128).
+template <typename T, int NB, int RB, int CPT, int TPB>
+__global__ __launch_bounds__(TPB) void mlp_decode_kernel(
     const T *__restrict__ x, int B, int H, const T *__restrict__ gate, const T *__restrict__ up,
-    const T *__restrict__ down, int n_host, const int *__restrict__ n_dev, T *__restrict__ combined, long ldc,
-    float *__restrict__ partials, int act, int has_gate, int gs_log2)
+    const T *__restrict__ down, int n_host, const int *__restrict__ n_dev, int n_hint, T *__restrict__ combined,
+    long ldc, float *__restrict__ partials, int act, int has_gate, int gs_log2)
 {
     constexpr int VEC = Elem<T>::kVec;
     extern __shared__ __align__(16) unsigned char region[];  // group combine buffer
-    __shared__ float red[kMlpWaves][RB][NB][2];               // per-wave partial (g,u)
-    __shared__ float hs[kMlpMaxGroups][RB][NB];               // h of the rows in flight
+    constexpr int kMlpThreads = TPB;
+    __shared__ float red[TPB / kWave][RB][NB][2];             // per-wave partial (g,u)
+    __shared__ float hs[TPB / kWave][RB][NB];                 // h of the rows in flight
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int G = gridDim.x, blk = blockIdx.x;
-    int n = n_host;
-    if (n_dev) {
-        const int nd = *n_dev;
-        n = nd < n ? nd : n;
-        if (n < 0) n = 0;
-    }
-    const int r0 = (int)(((long)blk * n) / G), r1 = (int)(((long)(blk + 1) * n) / G);
+    // Active count: requested first, consumed only after the first batch of
+    // weight loads has been issued.  Rows are dealt to blocks round-robin
+    // (row j belongs to block j % G), so which rows a block owns does not
+    // depend on the count, and rows below `n_spec` can be requested before
+    // the count has arrived (the active buffers hold I rows, so this is safe).
+    ST_TL(0);
+    const int nd_raw = n_dev ? *n_dev : n_host;
+    const int n_spec = n_dev ? (n_hint < n_host ? n_hint : n_host) : n_host;
     const int chunks = H / VEC;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
 
@@ -66,6 +74,24 @@ __global__ __launch_bounds__(kMlpThreads) void mlp_decode_kernel(
 #pragma unroll
         for (int q = 0; q < CPT; ++q) xr[b][q] = (valid[q] && b < B) ? ld16(x + (size_t)b * H + coff[q]) : zero4;
 
+    uint4 wg[RB][CPT], wu[RB][CPT], wd[RB][CPT];
+#pragma unroll
+    for (int k = 0; k < RB; ++k) {
+        const int row = blk + G * (grp + ngrp * k);
+#pragma unroll
+        for (int q = 0; q < CPT; ++q) {
+            const bool ok = valid[q] && row < n_spec;
+            const size_t o = (size_t)row * H + coff[q];
+            wg[k][q] = (ok && has_gate) ? ld16(gate + o) : zero4;
+            wu[k][q] = ok ? ld16(up + o) : zero4;
+            wd[k][q] = ok ? ld16(down + o) : zero4;
+        }
+    }
+
+    ST_TL(1);
+    int n = nd_raw < n_host ? nd_raw : n_host;
+    if (n < 0) n = 0;
+
     float acc[NB][CPT][VEC];
 #pragma unroll
     for (int b = 0; b < NB; ++b)
@@ -74,21 +100,25 @@ __global__ __launch_bounds__(kMlpThreads) void mlp_decode_kernel(
 #pragma unroll
             for (int e = 0; e < VEC; ++e) acc[b][q][e] = 0.f;
 
-    const int rpg = (r1 - r0 + ngrp - 1) / ngrp;  // rows per group, uniform over the block
-    const int nbat = (rpg + RB - 1) / RB;
+    const int jcount = n > blk ? (n - blk + G - 1) / G : 0;  // rows of this block
+    const int nbat = ((jcount + ngrp - 1) / ngrp + RB - 1) / RB;  // uniform over the block
     for (int bat = 0; bat < nbat; ++bat) {
-        const int base = r0 + grp + bat * RB * ngrp;
-        uint4 wg[RB][CPT], wu[RB][CPT], wd[RB][CPT];
 #pragma unroll
         for (int k = 0; k < RB; ++k) {
-            const int row = base + k * ngrp;
+            const int row = blk + G * (grp + ngrp * (bat * RB + k));
+            // batch 0 was requested speculatively; fetch what the guess missed, drop what it overshot
+            const bool have = bat == 0 && row < n_spec;
 #pragma unroll
             for (int q = 0; q < CPT; ++q) {
-                const bool ok = valid[q] && row < r1;
+                const bool ok = valid[q] && row < n;
                 const size_t o = (size_t)row * H + coff[q];
-                wg[k][q] = (ok && has_gate) ? ld16(gate + o) : zero4;
-                wu[k][q] = ok ? ld16(up + o) : zero4;
-                wd[k][q] = ok ? ld16(down + o) : zero4;
+                if (!have) {
+                    wg[k][q] = (ok && has_gate) ? ld16(gate + o) : zero4;
+                    wu[k][q] = ok ? ld16(up + o) : zero4;
+                    wd[k][q] = ok ? ld16(down + o) : zero4;
+                } else if (!ok) {
+                    wg[k][q] = zero4; wu[k][q] = zero4; wd[k][q] = zero4;
+                }
             }
         }
         // ---- phase 1: partial dot products on this thread's chunk(s)
@@ -125,18 +155,20 @@ __global__ __launch_bounds__(kMlpThreads) void mlp_decode_kernel(
                     red[wave][k][b][1] = su;
                 }
             }
+        ST_TL(2);
         __syncthreads();
+        ST_TL(3);
         if (tid < ngrp * RB * NB) {
             const int g_ = tid / (RB * NB), rem = tid - g_ * (RB * NB);
             const int k_ = rem / NB, b_ = rem - k_ * NB;
-            const int row = r0 + g_ + (bat * RB + k_) * ngrp;
+            const int row = blk + G * (g_ + ngrp * (bat * RB + k_));
             float sg = 0.f, su = 0.f;
             for (int w = g_ * wpg; w < (g_ + 1) * wpg; ++w) {
                 sg += red[w][k_][b_][0];
                 su += red[w][k_][b_][1];
             }
             const float hv = has_gate ? activate(sg, act) * su : activate(su, act);
-            const bool ok = row < r1;
+            const bool ok = row < n;
             hs[g_][k_][b_] = ok ? hv : 0.f;
             if (ok && combined && b_ < B) {
                 combined[(size_t)b_ * ldc + row] = from_float<T>(hv);
@@ -144,6 +176,7 @@ __global__ __launch_bounds__(kMlpThreads) void mlp_decode_kernel(
             }
         }
         __syncthreads();
+        ST_TL(4);
         // ---- phase 2: down projection from the rows already in registers
 #pragma unroll
         for (int k = 0; k < RB; ++k)
@@ -160,6 +193,7 @@ __global__ __launch_bounds__(kMlpThreads) void mlp_decode_kernel(
             }
     }
 
+    ST_TL(5);
     // ---- combine the thread groups through LDS (CPT == 1 whenever ngrp > 1)
     if (ngrp > 1) {
         float *redc = reinterpret_cast<float *>(region);  // [ngrp-1][NB][H]
@@ -196,6 +230,7 @@ __global__ __launch_bounds__(kMlpThreads) void mlp_decode_kernel(
                         make_float4(acc[b][q][e], acc[b][q][e + 1], acc[b][q][e + 2], acc[b][q][e + 3]);
         }
     }
+    ST_TL(6);
 }
 
 // out[b, c] = sum over blocks of partials[blk][b][c], fixed order.
@@ -209,9 +244,17 @@ __global__ __launch_bounds__(256) void mlp_reduce_kernel(const float *__restrict
     const int col = blockIdx.x * 64 + q * 4;
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     if (col < H) {
-        for (int blk = rg; blk < G; blk += 16) {
-            const float4 v = *reinterpret_cast<const float4 *>(partials + ((size_t)blk * NB + b) * H + col);
-            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        // 16 partial rows per thread are requested together (one memory round trip for G <= 256)
+        for (int blk0 = rg; blk0 < G; blk0 += 16 * 16) {
+            float4 v[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                const int blk = blk0 + 16 * k;
+                v[k] = blk < G ? *reinterpret_cast<const float4 *>(partials + ((size_t)blk * NB + b) * H + col)
+                               : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int k = 0; k < 16; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
         }
     }
     red[rg][q] = s;
@@ -235,7 +278,7 @@ constexpr int kMaxLds = 160 * 1024;
 struct MlpLaunch {
     const void *x; int B; int H;
     const void *gate, *up, *down;
-    int n; const int *n_dev;
+    int n; const int *n_dev; int n_hint;
     void *out; void *combined; long ldc;
     float *partials;
     int act, has_gate;
@@ -243,12 +286,17 @@ struct MlpLaunch {
     int G;
 };
 
-template <typename T, int NB, int RB, int CPT> static int launch_inst(const MlpLaunch &a, int b0, int bcount, int gs_log2)
+template <typename T, int NB, int RB, int CPT, int TPB>
+static int launch_inst(const MlpLaunch &a, int b0, int bcount)
 {
-    const int ngrp = kMlpThreads >> gs_log2;
+    const int chunks = a.H / Elem<T>::kVec;
+    int gs_log2 = 6;
+    while ((1 << gs_log2) < chunks && (1 << gs_log2) < TPB) ++gs_log2;
+    ST_REQUIRE(chunks <= CPT * (1 << gs_log2), "st_mlp_forward: hidden size %d too large for this dtype", a.H);
+    const int ngrp = TPB >> gs_log2;
     const size_t lds = (size_t)(ngrp - 1) * NB * a.H * 4;
     ST_REQUIRE(lds <= (size_t)kMaxLds - 8192, "st_mlp_forward: H=%d needs %zu bytes of LDS", a.H, lds);
-    auto kern = mlp_decode_kernel<T, NB, RB, CPT>;
+    auto kern = mlp_decode_kernel<T, NB, RB, CPT, TPB>;
     static bool attr_set = false;
     if (!attr_set) {
         ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -257,48 +305,61 @@ template <typename T, int NB, int RB, int CPT> static int launch_inst(const MlpL
     }
     const T *x = static_cast<const T *>(a.x) + (size_t)b0 * a.H;
     T *comb = a.combined ? static_cast<T *>(a.combined) + (size_t)b0 * a.ldc : nullptr;
-    hipLaunchKernelGGL(kern, dim3(a.G), dim3(kMlpThreads), lds, a.stream, x, bcount, a.H,
-                       static_cast<const T *>(a.gate), static_cast<const T *>(a.up), static_cast<const T *>(a.down),
-                       a.n, a.n_dev, comb, a.ldc, a.partials, a.act, a.has_gate, gs_log2);
+    {
+        ProfScope ps(ST_K_MLP_DECODE, a.stream);
+        hipLaunchKernelGGL(kern, dim3(a.G), dim3(TPB), lds, a.stream, x, bcount, a.H,
+                           static_cast<const T *>(a.gate), static_cast<const T *>(a.up),
+                           static_cast<const T *>(a.down), a.n, a.n_dev, a.n_hint, comb, a.ldc, a.partials, a.act,
+                           a.has_gate, gs_log2);
+    }
     ST_HIP(hipGetLastError());
     T *out = static_cast<T *>(a.out) + (size_t)b0 * a.H;
-    hipLaunchKernelGGL(mlp_reduce_kernel<T>, dim3((a.H + 63) / 64, bcount), dim3(256), 0, a.stream, a.partials, a.G,
-                       NB, bcount, a.H, out);
+    {
+        ProfScope ps(ST_K_MLP_REDUCE, a.stream);
+        hipLaunchKernelGGL(mlp_reduce_kernel<T>, dim3((a.H + 63) / 64, bcount), dim3(256), 0, a.stream, a.partials,
+                           a.G, NB, bcount, a.H, out);
+    }
     ST_HIP(hipGetLastError());
     return ST_OK;
 }
 
-// Picks the rows-in-flight depth: the smallest instantiated RB that covers the
-// rows a group owns, so the common case is a single batch with every load of
-// the block issued before any arithmetic.
+// Tuning knobs (0 = automatic), read once from the environment: ST_MLP_TPB
+// (512 | 1024) and ST_MLP_RB (rows a thread group keeps in flight).
+static int env_int(const char *name)
+{
+    const char *v = getenv(name);
+    return v ? atoi(v) : 0;
+}
+
+// The launch shape trades registers for loads in flight: measured on MI355X,
+// about 12-18 outstanding 16-byte loads per thread with 16 waves per CU
+// streams fastest; many more per thread is slower.
 template <typename T, int NB> static int launch_one(const MlpLaunch &a, int b0, int bcount)
 {
+    static const int want_tpb = env_int("ST_MLP_TPB"), want_rb = env_int("ST_MLP_RB");
     const int chunks = a.H / Elem<T>::kVec;
-    ST_REQUIRE(chunks <= 2 * kMlpThreads, "st_mlp_forward: hidden size %d too large for this dtype (max %d)", a.H,
-               2 * kMlpThreads * Elem<T>::kVec);
-    if (chunks > kMlpThreads) {
-        const int rows = (a.n + a.G - 1) / a.G;
-        if constexpr (NB == 1) {
-            if (rows <= 4) return launch_inst<T, NB, 4, 2>(a, b0, bcount, 9);
-            return launch_inst<T, NB, 7, 2>(a, b0, bcount, 9);
-        } else {
-            return launch_inst<T, NB, 2, 2>(a, b0, bcount, 9);
-        }
-    }
-    int gs_log2 = 6;
-    while ((1 << gs_log2) < chunks) ++gs_log2;
-    const int ngrp = kMlpThreads >> gs_log2;
-    const int rows = ((a.n + a.G - 1) / a.G + ngrp - 1) / ngrp;
+    ST_REQUIRE(chunks <= 2048, "st_mlp_forward: hidden size %d too large for this dtype (max %d)", a.H,
+               2048 * Elem<T>::kVec);
     if constexpr (NB == 1) {
-        if (rows <= 4) return launch_inst<T, NB, 4, 1>(a, b0, bcount, gs_log2);
-        if (rows <= 8) return launch_inst<T, NB, 8, 1>(a, b0, bcount, gs_log2);
-        if (rows <= 12) return launch_inst<T, NB, 12, 1>(a, b0, bcount, gs_log2);
-        return launch_inst<T, NB, 15, 1>(a, b0, bcount, gs_log2);
+        if (chunks > 1024) return launch_inst<T, 1, 3, 2, 1024>(a, b0, bcount);
+        if (want_tpb == 512 || (want_tpb == 0 && false)) {
+            if (chunks > 512) return want_rb == 4 ? launch_inst<T, 1, 4, 2, 512>(a, b0, bcount)
+                                                 : launch_inst<T, 1, 6, 2, 512>(a, b0, bcount);
+            switch (want_rb) {
+            case 4: return launch_inst<T, 1, 4, 1, 512>(a, b0, bcount);
+            case 8: return launch_inst<T, 1, 8, 1, 512>(a, b0, bcount);
+            case 12: return launch_inst<T, 1, 12, 1, 512>(a, b0, bcount);
+            default: return launch_inst<T, 1, 6, 1, 512>(a, b0, bcount);
+            }
+        }
+        if (want_rb == 4) return launch_inst<T, 1, 4, 1, 1024>(a, b0, bcount);
+        return launch_inst<T, 1, 6, 1, 1024>(a, b0, bcount);
     } else if constexpr (NB == 2) {
-        if (rows <= 4) return launch_inst<T, NB, 4, 1>(a, b0, bcount, gs_log2);
-        return launch_inst<T, NB, 8, 1>(a, b0, bcount, gs_log2);
+        if (chunks > 1024) return launch_inst<T, 2, 2, 2, 512>(a, b0, bcount);
+        return launch_inst<T, 2, 4, 1, 1024>(a, b0, bcount);
     } else {
-        return launch_inst<T, NB, 4, 1>(a, b0, bcount, gs_log2);
+        if (chunks > 512) return launch_inst<T, 4, 2, 2, 512>(a, b0, bcount);
+        return launch_inst<T, 4, 4, 1, 512>(a, b0, bcount);
     }
 }
 
@@ -335,9 +396,9 @@ extern "C" int64_t st_mlp_workspace_bytes(int64_t B, int64_t H)
 }
 
 extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
-                              const void *down_rows, int64_t n, const int32_t *n_dev, void *out, void *combined,
-                              int64_t ldc, void *workspace, int64_t workspace_bytes, int act, int dtype, int has_gate,
-                              void *stream)
+                              const void *down_rows, int64_t n, const int32_t *n_dev, int64_t n_hint, void *out,
+                              void *combined, int64_t ldc, void *workspace, int64_t workspace_bytes, int act,
+                              int dtype, int has_gate, void *stream)
 {
     using namespace st;
     ST_REQUIRE(x && up_rows && down_rows && out && workspace, "st_mlp_forward: null pointer");
@@ -360,6 +421,7 @@ extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *g
     a.x = x; a.B = (int)B; a.H = (int)H;
     a.gate = gate_rows; a.up = up_rows; a.down = down_rows;
     a.n = (int)n; a.n_dev = n_dev;
+    a.n_hint = (int)(n_hint < 0 ? 0 : (n_hint > n ? n : n_hint));
     a.out = out; a.combined = combined; a.ldc = (long)ldc;
     a.partials = static_cast<float *>(workspace);
     a.act = act; a.has_gate = has_gate ? 1 : 0;

@@ -12,94 +12,163 @@
 namespace st {
 
 constexpr int kPredBTile = 8;
+constexpr int kPredDownThreads = 256;
+constexpr int kPredDownUnroll = 4;  // chunks per thread issued together
 
+// One block per rank row k: all loads of the row (and of x) are issued before
+// any arithmetic, so the kernel costs one memory round trip.
 template <typename T>
-__global__ __launch_bounds__(kWave) void predictor_down_kernel(const T *__restrict__ x, int B, int H,
-                                                               const T *__restrict__ A, int r, float *__restrict__ t)
+__global__ __launch_bounds__(kPredDownThreads) void predictor_down_kernel(const T *__restrict__ x, int B, int H,
+                                                                          const T *__restrict__ A, int r,
+                                                                          float *__restrict__ t)
 {
     constexpr int VEC = Elem<T>::kVec;
-    const int k = blockIdx.x, lane = threadIdx.x;
+    __shared__ float red[kPredDownThreads / kWave][kPredBTile];
+    const int k = blockIdx.x, tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int chunks = H / VEC;
     const T *row = A + (size_t)k * H;
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
     for (int b0 = 0; b0 < B; b0 += kPredBTile) {
         float acc[kPredBTile];
 #pragma unroll
         for (int b = 0; b < kPredBTile; ++b) acc[b] = 0.f;
-        for (int c = lane; c < chunks; c += kWave) {
-            float fw[VEC];
-            unpack<T>(ld16(row + (size_t)c * VEC), fw);
+        for (int c0 = 0; c0 < chunks; c0 += kPredDownThreads * kPredDownUnroll) {
+            uint4 w[kPredDownUnroll];
+#pragma unroll
+            for (int u = 0; u < kPredDownUnroll; ++u) {
+                const int c = c0 + u * kPredDownThreads + tid;
+                w[u] = c < chunks ? ld16(row + (size_t)c * VEC) : zero4;
+            }
 #pragma unroll
             for (int b = 0; b < kPredBTile; ++b) {
                 if (b0 + b < B) {
-                    float fx[VEC];
-                    unpack<T>(ld16(x + (size_t)(b0 + b) * H + (size_t)c * VEC), fx);
+                    uint4 xv[kPredDownUnroll];
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) acc[b] = fmaf(fw[e], fx[e], acc[b]);
+                    for (int u = 0; u < kPredDownUnroll; ++u) {
+                        const int c = c0 + u * kPredDownThreads + tid;
+                        xv[u] = c < chunks ? ld16(x + (size_t)(b0 + b) * H + (size_t)c * VEC) : zero4;
+                    }
+#pragma unroll
+                    for (int u = 0; u < kPredDownUnroll; ++u) {
+                        float fw[VEC], fx[VEC];
+                        unpack<T>(w[u], fw);
+                        unpack<T>(xv[u], fx);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) acc[b] = fmaf(fw[e], fx[e], acc[b]);
+                    }
                 }
             }
         }
 #pragma unroll
         for (int b = 0; b < kPredBTile; ++b) {
-            const float s = wave_sum(acc[b]);
-            if (lane == 0 && b0 + b < B) t[(size_t)(b0 + b) * r + k] = s;
+            const float s = wave_sum_dpp(acc[b]);
+            if (lane == 0) red[wave][b] = s;
         }
+        __syncthreads();
+        if (tid < kPredBTile && b0 + tid < B) {
+            float s = 0.f;
+#pragma unroll
+            for (int w2 = 0; w2 < kPredDownThreads / kWave; ++w2) s += red[w2][tid];
+            t[(size_t)(b0 + tid) * r + k] = s;
+        }
+        __syncthreads();
     }
 }
 
 constexpr int kPredRowsPerWave = 16;
+constexpr int kPredUpBTile = 4;
 
-// lpr_log2: lanes that share one row of Bm (2^lpr_log2 >= r/VEC, capped at 64)
-template <typename T>
+// LPR lanes share one row of Bm (LPR >= r/VEC unless the row needs several
+// passes); a wave owns 16 consecutive rows and issues the loads of all of them
+// before the rank-r intermediate is staged in LDS.
+template <typename T, int LPR>
 __global__ __launch_bounds__(kWave) void predictor_up_mask_kernel(const float *__restrict__ t, int B, int r,
                                                                   const T *__restrict__ Bm, int I, float thr,
-                                                                  int cmp_ge, int lpr_log2,
-                                                                  float *__restrict__ scores,
+                                                                  int cmp_ge, float *__restrict__ scores,
                                                                   uint8_t *__restrict__ mask)
 {
     constexpr int VEC = Elem<T>::kVec;
+    constexpr int RPI = kWave / LPR;                                          // rows per iteration
+    constexpr int NIT = kPredRowsPerWave / RPI > 0 ? kPredRowsPerWave / RPI : 1;  // iterations per tile
     extern __shared__ __align__(16) unsigned char smem[];
     float *ts = reinterpret_cast<float *>(smem);  // [B][r]
     const int lane = threadIdx.x;
-    for (int i = lane; i < B * r; i += kWave) ts[i] = t[i];
-    __syncthreads();
-
     const int chunks = r / VEC;
-    const int LPR = 1 << lpr_log2, rpi = kWave >> lpr_log2;  // rows per iteration
-    const int cl = lane & (LPR - 1), gidx = lane >> lpr_log2;
+    const int cl = lane & (LPR - 1), gidx = lane / LPR;
     const int tile = blockIdx.x * kPredRowsPerWave;
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
 
-    for (int it = 0; it * rpi < kPredRowsPerWave; ++it) {
-        const int row = tile + it * rpi + gidx;
-        const bool row_ok = row < I && (it * rpi + gidx) < kPredRowsPerWave;
-        bool any = false;
-        for (int b0 = 0; b0 < B; b0 += kPredBTile) {
-            float s[kPredBTile];
+    float s[NIT][kPredUpBTile];
+    bool any[NIT];
 #pragma unroll
-            for (int b = 0; b < kPredBTile; ++b) s[b] = 0.f;
-            for (int c = cl; c < chunks; c += LPR) {
-                float fw[VEC];
-                const uint4 w = row_ok ? ld16(Bm + (size_t)row * r + (size_t)c * VEC) : make_uint4(0u, 0u, 0u, 0u);
-                unpack<T>(w, fw);
+    for (int it = 0; it < NIT; ++it) any[it] = false;
+
+    for (int b0 = 0; b0 < B || b0 == 0; b0 += kPredUpBTile) {
 #pragma unroll
-                for (int b = 0; b < kPredBTile; ++b) {
-                    if (b0 + b < B) {
-                        const float *tp = ts + (size_t)(b0 + b) * r + c * VEC;
+        for (int it = 0; it < NIT; ++it)
 #pragma unroll
-                        for (int e = 0; e < VEC; ++e) s[b] = fmaf(fw[e], tp[e], s[b]);
+            for (int b = 0; b < kPredUpBTile; ++b) s[it][b] = 0.f;
+        for (int c = cl; c < chunks || c == cl; c += LPR) {  // one pass unless r/VEC > LPR
+            uint4 w[NIT];
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+                const int ro = it * RPI + gidx;
+                const int row = tile + ro;
+                w[it] = (c < chunks && ro < kPredRowsPerWave && row < I) ? ld16(Bm + (size_t)row * r + (size_t)c * VEC)
+                                                                        : zero4;
+            }
+            if (b0 == 0 && c == cl) {  // stage t after the row loads are in flight
+                for (int i = lane; i < B * r; i += kWave) ts[i] = t[i];
+                __syncthreads();
+            }
+            if (c < chunks) {
+#pragma unroll
+                for (int it = 0; it < NIT; ++it) {
+                    float fw[VEC];
+                    unpack<T>(w[it], fw);
+#pragma unroll
+                    for (int b = 0; b < kPredUpBTile; ++b) {
+                        if (b0 + b < B) {
+                            const float *tp = ts + (size_t)(b0 + b) * r + c * VEC;
+#pragma unroll
+                            for (int e = 0; e < VEC; ++e) s[it][b] = fmaf(fw[e], tp[e], s[it][b]);
+                        }
                     }
                 }
             }
+            if (c + LPR >= chunks) break;
+        }
 #pragma unroll
-            for (int b = 0; b < kPredBTile; ++b) {
+        for (int it = 0; it < NIT; ++it) {
+            const int ro = it * RPI + gidx;
+            const int row = tile + ro;
+            const bool row_ok = ro < kPredRowsPerWave && row < I;
+#pragma unroll
+            for (int b = 0; b < kPredUpBTile; ++b) {
                 if (b0 + b < B) {  // uniform across the wave
-                    const float v = group_sum(s[b], LPR);
-                    any = any || (cmp_ge ? (v >= thr) : (v > thr));
+                    const float v = group_sum(s[it][b], LPR);
+                    any[it] = any[it] || (cmp_ge ? (v >= thr) : (v > thr));
                     if (scores && cl == 0 && row_ok) scores[(size_t)(b0 + b) * I + row] = v;
                 }
             }
         }
-        if (cl == 0 && row_ok) mask[row] = any ? 1 : 0;
+        if (b0 + kPredUpBTile >= B) break;
     }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+        const int ro = it * RPI + gidx;
+        const int row = tile + ro;
+        if (cl == 0 && ro < kPredRowsPerWave && row < I) mask[row] = any[it] ? 1 : 0;
+    }
+}
+
+template <typename T, int LPR>
+static void launch_up(const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge, float *scores,
+                      uint8_t *mask, hipStream_t stream)
+{
+    const size_t lds = (size_t)B * r * sizeof(float);
+    hipLaunchKernelGGL((predictor_up_mask_kernel<T, LPR>), dim3((I + kPredRowsPerWave - 1) / kPredRowsPerWave),
+                       dim3(kWave), lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask);
 }
 
 template <typename T>
@@ -107,15 +176,21 @@ static int launch_predictor(const void *x, int B, int H, const void *A, int r, c
                             int cmp_ge, float *t_ws, float *scores, uint8_t *mask, hipStream_t stream)
 {
     constexpr int VEC = Elem<T>::kVec;
-    hipLaunchKernelGGL(predictor_down_kernel<T>, dim3(r), dim3(kWave), 0, stream, static_cast<const T *>(x), B, H,
-                       static_cast<const T *>(A), r, t_ws);
+    {
+        ProfScope ps(ST_K_PRED_DOWN, stream);
+        hipLaunchKernelGGL(predictor_down_kernel<T>, dim3(r), dim3(kPredDownThreads), 0, stream,
+                           static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
+    }
     ST_HIP(hipGetLastError());
     const int chunks = r / VEC;
-    int lpr_log2 = 0;
-    while ((1 << lpr_log2) < chunks && lpr_log2 < 6) ++lpr_log2;
-    const size_t lds = (size_t)B * r * sizeof(float);
-    hipLaunchKernelGGL(predictor_up_mask_kernel<T>, dim3((I + kPredRowsPerWave - 1) / kPredRowsPerWave), dim3(kWave),
-                       lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, lpr_log2, scores, mask);
+    {
+        ProfScope ps(ST_K_PRED_UP_MASK, stream);
+        if (chunks <= 4) launch_up<T, 4>(t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+        else if (chunks <= 8) launch_up<T, 8>(t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+        else if (chunks <= 16) launch_up<T, 16>(t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+        else if (chunks <= 32) launch_up<T, 32>(t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+        else launch_up<T, 64>(t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+    }
     ST_HIP(hipGetLastError());
     return ST_OK;
 }

@@ -145,4 +145,12 @@ int hip_fail(hipError_t e, const char *what);
 
 int device_cu_count();
 
+// Event bracket around one kernel launch; a no-op unless profiling is enabled.
+struct ProfScope {
+    int slot;
+    hipStream_t stream;
+    ProfScope(int kind, hipStream_t s);
+    ~ProfScope();
+};
+
 }  // namespace st

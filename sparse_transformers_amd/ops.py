@@ -64,8 +64,10 @@ def mlp_workspace(device: torch.device, B: int, H: int) -> torch.Tensor:
 
 def mlp_forward_rows(x2: torch.Tensor, gate_rows: Optional[torch.Tensor], up_rows: torch.Tensor,
                      down_rows: torch.Tensor, n: int, n_dev: Optional[torch.Tensor], out: torch.Tensor,
-                     combined: Optional[torch.Tensor], act: str, has_gate: bool) -> None:
-    """Raw launch on packed rows: gate/up/down are [>=n, H] row-major, x2/out are [B, H]."""
+                     combined: Optional[torch.Tensor], act: str, has_gate: bool, n_hint: int = 0) -> None:
+    """Raw launch on packed rows: gate/up/down are [>=n, H] row-major, x2/out are [B, H].
+    With ``n_dev`` (device int32 count) the kernels use min(*n_dev, n); ``n_hint`` is the count the host
+    expects, used only to request rows before the device count has arrived."""
     dev = require_gpu(x2, gate_rows, up_rows, down_rows, out, combined, n_dev)
     B, H = x2.shape
     ws = mlp_workspace(dev, B, H)
@@ -73,7 +75,7 @@ def mlp_forward_rows(x2: torch.Tensor, gate_rows: Optional[torch.Tensor], up_row
         raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
     rc = _lib.lib().st_mlp_forward(
         x2.data_ptr(), B, H, gate_rows.data_ptr() if has_gate else None, up_rows.data_ptr(), down_rows.data_ptr(),
-        int(n), n_dev.data_ptr() if n_dev is not None else None, out.data_ptr(),
+        int(n), n_dev.data_ptr() if n_dev is not None else None, int(n_hint), out.data_ptr(),
         combined.data_ptr() if combined is not None else None, combined.stride(0) if combined is not None else 0,
         ws.data_ptr(), ws.numel(), _lib.ACT_CODES[act], dtype_code(x2), int(bool(has_gate)), current_stream_ptr(dev))
     _lib.check(rc, "st_mlp_forward")
@@ -136,7 +138,8 @@ def sparse_mlp_forward(x: torch.Tensor, concat_weight: torch.Tensor, active_down
 
 
 def predictor_mask(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.Tensor, thr: float = 0.0,
-                   ge: bool = True, return_scores: bool = False, out: Optional[torch.Tensor] = None):
+                   ge: bool = True, return_scores: bool = False, out: Optional[torch.Tensor] = None,
+                   t_ws: Optional[torch.Tensor] = None):
     """mask[i] = any over rows b of ((x @ down^T) @ up^T)[b, i] >= thr  (``>`` when ``ge`` is False).
 
     x: [..., H]; down_weight: [r, H] (FastLoRAProjection.down.weight); up_weight: [I, r].
@@ -157,7 +160,10 @@ def predictor_mask(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.
         raise TypeError("predictor weights and x must share one dtype")
     down_weight = down_weight if down_weight.is_contiguous() else down_weight.contiguous()
     up_weight = up_weight if up_weight.is_contiguous() else up_weight.contiguous()
-    t_ws = torch.empty(B, r, dtype=torch.float32, device=dev)
+    if t_ws is None:
+        t_ws = torch.empty(B, r, dtype=torch.float32, device=dev)
+    elif t_ws.dtype != torch.float32 or t_ws.numel() < B * r or not t_ws.is_cuda:
+        raise ValueError("t_ws must be a float32 GPU tensor with at least B*r elements")
     scores = torch.empty(B, I, dtype=torch.float32, device=dev) if return_scores else None
     mask = out if out is not None else torch.empty(I, dtype=torch.bool, device=dev)
     if mask.dtype != torch.bool or mask.numel() != I or not mask.is_contiguous():

@@ -40,7 +40,8 @@ class FastLoRAProjection:
     __call__ = forward
 
     def mask(self, x: torch.Tensor, method: str = "naive", thr: float = 0.0, ge: bool = True, k: int = 0,
-             std_multiplier: float = 0.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+             std_multiplier: float = 0.0, out: Optional[torch.Tensor] = None,
+             t_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Union-over-rows boolean mask, src/modeling_skip.py:204-214.
 
         ``naive`` (score >= 0) and ``threshold`` (score >= thr, or > thr) are fused into the predictor
@@ -48,9 +49,9 @@ class FastLoRAProjection:
         reductions on the device.
         """
         if method == "naive":
-            return predictor_mask(x, self.down_weight, self.up_weight, 0.0, True, out=out)
+            return predictor_mask(x, self.down_weight, self.up_weight, 0.0, True, out=out, t_ws=t_ws)
         if method == "threshold":
-            return predictor_mask(x, self.down_weight, self.up_weight, thr, ge, out=out)
+            return predictor_mask(x, self.down_weight, self.up_weight, thr, ge, out=out, t_ws=t_ws)
         scores = self.forward(x)
         if method == "topk":
             idx = scores.topk(k, sorted=False)[1]
@@ -111,8 +112,9 @@ class SparseDecodeLayer:
         self.predictor, self.cache, self.act, self.thr, self.ge = predictor, cache, act, thr, ge
         self.mask = torch.zeros(cache.intermediate_size, dtype=torch.bool, device=cache.device)
 
-    def compute_mask_and_update(self, x_pred: torch.Tensor, mask_override: Optional[torch.Tensor] = None) -> None:
-        self.predictor.mask(x_pred, "threshold", self.thr, self.ge, out=self.mask)
+    def compute_mask_and_update(self, x_pred: torch.Tensor, mask_override: Optional[torch.Tensor] = None,
+                                t_ws: Optional[torch.Tensor] = None) -> None:
+        self.predictor.mask(x_pred, "threshold", self.thr, self.ge, out=self.mask, t_ws=t_ws)
         self.cache.update_active_weights_async(self.mask if mask_override is None else mask_override)
 
     def mlp(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -125,6 +127,74 @@ class SparseMLPStack:
 
     def __init__(self, layers: Sequence[SparseDecodeLayer]):
         self.layers: List[SparseDecodeLayer] = list(layers)
+
+    # ---- staged / graph-replayed stepping: fixed device buffers, no allocation, no host reads ----
+    def prepare(self, batch: int, overlap: bool = True) -> None:
+        c0 = self.layers[0].cache
+        dev, dt, H, I = c0.device, c0.dtype, c0.hidden_size, c0.intermediate_size
+        L = len(self.layers)
+        self.x_stage = torch.empty(batch, H, dtype=dt, device=dev)
+        self.xp_stage = torch.empty(L, batch, H, dtype=dt, device=dev)
+        self.mask_stage = torch.empty(L, I, dtype=torch.bool, device=dev)
+        self._pingpong = [torch.empty(batch, H, dtype=dt, device=dev) for _ in range(2)]
+        rmax = max(layer.predictor.lora_size for layer in self.layers)
+        self._t_ws = torch.empty(batch * rmax, dtype=torch.float32, device=dev)
+        self.out = self._pingpong[0]
+        self.graph = None
+        self.use_trace_masks = True
+        self.overlap = overlap
+        self._side = torch.cuda.Stream(device=dev) if overlap else None   # default priority
+        self._ev_fork = torch.cuda.Event()
+        self._ev_upd = [torch.cuda.Event() for _ in range(L)]
+
+    def _enqueue(self) -> None:
+        """One decode step.  With ``overlap`` the predictor + cache update of every layer run on a side
+        stream (they depend on the staged predictor inputs / masks only, as in the reference where the
+        mask is computed from the pre-attention state, src/modeling_skip.py:235-238) and each layer's
+        MLP waits for its own update; the two streams join at the end of the step."""
+        x = self.x_stage
+        main = torch.cuda.current_stream(self.x_stage.device)
+        side = self._side if self.overlap else None
+        if side is not None:
+            self._ev_fork.record(main)
+            side.wait_event(self._ev_fork)
+        for l, layer in enumerate(self.layers):
+            mask = self.mask_stage[l] if self.use_trace_masks else None
+            if side is not None:
+                with torch.cuda.stream(side):
+                    layer.compute_mask_and_update(self.xp_stage[l], mask, t_ws=self._t_ws)
+                    self._ev_upd[l].record(side)
+                main.wait_event(self._ev_upd[l])
+            else:
+                layer.compute_mask_and_update(self.xp_stage[l], mask, t_ws=self._t_ws)
+            out = self._pingpong[l & 1]
+            layer.cache.forward(x, layer.act, out=out)
+            x = out
+        self.out = x
+
+    def capture(self) -> None:
+        """Record one decode step into a HIP graph (call after at least one eager step)."""
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self._enqueue()
+        self.graph = g
+
+    def step_staged(self, x: torch.Tensor, x_pred: torch.Tensor, masks: Optional[torch.Tensor] = None,
+                    replay: bool = False) -> torch.Tensor:
+        """x [B,H], x_pred [L,B,H], masks bool [L,I] (trace-driven cache masks; ignored when
+        ``use_trace_masks`` is False).  Copies the inputs into the staging buffers and either replays
+        the captured graph or launches the kernels eagerly."""
+        self.x_stage.copy_(x)
+        self.xp_stage.copy_(x_pred)
+        if masks is not None:
+            self.mask_stage.copy_(masks)
+        if replay:
+            self.graph.replay()
+            for layer in self.layers:
+                layer.cache._dirty = True
+        else:
+            self._enqueue()
+        return self.out
 
     def decode_step(self, x: torch.Tensor, x_pred: Optional[Sequence[torch.Tensor]] = None,
                     mask_override: Optional[Sequence[torch.Tensor]] = None) -> torch.Tensor:

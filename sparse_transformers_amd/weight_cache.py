@@ -70,7 +70,7 @@ class WeightCache:
             self.scratch.data_ptr())
         self._h = L.st_cache_create(C.byref(bufs), I, H, code, int(self.has_gate))
         if not self._h:
-            raise RuntimeError(f"st_cache_create: {_lib.last_error()}")
+            raise ValueError(_lib.last_error())
 
         up_c = up_weight.detach().contiguous()
         down_c = down_weight.detach().contiguous()
@@ -167,6 +167,8 @@ class WeightCache:
             x2 = x2.contiguous()
         if out is None:
             out = torch.empty_like(x2)
+        # the last count the host saw is only a prefetch hint; the kernels read the true one on the device
         mlp_forward_rows(x2, self.gate_active, self.up_active, self.down_active, self.intermediate_size,
-                         self.n_active_dev, out, combined, act, self.has_gate)
+                         self.n_active_dev, out, combined, act, self.has_gate,
+                         n_hint=int(self._host_state[_lib.STATE_N_ACTIVE]))
         return out.view(x.shape)

@@ -1,0 +1,143 @@
+"""Fused sparse MLP on the GPU vs the oracle (float64-accumulating CPU restatement), through the C ABI.
+
+Tolerances (north star): fp32 1e-5 relative; fp16 / bf16 2e-2 absolute, 1e-2 relative, against an fp32
+evaluation of the dtype-rounded weights and inputs."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import sparse_transformers_amd as st
+from sparse_transformers_amd.ops import mlp_forward_rows
+from conftest import assert_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _case(seed, B, H, n, dtype, has_gate, std=0.02, lead_shape=None):
+    g = torch.Generator().manual_seed(seed)
+    tdt = getattr(torch, dtype)
+    cw = (torch.randn((2 if has_gate else 1) * n, H, generator=g) * std).to(tdt)
+    dn = (torch.randn(n, H, generator=g) * std).to(tdt)
+    x = torch.randn(*(lead_shape or (B,)), H, generator=g).to(tdt)
+    return x, cw, dn
+
+
+def _run(x, cw, dn, act, has_gate):
+    H = x.shape[-1]
+    db = torch.zeros(1, H, dtype=x.dtype, device=DEV)
+    cb = torch.zeros(1, 2, dtype=x.dtype, device=DEV)
+    out = st.sparse_mlp_forward(x.to(DEV), cw.to(DEV), dn.to(DEV).t(), db, cb, act, has_gate)
+    torch.cuda.synchronize()
+    return out, db, cb
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16"])
+@pytest.mark.parametrize("act", ["silu", "relu", "gelu_pytorch_tanh", "sigmoid"])
+@pytest.mark.parametrize("has_gate", [True, False])
+def test_forward_vs_oracle_small(dtype, act, has_gate):
+    for seed, (B, H, n) in enumerate([(1, 64, 5), (1, 256, 300), (2, 128, 77), (3, 1024, 129), (5, 512, 1000)]):
+        x, cw, dn = _case(seed, B, H, n, dtype, has_gate, std=0.05)
+        out, db, cb = _run(x, cw, dn, act, has_gate)
+        want, wantc = oracle.mlp_forward(x.float().numpy(), cw.float().numpy(), dn.float().numpy().T, act, has_gate)
+        assert out.shape == x.shape and out.data_ptr() == db.data_ptr()        # aliases down_proj_buffer
+        assert tuple(db.shape) == (B, H) and tuple(cb.shape) == (B, cw.shape[0])  # buffers resized in place
+        assert_close(out.float().cpu().numpy(), want, dtype, f"out B={B} H={H} n={n}")
+        assert_close(cb.float().cpu().numpy(), wantc, dtype, "combined_proj_buffer")
+
+
+@pytest.mark.parametrize("name,B,H,n,dtype,act,has_gate", [
+    ("cfg1 llama-1b layer", 1, 2048, 2457, "float32", "silu", True),
+    ("cfg2 llama-3b layer", 1, 3072, 2867, "float16", "silu", True),
+    ("cfg3 batched decode", 4, 3072, 4620, "bfloat16", "silu", True),
+    ("cfg3 batched decode 8", 8, 3072, 6300, "bfloat16", "silu", True),
+    ("cfg4 mistral-7b layer", 1, 4096, 3584, "bfloat16", "silu", True),
+    ("cfg4 mistral-7b batch 2", 2, 4096, 3584, "bfloat16", "silu", True),
+    ("cfg5 relu-llama gated", 1, 4096, 1100, "float16", "relu", True),
+    ("cfg5 relu-llama ungated", 1, 4096, 1100, "float16", "relu", False),
+    ("fp32 wide rows (two chunks per thread)", 1, 4096, 700, "float32", "silu", True),
+    ("fp32 8192 hidden", 1, 8192, 300, "float32", "relu", True),
+    ("fp16 8192 hidden", 3, 8192, 900, "float16", "silu", True),
+])
+def test_forward_vs_oracle_config_shapes(name, B, H, n, dtype, act, has_gate):
+    x, cw, dn = _case(11, B, H, n, dtype, has_gate, lead_shape=(B, 1))
+    out, _, cb = _run(x, cw, dn, act, has_gate)
+    want, wantc = oracle.mlp_forward(x.float().numpy(), cw.float().numpy(), dn.float().numpy().T, act, has_gate)
+    assert out.shape == (B, 1, H)
+    assert_close(out.float().cpu().numpy(), want, dtype, name)
+    assert_close(cb.float().cpu().numpy(), wantc, dtype, name + " combined")
+
+
+def test_matches_reference_operator_vectors(golden_mlp):
+    """Outputs of the reference's compiled ReLU operator (tests/golden/mlp_forward.json)."""
+    for case in golden_mlp:
+        H, n, hg = case["H"], case["n"], case["has_gate"]
+        x = torch.tensor(case["x"]).reshape(case["x_shape"])
+        cw = torch.tensor(case["concat"]).reshape(-1, H)
+        dn = torch.tensor(case["down_rows"]).reshape(n, H)
+        out, _, cb = _run(x, cw, dn, "relu", hg)
+        np.testing.assert_allclose(out.cpu().numpy().ravel(), np.array(case["out"], np.float32), rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(cb.cpu().numpy().ravel(), np.array(case["combined"], np.float32), rtol=2e-5,
+                                   atol=2e-5)
+
+
+def test_device_count_and_hint_paths():
+    """With a device-side count the result must not depend on the host's hint (too low, exact, too
+    high, absent) nor on rows beyond the count."""
+    I, H, n = 4096, 3072, 1500
+    g = torch.Generator().manual_seed(2)
+    gate = (torch.randn(I, H, generator=g) * 0.02).half().to(DEV)
+    up = (torch.randn(I, H, generator=g) * 0.02).half().to(DEV)
+    dn = (torch.randn(I, H, generator=g) * 0.02).half().to(DEV)
+    x = torch.randn(1, H, generator=g).half().to(DEV)
+    n_dev = torch.tensor([n], dtype=torch.int32, device=DEV)
+    ref = torch.empty(1, H, dtype=torch.float16, device=DEV)
+    mlp_forward_rows(x, gate, up, dn, n, None, ref, None, "silu", True)
+    want, _ = oracle.mlp_forward(x.float().cpu().numpy(), torch.cat([gate[:n], up[:n]]).float().cpu().numpy(),
+                                 dn[:n].float().cpu().numpy().T, "silu", True)
+    assert_close(ref.float().cpu().numpy(), want, "float16", "host count")
+    for hint in (0, 1, 700, n, n + 500, I):
+        out = torch.full((1, H), float("nan"), dtype=torch.float16, device=DEV)
+        mlp_forward_rows(x, gate, up, dn, I, n_dev, out, None, "silu", True, n_hint=hint)
+        assert torch.equal(out, ref), f"hint {hint}"
+    n_dev.fill_(0)
+    out = torch.full((1, H), 1.0, dtype=torch.float16, device=DEV)
+    mlp_forward_rows(x, gate, up, dn, I, n_dev, out, None, "silu", True, n_hint=n)
+    assert not out.any()                                       # empty active set -> zeros
+
+
+def test_run_to_run_determinism_and_linearity_full_size():
+    x, cw, dn = _case(5, 1, 3072, 2867, "float16", True)
+    a, _, _ = _run(x, cw, dn, "silu", True)
+    b, _, _ = _run(x, cw, dn, "silu", True)
+    assert torch.equal(a, b)                                   # fixed summation order
+    # identity activation, ungated: the op is linear in x
+    xs = torch.randn(2, 3072, generator=torch.Generator().manual_seed(1)).float()
+    cwu, dnf = cw[2867:].float(), dn.float()
+    y0, _, _ = _run(xs[:1], cwu, dnf, "identity", False)
+    y0 = y0.clone()
+    y1, _, _ = _run(xs[1:], cwu, dnf, "identity", False)
+    y1 = y1.clone()
+    ys, _, _ = _run(xs[:1] + xs[1:], cwu, dnf, "identity", False)
+    assert_close((y0 + y1).cpu().numpy(), ys.cpu().numpy(), "float32", "linearity")
+
+
+def test_argument_errors():
+    x, cw, dn = _case(0, 1, 64, 8, "float32", True)
+    db = torch.zeros(1, 64, device=DEV)
+    cb = torch.zeros(1, 2, device=DEV)
+    with pytest.raises(ValueError):
+        st.sparse_mlp_forward(x.to(DEV), cw.to(DEV)[:-1], dn.to(DEV).t(), db, cb, "silu")      # odd row count
+    with pytest.raises(ValueError):
+        st.sparse_mlp_forward(x.to(DEV), cw.to(DEV), dn.to(DEV)[:-1].t(), db, cb, "silu")      # n mismatch
+    with pytest.raises(ValueError):
+        st.sparse_mlp_forward(x.to(DEV), cw.to(DEV), dn.to(DEV).t(), db, cb, "tanh")           # unknown act
+    with pytest.raises(TypeError):
+        st.sparse_mlp_forward(x.to(DEV), cw.to(DEV).half(), dn.to(DEV).t(), db, cb, "silu")    # dtype mismatch
+    # a contiguous [H, n] down matrix (not the cache's view) still gives the right answer
+    dwc = dn.to(DEV).t().contiguous()
+    with pytest.warns(UserWarning):
+        out = st.sparse_mlp_forward(x.to(DEV), cw.to(DEV), dwc, db, cb, "silu")
+    want, _ = oracle.mlp_forward(x.numpy(), cw.numpy(), dn.numpy().T, "silu", True)
+    assert_close(out.cpu().numpy(), want, "float32", "repacked down")

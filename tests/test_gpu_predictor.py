@@ -1,0 +1,103 @@
+"""LoRA predictor + threshold mask + batch union on the GPU vs the oracle.  Scores are floating point
+(tolerance); masks are bits and must be exact, so thresholds are placed in a gap between scores that is
+much wider than the rounding difference between the two implementations (the guard band is asserted)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import sparse_transformers_amd as st
+from sparse_transformers_amd import synthetic as syn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _weights(seed, B, H, r, I, dtype):
+    g = torch.Generator().manual_seed(seed)
+    tdt = getattr(torch, dtype)
+    A = (torch.randn(r, H, generator=g) * 0.02).to(tdt)
+    Bm = (torch.randn(I, r, generator=g) * 0.02).to(tdt)
+    x = torch.randn(B, H, generator=g).to(tdt)
+    return x, A, Bm
+
+
+@pytest.mark.parametrize("B,H,r,I,dtype,frac", [
+    (1, 2048, 64, 8192, "float32", 0.30),      # cfg1
+    (1, 3072, 128, 8192, "float16", 0.35),     # cfg2
+    (8, 4096, 256, 14336, "bfloat16", 0.25),   # cfg4, batch union
+    (1, 4096, 440, 11008, "float16", 0.10),    # cfg5: rank int(0.04 * I), 55 chunks per row
+    (16, 3072, 128, 8192, "bfloat16", 0.30),   # cfg3 decode batch 16
+    (3, 128, 8, 50, "float16", 0.5),           # tiny / ragged
+    (2, 64, 4, 17, "float32", 0.5),
+    (1, 1024, 1024, 300, "float16", 0.4),      # rank rows longer than one pass of the wave
+])
+def test_scores_and_mask(B, H, r, I, dtype, frac):
+    x, A, Bm = _weights(B * 7 + r, B, H, r, I, dtype)
+    s_ref = oracle.predictor_scores(x.float().numpy(), A.float().numpy(), Bm.float().numpy())
+    m, s = st.predictor_mask(x.to(DEV), A.to(DEV), Bm.to(DEV), 0.0, True, return_scores=True)
+    s = s.cpu().numpy()
+    scale = np.abs(s_ref).max()
+    assert np.abs(s - s_ref).max() <= 2e-6 * scale + 1e-9           # fp32 accumulation on both sides
+    guard = 8e-6 * scale
+    thr = syn.threshold_for_fraction(s_ref.max(0) if B > 1 else s_ref, frac, guard=0.0)
+    near = np.abs(s_ref - thr) < guard
+    for ge in (True, False):
+        want = oracle.mask_threshold(s_ref, thr, ge)
+        got = st.predictor_mask(x.to(DEV), A.to(DEV), Bm.to(DEV), thr, ge).cpu().numpy()
+        diff = got != want
+        assert not (diff & ~near.any(0)).any(), "mask bit differs outside the guard band"
+        assert diff.sum() <= near.any(0).sum()
+    assert near.sum() <= 3, f"guard band population {near.sum()}"      # expected 0, reported if not
+
+
+def test_naive_threshold_is_score_ge_zero():
+    x, A, Bm = _weights(1, 2, 256, 16, 512, "float32")
+    # make some scores exactly zero: a zero row of Bm gives score 0 for every input row
+    Bm[5] = 0.0
+    Bm[77] = 0.0
+    m_ge = st.predictor_mask(x.to(DEV), A.to(DEV), Bm.to(DEV), 0.0, True).cpu().numpy()
+    m_gt = st.predictor_mask(x.to(DEV), A.to(DEV), Bm.to(DEV), 0.0, False).cpu().numpy()
+    assert m_ge[5] and m_ge[77] and not m_gt[5] and not m_gt[77]     # >= vs > on an exact tie
+    s = oracle.predictor_scores(x.numpy(), A.numpy(), Bm.numpy())
+    safe = np.abs(s).min(0) > 1e-6
+    assert np.array_equal(m_ge[safe], (s >= 0).any(0)[safe])
+
+
+@pytest.mark.parametrize("method", ["naive", "topk", "statistical_topk"])
+def test_mask_methods_of_the_reference(method):
+    """The three sparsity methods of SkipDecoderLayer._compute_binary_mask, union over rows included."""
+    B, H, r, I = 4, 512, 32, 2048
+    x, A, Bm = _weights(3, B, H, r, I, "float32")
+    pred = st.FastLoRAProjection(A.to(DEV), Bm.to(DEV))
+    s_ref = oracle.predictor_scores(x.numpy(), A.numpy(), Bm.numpy())
+    if method == "naive":
+        got = pred.mask(x.to(DEV), "naive").cpu().numpy()
+        want, margin = oracle.mask_threshold(s_ref, 0.0, True), np.abs(s_ref).min(0)
+    elif method == "topk":
+        k = 300
+        got = pred.mask(x.to(DEV), "topk", k=k).cpu().numpy()
+        want = oracle.mask_topk(s_ref, k)
+        kth = np.sort(s_ref, axis=1)[:, -k][:, None]
+        margin = np.abs(s_ref - kth).min(0)
+    else:
+        z = float(torch.distributions.normal.Normal(0, 1).icdf(torch.tensor(0.7)))
+        got = pred.mask(x.to(DEV), "statistical_topk", std_multiplier=z).cpu().numpy()
+        want, cut = oracle.mask_statistical(s_ref, z)
+        margin = np.abs(s_ref - cut[:, None]).min(0)
+    safe = margin > 1e-5 * np.abs(s_ref).max()
+    assert safe.mean() > 0.99
+    assert np.array_equal(got[safe], want[safe])
+
+
+def test_predictor_argument_errors():
+    x, A, Bm = _weights(0, 1, 64, 8, 32, "float32")
+    with pytest.raises(ValueError):
+        st.predictor_mask(x.to(DEV), A.to(DEV)[:, :32], Bm.to(DEV))
+    with pytest.raises(TypeError):
+        st.predictor_mask(x.to(DEV), A.to(DEV).half(), Bm.to(DEV))
+    with pytest.raises(ValueError):
+        st.predictor_mask(x.to(DEV), A.to(DEV), Bm.to(DEV), out=torch.zeros(31, dtype=torch.bool, device=DEV))
+    sd = {"down.weight": A, "up.weight": Bm}
+    p = st.FastLoRAProjection.from_state_dict(sd, device=DEV, dtype=torch.float32)   # the reference's checkpoint keys
+    assert p.lora_size == 8 and p.intermediate_size == 32

@@ -1,0 +1,120 @@
+"""The per-layer sequence (predictor -> mask -> union -> cache update -> sparse MLP) over a small stack,
+GPU vs the oracle pipeline, eager and replayed from a HIP graph."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import sparse_transformers_amd as st
+from sparse_transformers_amd import synthetic as syn
+from conftest import assert_close, round_to
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _build(dtype, L=3, H=256, I=640, r=16, B=1, has_gate=True, act="silu", seed=0):
+    rng = np.random.default_rng(seed)
+    tdt = getattr(torch, dtype)
+    layers, oracles = [], []
+    for _ in range(L):
+        w = syn.layer_weights(rng, H, I, r, std=0.05, has_gate=has_gate)
+        w = {k: (None if v is None else round_to(v, dtype)) for k, v in w.items()}
+        t = {k: (None if v is None else torch.from_numpy(v).to(DEV, tdt)) for k, v in w.items()}
+        init = np.ones(I, bool)
+        cache = st.WeightCache(torch.from_numpy(init).to(DEV), H, t["gate"], t["up"], t["down"], has_gate)
+        layers.append(st.SparseDecodeLayer(st.FastLoRAProjection(t["A"], t["Bm"]), cache, act, 0.0, True))
+        oracles.append((oracle.OracleWeightCache(init, H, w["gate"], w["up"], w["down"], has_gate), w))
+    return st.SparseMLPStack(layers), oracles
+
+
+def _oracle_step(oracles, x, x_pred, thr, act, has_gate, dtype):
+    masks = []
+    for l, (oc, w) in enumerate(oracles):
+        s = oracle.predictor_scores(x_pred[l], w["A"], w["Bm"])
+        m = oracle.mask_threshold(s, thr[l], True)
+        masks.append((m, s))
+        oc.update_active_weights(m)
+        y, _ = oracle.mlp_forward(x, oc.get_concat_weight(), oc.get_active_down_weight(), act, has_gate)
+        x = round_to(y, dtype)            # the GPU path stores each layer's output in the storage type
+    return x, masks
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16"])
+@pytest.mark.parametrize("has_gate", [True, False])
+def test_predictor_driven_decode_steps(dtype, has_gate):
+    L, H, I, B = 3, 256, 640, 2
+    act = "silu" if has_gate else "relu"
+    stack, oracles = _build(dtype, L, H, I, 16, B, has_gate, act)
+    rng = np.random.default_rng(1)
+    tdt = getattr(torch, dtype)
+    for step in range(6):
+        x = round_to(rng.standard_normal((B, H)).astype(np.float32), dtype)
+        x_pred = round_to(rng.standard_normal((L, B, H)).astype(np.float32), dtype)
+        # per-layer thresholds in a wide score gap so that the masks are unambiguous
+        thr = []
+        for l, (oc, w) in enumerate(oracles):
+            s = oracle.predictor_scores(x_pred[l], w["A"], w["Bm"])
+            thr.append(syn.threshold_for_fraction(s.max(0), 0.4))
+            stack.layers[l].thr = thr[l]
+        want, masks = _oracle_step(oracles, x, x_pred, thr, act, has_gate, dtype)
+        got = stack.decode_step(torch.from_numpy(x).to(DEV, tdt), [torch.from_numpy(x_pred[l]).to(DEV, tdt)
+                                                                    for l in range(L)])
+        for l, (oc, _) in enumerate(oracles):
+            m, s = masks[l]
+            near = (np.abs(s - thr[l]) < 1e-5 * np.abs(s).max()).any(0)
+            assert not near.any(), "threshold inside the guard band"
+            assert np.array_equal(stack.layers[l].mask.cpu().numpy(), m), (step, l)
+            assert stack.layers[l].cache.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist()
+        assert_close(got.float().cpu().numpy(), want, dtype, f"step {step}")
+
+
+@pytest.mark.parametrize("overlap", [False, True])
+def test_graph_replay_equals_eager(overlap):
+    """Replays of the captured step (with eager work and synchronisations in between) reproduce the
+    eager results and index lists exactly."""
+    L, H, I, B = 4, 512, 1024, 1
+    stack_g, _ = _build("float16", L, H, I, 32, B, seed=5)
+    stack_e, _ = _build("float16", L, H, I, 32, B, seed=5)
+    trace = torch.from_numpy(syn.mask_trace(3, L, I, 400, 12, 0.05, 0.2)).to(DEV)
+    gen = torch.Generator(device=DEV).manual_seed(0)
+    xs = torch.randn(12, B, H, device=DEV, generator=gen).half()
+    xp = torch.randn(12, L, B, H, device=DEV, generator=gen).half()
+    for s in (stack_g, stack_e):
+        s.prepare(B, overlap=overlap)
+        s.step_staged(xs[0], xp[0], trace[0])
+    torch.cuda.synchronize()
+    stack_g.capture()
+    for t in range(1, 12):
+        a = stack_g.step_staged(xs[t], xp[t], trace[t], replay=True).clone()
+        b = stack_e.step_staged(xs[t], xp[t], trace[t], replay=False).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), t
+        for lg, le in zip(stack_g.layers, stack_e.layers):
+            assert torch.equal(lg.mask, le.mask)
+            assert torch.equal(lg.cache.get_active_indices(), le.cache.get_active_indices())
+            assert lg.cache.get_num_active() == 400
+        _ = (xs[t].float() @ xs[t].float().t()).sum().item()   # unrelated eager work + a host sync between replays
+
+
+def test_skip_mlp_module_surface():
+    """SkipMLP mirrors the reference module: buffers, initialize_weight_cache, sparse forward."""
+    H, I = 128, 320
+    g = torch.Generator().manual_seed(0)
+    gate, up, down = (torch.randn(I, H, generator=g) * 0.05), (torch.randn(I, H, generator=g) * 0.05), \
+        (torch.randn(H, I, generator=g) * 0.05)
+    mlp = st.SkipMLP(gate.to(DEV), up.to(DEV), down.to(DEV), sparsity=0.5, act_fn="silu")
+    assert tuple(mlp.down_proj_buffer.shape) == (1, H) and tuple(mlp.combined_proj_buffer.shape) == (1, 2 * 160)
+    with pytest.raises(RuntimeError):
+        mlp(torch.randn(1, 1, H, device=DEV))
+    mlp.initialize_weight_cache()
+    m = torch.rand(I, generator=g) < 0.5
+    mlp.weight_cache.update_active_weights(m.to(DEV))
+    x = torch.randn(2, 1, H, generator=g)
+    out = mlp(x.to(DEV))
+    idx = torch.nonzero(m).flatten()
+    oc = oracle.OracleWeightCache(np.ones(I, bool), H, gate.numpy(), up.numpy(), down.numpy(), True)
+    oc.update_active_weights(m.numpy())
+    want, _ = oracle.mlp_forward(x.numpy(), oc.get_concat_weight(), oc.get_active_down_weight(), "silu", True)
+    assert_close(out.cpu().numpy(), want, "float32", "SkipMLP")
+    assert sorted(mlp.weight_cache.get_active_indices().cpu().tolist()) == idx.tolist()

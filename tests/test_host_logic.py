@@ -1,0 +1,69 @@
+"""Host-side behaviour that needs no GPU: loud failure without the HIP path, synthetic generators."""
+import numpy as np
+import pytest
+import torch
+
+import sparse_transformers_amd as st
+from sparse_transformers_amd import _lib, synthetic as syn
+
+
+def test_cpu_tensors_are_refused():
+    H, n = 16, 4
+    x = torch.randn(1, H)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        st.sparse_mlp_forward(x, torch.randn(2 * n, H), torch.randn(n, H).t(), torch.zeros(1, H), torch.zeros(1, 2),
+                              "silu")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        st.WeightCache(torch.ones(8, dtype=torch.bool), H, torch.randn(8, H), torch.randn(8, H), torch.randn(H, 8))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        st.predictor_mask(x, torch.randn(4, H), torch.randn(8, 4))
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libsparse_mlp_amd.so")
+    with pytest.raises(_lib.NativeLibraryMissing, match="no CPU fallback"):
+        _lib.lib()
+
+
+def test_product_never_imports_the_oracle():
+    import os
+    root = os.path.dirname(os.path.abspath(st.__file__))
+    for dirpath, _, files in os.walk(root):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text and "liboracle" not in text, f
+
+
+def test_mask_trace_properties():
+    tr = syn.mask_trace(1, 3, 512, 180, 40, 0.05, 0.15)
+    assert tr.shape == (40, 3, 512) and tr.dtype == bool
+    assert (tr.sum(-1) == 180).all()
+    changed = (tr[1:] & ~tr[:-1]).sum(-1) / 180.0
+    assert changed.min() >= 0.04 and changed.max() <= 0.16
+    assert np.array_equal(tr, syn.mask_trace(1, 3, 512, 180, 40, 0.05, 0.15))  # seeded
+
+
+def test_overlapping_token_masks():
+    m = syn.overlapping_token_masks(2, 8192, 8, 2457, 0.6)
+    assert (m.sum(1) == 2457).all()
+    core = m.all(0).sum()
+    assert core >= round(0.6 * 2457)
+    assert 5500 < m.any(0).sum() < 7000   # union over 8 tokens, about 6300 expected
+
+
+def test_threshold_guard_band():
+    rng = np.random.default_rng(0)
+    s = rng.standard_normal(8192)
+    thr = syn.threshold_for_fraction(s, 0.35, guard=1e-7)
+    frac = (s >= thr).mean()
+    assert abs(frac - 0.35) < 0.002
+    assert np.min(np.abs(s - thr)) >= 1e-7
+
+
+def test_workloads_match_reference_shapes():
+    w = syn.WORKLOADS["llama3b_stack_fp16"]
+    assert (w.layers, w.hidden, w.intermediate, w.rank, w.n_active) == (28, 3072, 8192, 128, 2867)
+    assert syn.WORKLOADS["mistral7b_stack_bf16"].n_active == 3584
+    assert syn.WORKLOADS["relullama7b_stack_fp16"].rank == int(0.04 * 11008)
