@@ -70,10 +70,13 @@ const char *st_last_error(void);
  *                      act(gate)*up in columns [0,n) and, when gated, the raw
  *                      up projection in [n,2n) — what the in-place operator
  *                      leaves in combined_proj_buffer
- *   workspace          float scratch of st_mlp_workspace_bytes(B,H) bytes
+ *   workspace          scratch of st_mlp_workspace_bytes(B,H,n) bytes
  * All rows must be 16-byte aligned (H*sizeof(dtype) % 16 == 0). B <= 4096.
+ * B < 32 runs the streaming decode kernel (HBM-bound); B >= 32 in fp16 / bf16
+ * with H % 32 == 0 runs the MFMA kernels (then only columns [0,n) of
+ * `combined` are written).
  * ------------------------------------------------------------------------ */
-int64_t st_mlp_workspace_bytes(int64_t B, int64_t H);
+int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n);
 int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
                    const void *down_rows, int64_t n, const int32_t *n_dev, int64_t n_hint, void *out, void *combined,
                    int64_t ldc, void *workspace, int64_t workspace_bytes, int act, int dtype, int has_gate,

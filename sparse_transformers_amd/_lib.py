@@ -37,7 +37,7 @@ _vp, _i64, _ci, _f = C.c_void_p, C.c_int64, C.c_int, C.c_float
 SIGNATURES = {
     "st_version": (_ci, []),
     "st_last_error": (C.c_char_p, []),
-    "st_mlp_workspace_bytes": (_i64, [_i64, _i64]),
+    "st_mlp_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "st_mlp_forward": (_ci, [_vp, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _ci, _ci, _ci,
                              _vp]),
     "st_predictor_mask": (_ci, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _ci, _f, _ci, _vp, _vp, _vp, _vp]),

@@ -386,13 +386,22 @@ template <typename T> static int launch_nb(const MlpLaunch &a)
 
 constexpr int kMlpMaxBatchPerLaunch = 4;
 
+// Blocks per launch: one per CU by default; ST_MLP_GMULT (1..4) multiplies it.
+int mlp_grid()
+{
+    static const int mult = [] { const int m = env_int("ST_MLP_GMULT"); return m >= 1 && m <= 4 ? m : 1; }();
+    return device_cu_count() * mult;
+}
+
 }  // namespace st
 
-extern "C" int64_t st_mlp_workspace_bytes(int64_t B, int64_t H)
+extern "C" int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n)
 {
-    (void)B;
-    const int64_t G = st::device_cu_count();
-    return G * st::kMlpMaxBatchPerLaunch * H * 4;
+    const int64_t G = st::mlp_grid();
+    const int64_t decode = G * st::kMlpMaxBatchPerLaunch * H * 4;
+    if (B < st::kPrefillMinRows) return decode;
+    const int64_t prefill = st::prefill_workspace_bytes(B, H, n);
+    return prefill > decode ? prefill : decode;
 }
 
 extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
@@ -409,13 +418,17 @@ extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *g
     ST_REQUIRE(dtype >= ST_F32 && dtype <= ST_BF16, "st_mlp_forward: unknown dtype %d", dtype);
     const int esz = dtype == ST_F32 ? 4 : 2;
     ST_REQUIRE(H >= 1 && (H * esz) % 16 == 0, "st_mlp_forward: H=%lld rows are not 16-byte multiples", (long long)H);
-    ST_REQUIRE(workspace_bytes >= st_mlp_workspace_bytes(B, H), "st_mlp_forward: workspace too small (%lld < %lld)",
-               (long long)workspace_bytes, (long long)st_mlp_workspace_bytes(B, H));
+    ST_REQUIRE(workspace_bytes >= st_mlp_workspace_bytes(B, H, n), "st_mlp_forward: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)st_mlp_workspace_bytes(B, H, n));
     ST_REQUIRE(!combined || ldc >= (has_gate ? 2 * n : n), "st_mlp_forward: ldc=%lld too small for n=%lld",
                (long long)ldc, (long long)n);
     const uintptr_t align = (uintptr_t)x | (uintptr_t)gate_rows | (uintptr_t)up_rows | (uintptr_t)down_rows |
                             (uintptr_t)workspace;
     ST_REQUIRE((align & 15) == 0, "st_mlp_forward: pointers must be 16-byte aligned");
+
+    if (B >= kPrefillMinRows && dtype != ST_F32 && H % 32 == 0)
+        return launch_prefill(dtype, x, (int)B, (int)H, gate_rows, up_rows, down_rows, (int)n, n_dev, out, combined,
+                              (long)ldc, workspace, act, has_gate ? 1 : 0, static_cast<hipStream_t>(stream));
 
     MlpLaunch a;
     a.x = x; a.B = (int)B; a.H = (int)H;
@@ -426,7 +439,7 @@ extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *g
     a.partials = static_cast<float *>(workspace);
     a.act = act; a.has_gate = has_gate ? 1 : 0;
     a.stream = static_cast<hipStream_t>(stream);
-    a.G = device_cu_count();
+    a.G = mlp_grid();
     switch (dtype) {
     case ST_F32: return launch_nb<float>(a);
     case ST_F16: return launch_nb<f16_t>(a);

@@ -145,6 +145,14 @@ int hip_fail(hipError_t e, const char *what);
 
 int device_cu_count();
 
+// Rows of x from which st_mlp_forward switches from the streaming decode
+// kernel to the MFMA kernels (fp16 / bf16 only).
+constexpr int kPrefillMinRows = 32;
+int64_t prefill_workspace_bytes(int64_t M, int64_t H, int64_t n);
+int launch_prefill(int dtype, const void *x, int M, int H, const void *gate, const void *up, const void *down, int n,
+                   const int *n_dev, void *out, void *comb, long ldc, void *workspace, int act, int has_gate,
+                   hipStream_t stream);
+
 // Event bracket around one kernel launch; a no-op unless profiling is enabled.
 struct ProfScope {
     int slot;

@@ -52,8 +52,8 @@ def current_stream_ptr(device: torch.device) -> int:
 _workspaces: dict = {}
 
 
-def mlp_workspace(device: torch.device, B: int, H: int) -> torch.Tensor:
-    need = int(_lib.lib().st_mlp_workspace_bytes(B, H))
+def mlp_workspace(device: torch.device, B: int, H: int, n: int) -> torch.Tensor:
+    need = int(_lib.lib().st_mlp_workspace_bytes(B, H, n))
     key = (device.index if device.index is not None else torch.cuda.current_device())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
@@ -70,7 +70,7 @@ def mlp_forward_rows(x2: torch.Tensor, gate_rows: Optional[torch.Tensor], up_row
     expects, used only to request rows before the device count has arrived."""
     dev = require_gpu(x2, gate_rows, up_rows, down_rows, out, combined, n_dev)
     B, H = x2.shape
-    ws = mlp_workspace(dev, B, H)
+    ws = mlp_workspace(dev, B, H, int(n))
     if act not in _lib.ACT_CODES:
         raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
     rc = _lib.lib().st_mlp_forward(

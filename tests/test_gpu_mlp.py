@@ -141,3 +141,29 @@ def test_argument_errors():
         out = st.sparse_mlp_forward(x.to(DEV), cw.to(DEV), dwc, db, cb, "silu")
     want, _ = oracle.mlp_forward(x.numpy(), cw.numpy(), dn.numpy().T, "silu", True)
     assert_close(out.cpu().numpy(), want, "float32", "repacked down")
+
+
+@pytest.mark.parametrize("name,M,H,n,dtype,act,has_gate", [
+    ("small ragged", 130, 256, 200, "float16", "silu", True),
+    ("one row tile, n below a K step", 32, 128, 20, "bfloat16", "relu", True),
+    ("ungated", 77, 512, 333, "float16", "relu", False),
+    ("cfg3 prefill shape, part of the active set", 512, 3072, 1000, "bfloat16", "silu", True),
+    ("wide hidden", 96, 4096, 600, "float16", "gelu_pytorch_tanh", True),
+])
+def test_prefill_mfma_vs_oracle(name, M, H, n, dtype, act, has_gate):
+    """B >= 32 rows in fp16 / bf16 run on the MFMA kernels; same tolerance as decode."""
+    x, cw, dn = _case(21, M, H, n, dtype, has_gate)
+    out, _, cb = _run(x, cw, dn, act, has_gate)
+    want, wantc = oracle.mlp_forward(x.float().numpy(), cw.float().numpy(), dn.float().numpy().T, act, has_gate)
+    assert_close(out.float().cpu().numpy(), want, dtype, name)
+    assert_close(cb.float().cpu().numpy()[:, :n], wantc[:, :n], dtype, name + " combined[:, :n]")
+
+
+def test_prefill_agrees_with_decode_kernel():
+    """The MFMA path (B = 40) and the streaming path (the same rows, 4 at a time) agree to rounding."""
+    x, cw, dn = _case(22, 40, 1024, 700, "float16", True)
+    big, _, _ = _run(x, cw, dn, "silu", True)
+    big = big.clone()
+    for b0 in range(0, 40, 8):
+        small, _, _ = _run(x[b0:b0 + 8], cw, dn, "silu", True)
+        assert_close(small.float().cpu().numpy(), big[b0:b0 + 8].float().cpu().numpy(), "float16", f"rows {b0}")
