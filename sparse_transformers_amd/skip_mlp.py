@@ -129,7 +129,7 @@ class SparseMLPStack:
         self.layers: List[SparseDecodeLayer] = list(layers)
 
     # ---- staged / graph-replayed stepping: fixed device buffers, no allocation, no host reads ----
-    def prepare(self, batch: int, overlap: bool = True) -> None:
+    def prepare(self, batch: int, overlap: bool = False) -> None:
         c0 = self.layers[0].cache
         dev, dt, H, I = c0.device, c0.dtype, c0.hidden_size, c0.intermediate_size
         L = len(self.layers)
