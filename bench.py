@@ -217,7 +217,7 @@ def main():
     alg_bytes = mats * n * H * esz                      # active-weight bytes one launch streams
     mlp_us = per_kernel["mlp_decode"]["mean_us"]
     achieved = alg_bytes / (mlp_us * 1e-6) / 1e9
-    upd_us = per_kernel["cache_plan"]["mean_us"] + per_kernel["cache_copy"]["mean_us"]
+    upd_us = per_kernel["cache_update"]["mean_us"]
 
     churn_mean = 0.5 * (wl.churn_lo + wl.churn_hi)
     result = {

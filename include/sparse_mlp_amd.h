@@ -115,10 +115,10 @@ typedef struct st_cache_buffers {
     void *gate_active; /* [I,H] (NULL when !has_gate) */
     void *up_active;   /* [I,H] */
     void *down_active; /* [I,H] */
-    int32_t *indices;  /* [I] ordered active list (the reference's active_indices) */
-    uint8_t *cur_mask; /* [I] the reference's current_mask */
+    /* bookkeeping, double-buffered: buffer e lives at offset e*I, the current e is state[ST_STATE_EPOCH] */
+    int32_t *indices;  /* [2*I] ordered active list (the reference's active_indices) */
+    uint8_t *cur_mask; /* [2*I] the reference's current_mask */
     int32_t *state;    /* [ST_STATE_WORDS] see st_state_word */
-    int32_t *scratch;  /* [2*I] work lists of one update */
 } st_cache_buffers;
 
 enum st_state_word {
@@ -129,7 +129,11 @@ enum st_state_word {
     ST_STATE_N_ADDED = 4,   /* |new & ~old| of the last update */
     ST_STATE_N_REMOVED = 5, /* |old & ~new| of the last update */
     ST_STATE_SERIAL = 6,    /* updates that changed something */
-    ST_STATE_WORDS = 8
+    ST_STATE_EPOCH = 7,     /* which half of indices / cur_mask is current */
+    ST_STATE_TICKET = 8,    /* internal: (epoch << 16) | blocks arrived in the running update */
+    ST_STATE_N_BUF0 = 9,    /* internal: active count of bookkeeping buffer 0 */
+    ST_STATE_N_BUF1 = 10,   /* internal: active count of bookkeeping buffer 1 */
+    ST_STATE_WORDS = 16
 };
 
 typedef struct st_cache st_cache;
@@ -148,7 +152,7 @@ int st_cache_load_weights(st_cache *c, const void *gate, const void *up, const v
 
 /* update_active_weights(mask): weight_cache.h:229-359 (diff :84-110, pairing
  * :248-277, append :280-307, swap-with-last :310-353).  mask: uint8/bool [I]
- * on the device.  Enqueues a plan kernel and a row-copy kernel; returns
+ * on the device.  Enqueues one kernel (bookkeeping + row copies); returns
  * without waiting.  An update that empties the cache sets
  * state[ST_STATE_STATUS] = ST_ERR_NO_ACTIVE and, like the reference, leaves
  * cur_mask unchanged. */
@@ -177,8 +181,8 @@ int st_cache_materialize_concat(st_cache *c, void *dst, int64_t n, void *stream)
 typedef enum st_kernel_kind {
     ST_K_MLP_DECODE = 0,
     ST_K_MLP_REDUCE = 1,
-    ST_K_CACHE_PLAN = 2,
-    ST_K_CACHE_COPY = 3,
+    ST_K_CACHE_UPDATE = 2,
+    ST_K_RESERVED = 3,
     ST_K_PRED_DOWN = 4,
     ST_K_PRED_UP_MASK = 5,
     ST_K_MLP_PREFILL_GATEUP = 6,

@@ -21,14 +21,14 @@ ST_F32, ST_F16, ST_BF16 = 0, 1, 2
 ACT_CODES = {"relu": 0, "silu": 1, "gelu_pytorch_tanh": 2, "sigmoid": 3, "identity": 4}
 
 STATE_N_ACTIVE, STATE_N_CHANGED, STATE_STATUS, STATE_VALID = 0, 1, 2, 3
-STATE_N_ADDED, STATE_N_REMOVED, STATE_SERIAL, STATE_WORDS = 4, 5, 6, 8
+STATE_N_ADDED, STATE_N_REMOVED, STATE_SERIAL, STATE_EPOCH, STATE_WORDS = 4, 5, 6, 7, 16
 
 
 class CacheBuffers(C.Structure):
     _fields_ = [
         ("gate_pool", C.c_void_p), ("up_pool", C.c_void_p), ("downT_pool", C.c_void_p),
         ("gate_active", C.c_void_p), ("up_active", C.c_void_p), ("down_active", C.c_void_p),
-        ("indices", C.c_void_p), ("cur_mask", C.c_void_p), ("state", C.c_void_p), ("scratch", C.c_void_p),
+        ("indices", C.c_void_p), ("cur_mask", C.c_void_p), ("state", C.c_void_p),
     ]
 
 
@@ -53,7 +53,7 @@ SIGNATURES = {
     "st_profile_collect": (_ci, [_vp, _vp, _ci]),
 }
 
-KERNEL_KINDS = ["mlp_decode", "mlp_reduce", "cache_plan", "cache_copy", "pred_down", "pred_up_mask",
+KERNEL_KINDS = ["mlp_decode", "mlp_reduce", "cache_update", "reserved", "pred_down", "pred_up_mask",
                 "mlp_prefill_gateup", "mlp_prefill_down"]
 
 _lib = None

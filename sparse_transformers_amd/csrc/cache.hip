@@ -1,22 +1,29 @@
 // Differential weight cache resident in HBM.
 //
-// update = one "plan" kernel (a single 1024-thread workgroup doing only
-// integer bookkeeping in LDS) + one "copy" kernel (16-byte row copies).
-//
-// The plan kernel replays WeightCache::update_active_weights
-// (sparse_transformers/csrc/weight_cache.h:229-359) exactly:
+// update = ONE kernel.  Every block (1024 threads) first replays the
+// bookkeeping of WeightCache::update_active_weights
+// (sparse_transformers/csrc/weight_cache.h:229-359) redundantly in its own LDS
+// (integer work only, identical in every block):
 //   diff      ascending added / removed lists     (weight_cache.h:84-110)
 //   phase 1   i-th removed position <- i-th added  (:248-277)   parallel
 //   phase 2   surplus additions appended           (:280-307)   parallel
 //   phase 3   surplus removals, swap-with-last     (:310-353)   one lane,
 //             because each step depends on the list the previous one left
-// It only decides WHICH index ends up at WHICH position.  Because every active
-// row is a bit-copy of a pool row, the data movement never has to follow the
-// sequential order: the copy kernel rewrites each position whose index
-// changed straight from the pool (no reads of the active buffers, hence no
-// hazards between copies).
+// and then copies its share of the changed rows with 16-byte loads/stores.
+// The plan only decides WHICH index ends up at WHICH position.  Because every
+// active row is a bit-copy of a pool row, the data movement never has to
+// follow the sequential order: each position whose index changed is rewritten
+// straight from the pool (no reads of the active buffers, hence no hazards
+// between copies).
+//
+// The bookkeeping (index list, remembered mask, count) is double-buffered:
+// blocks read buffer `epoch`, one block writes buffer `epoch ^ 1`, and the
+// block that arrives last (a ticket counter packed with the epoch in one word)
+// flips the epoch.  Nothing ever waits: a block that starts late still reads
+// the old buffer, because nobody writes it during this launch.
 #include "st_common.h"
 
+#include <cstdlib>
 #include <new>
 
 namespace st {
@@ -55,43 +62,116 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wave_t
     return prefix + incl - v;
 }
 
-__global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t *__restrict__ new_mask,
-                                                                  uint8_t *__restrict__ cur_mask,
-                                                                  int32_t *__restrict__ indices,
-                                                                  int32_t *__restrict__ state,
-                                                                  int32_t *__restrict__ scratch, int I)
+struct CopyPlan {
+    const unsigned char *pool[3];
+    unsigned char *active[3];
+    int nmat;
+    int row_bytes;
+};
+
+constexpr int kCopyUnroll = 4;  // rows a thread group keeps in flight
+
+constexpr int kPlanMaxWords = 3;  // 8-element words per thread in the vector path: I <= 24576
+
+__device__ __forceinline__ uint64_t nonzero_bytes(uint64_t x)
+{
+    x |= x >> 4; x |= x >> 2; x |= x >> 1;
+    return x & 0x0101010101010101ull;
+}
+
+// VEC: I % 8 == 0 and the mask is 8-byte aligned, so masks are read as 8-byte
+// words and indices as 16-byte vectors; both bookkeeping buffers are requested
+// together with the ticket, so the kernel front costs one memory round trip.
+template <bool VEC>
+__global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp, const uint8_t *__restrict__ new_mask,
+                                                                    uint8_t *__restrict__ cur_mask2,
+                                                                    int32_t *__restrict__ indices2,
+                                                                    int32_t *__restrict__ state, int I, int gs_log2)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);  // index -> position
     uint16_t *idx_l = pos_l + I;                           // position -> index
     // added indices ascending from the front, removed indices ascending from the
-    // back (k-th removed at lists[I-1-k]); the two never meet: na + nr <= I
+    // back (k-th removed at lists[I-1-k]); the two never meet: na + nr <= I.
+    // After the plan the same array holds the positions to rewrite.
     uint16_t *lists = idx_l + I;
     uint32_t *dirty = reinterpret_cast<uint32_t *>(lists + I + (I & 1));  // bit per position
     const int dirty_words = (I + 31) >> 5;
-    uint8_t *flag_l = reinterpret_cast<uint8_t *>(dirty + dirty_words);   // bit0 new, bit1 old
+    uint8_t *flag_l = reinterpret_cast<uint8_t *>(dirty + ((dirty_words + 1) & ~1));  // bit0 new, bit1 old; 8-byte aligned
     __shared__ uint32_t wave_tot[kPlanWaves];
     __shared__ int n_new_s;
-
-    int32_t *changed_g = scratch;      // [I] positions to rewrite
-    int32_t *source_g = scratch + I;   // [I] pool row for each of them
+    __shared__ uint32_t ticket_s;
 
     const int tid = threadIdx.x;
-    // Everything the plan needs from global memory is requested in one go:
-    // the count, both masks and the whole index list (entries >= n are ignored).
-    const int n = state[ST_STATE_N_ACTIVE];
-    for (int i = tid; i < I; i += kPlanThreads) {
-        pos_l[i] = kNone;
-        flag_l[i] = (new_mask[i] ? 1 : 0) | (cur_mask[i] ? 2 : 0);
-        idx_l[i] = (uint16_t)indices[i];
+    ST_TL(0);
+    // Elements per thread (a contiguous range, so the diff lists come out ascending).
+    const int E = VEC ? ((I + 8 * kPlanThreads - 1) / (8 * kPlanThreads)) * 8 : (I + kPlanThreads - 1) / kPlanThreads;
+    const int e0 = tid * E < I ? tid * E : I, e1 = e0 + E < I ? e0 + E : I;
+
+    uint64_t v_new[kPlanMaxWords], v_cur[2][kPlanMaxWords];
+    int4 v_idx[2][kPlanMaxWords][2];
+    int n_both[2];
+    if constexpr (VEC) {
+#pragma unroll
+        for (int w = 0; w < kPlanMaxWords; ++w) {
+            const int e = e0 + 8 * w;
+            if (e < e1) {
+                v_new[w] = *reinterpret_cast<const uint64_t *>(new_mask + e);
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    v_cur[b][w] = *reinterpret_cast<const uint64_t *>(cur_mask2 + (size_t)b * I + e);
+                    v_idx[b][w][0] = *reinterpret_cast<const int4 *>(indices2 + (size_t)b * I + e);
+                    v_idx[b][w][1] = *reinterpret_cast<const int4 *>(indices2 + (size_t)b * I + e + 4);
+                }
+            }
+        }
+        n_both[0] = state[ST_STATE_N_BUF0];
+        n_both[1] = state[ST_STATE_N_BUF1];
     }
+    // One atomic returns both the epoch (which buffer to read) and this block's ticket.
+    if (tid == 0) ticket_s = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
     for (int w = tid; w < dirty_words; w += kPlanThreads) dirty[w] = 0u;
     __syncthreads();
+    const uint32_t ticket = ticket_s;
+    const int ep = (int)((ticket >> 16) & 1u);
+    const bool last_arrival = (ticket & 0xffffu) == gridDim.x - 1;
+    const bool writer = blockIdx.x == 0;
+
+    int n;
+    if constexpr (VEC) {
+        n = ep ? n_both[1] : n_both[0];
+#pragma unroll
+        for (int w = 0; w < kPlanMaxWords; ++w) {
+            const int e = e0 + 8 * w;
+            if (e < e1) {
+                const uint64_t nw = nonzero_bytes(v_new[w]), cw = nonzero_bytes(ep ? v_cur[1][w] : v_cur[0][w]);
+                *reinterpret_cast<uint64_t *>(flag_l + e) = nw | (cw << 1);
+                const int4 a = ep ? v_idx[1][w][0] : v_idx[0][w][0], b4 = ep ? v_idx[1][w][1] : v_idx[0][w][1];
+                uint4 packed;
+                packed.x = (uint32_t)(a.x & 0xffff) | ((uint32_t)a.y << 16);
+                packed.y = (uint32_t)(a.z & 0xffff) | ((uint32_t)a.w << 16);
+                packed.z = (uint32_t)(b4.x & 0xffff) | ((uint32_t)b4.y << 16);
+                packed.w = (uint32_t)(b4.z & 0xffff) | ((uint32_t)b4.w << 16);
+                *reinterpret_cast<uint4 *>(idx_l + e) = packed;
+                *reinterpret_cast<uint4 *>(pos_l + e) = make_uint4(0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu);
+            }
+        }
+    } else {
+        const uint8_t *cur_mask = cur_mask2 + (size_t)ep * I;
+        const int32_t *indices = indices2 + (size_t)ep * I;
+        n = state[ST_STATE_N_BUF0 + ep];
+        for (int i = tid; i < I; i += kPlanThreads) {
+            pos_l[i] = kNone;
+            flag_l[i] = (new_mask[i] ? 1 : 0) | (cur_mask[i] ? 2 : 0);
+            idx_l[i] = (uint16_t)indices[i];
+        }
+    }
+    ST_TL(1);
+    __syncthreads();
+    ST_TL(2);
     for (int p = tid; p < n; p += kPlanThreads) pos_l[idx_l[p]] = (uint16_t)p;
 
     // ---- diff: contiguous element range per thread keeps the lists ascending
-    const int E = (I + kPlanThreads - 1) / kPlanThreads;
-    const int e0 = tid * E < I ? tid * E : I, e1 = e0 + E < I ? e0 + E : I;
     uint32_t cnt = 0;  // added in the low half, removed in the high half
     for (int i = e0; i < e1; ++i) {
         const uint8_t f = flag_l[i];
@@ -100,12 +180,16 @@ __global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t 
     }
     uint32_t total;
     const uint32_t off = block_excl_scan(cnt, wave_tot, &total);  // contains __syncthreads
+    ST_TL(3);
     const int na = (int)(total & 0xffffu), nr = (int)(total >> 16);
     if (na == 0 && nr == 0) {  // unchanged mask: nothing is touched (weight_cache.h:237-240)
         if (tid == 0) {
-            state[ST_STATE_N_CHANGED] = 0;
-            state[ST_STATE_N_ADDED] = 0;
-            state[ST_STATE_N_REMOVED] = 0;
+            if (last_arrival) atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)ep << 16);
+            if (writer) {
+                state[ST_STATE_N_CHANGED] = 0;
+                state[ST_STATE_N_ADDED] = 0;
+                state[ST_STATE_N_REMOVED] = 0;
+            }
         }
         return;
     }
@@ -120,6 +204,9 @@ __global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t 
     __syncthreads();
 
     const int pairs = na < nr ? na : nr;
+    // Without surplus removals (nr <= na) the rewritten positions are known as soon as phases 1 and 2
+    // have run: they replace the added indices in `lists` in place and no compaction is needed.
+    const bool fast = nr <= na;
     // ---- phase 1: paired replacement
     for (int i = tid; i < pairs; i += kPlanThreads) {
         const int e = lists[I - 1 - i];
@@ -129,8 +216,9 @@ __global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t 
             idx_l[p] = (uint16_t)a;
             pos_l[a] = p;
             pos_l[e] = kNone;
-            atomicOr(&dirty[p >> 5], 1u << (p & 31));
+            if (!fast) atomicOr(&dirty[p >> 5], 1u << (p & 31));
         }
+        if (fast) lists[i] = p;
     }
     // ---- phase 2: append surplus additions
     for (int i = pairs + tid; i < na; i += kPlanThreads) {
@@ -139,121 +227,121 @@ __global__ __launch_bounds__(kPlanThreads) void cache_plan_kernel(const uint8_t 
             const int a = lists[i];
             idx_l[p] = (uint16_t)a;
             pos_l[a] = (uint16_t)p;
-            atomicOr(&dirty[p >> 5], 1u << (p & 31));
         }
+        lists[i] = p < I ? (uint16_t)p : kNone;
     }
     __syncthreads();
 
-    // ---- phase 3: surplus removals, sequential by construction
-    if (tid == 0) {
-        int m = n + (na - pairs);
-        if (m > I) m = I;
-        for (int k = pairs; k < nr; ++k) {
-            const int e = lists[I - 1 - k];
-            const uint16_t p = pos_l[e];
-            if (p == kNone) continue;
-            if (m <= 0) break;
-            const int last = m - 1;
-            if ((int)p != last) {
-                const uint16_t li = idx_l[last];
-                idx_l[p] = li;
-                pos_l[li] = p;
-                dirty[p >> 5] |= 1u << (p & 31);
-            }
-            --m;
-            pos_l[e] = kNone;
-        }
-        n_new_s = m;
-    }
-    __syncthreads();
-    const int n_new = n_new_s;
-
-    // ---- compact the dirty positions below n_new into the copy list
-    uint32_t word = 0;
-    if (tid < dirty_words) {
-        word = dirty[tid];
-        const int lo = tid << 5;
-        if (lo >= n_new) word = 0;
-        else if (lo + 32 > n_new) word &= (1u << (n_new - lo)) - 1u;
-    }
+    int n_new;
     uint32_t n_changed;
-    uint32_t coff = block_excl_scan((uint32_t)__popc(word), wave_tot, &n_changed);
-    while (word) {
-        const int bit = __ffs(word) - 1;
-        word &= word - 1;
-        const int p = (tid << 5) + bit;
-        const int idx = idx_l[p];
-        changed_g[coff] = p;
-        source_g[coff] = idx;
-        ++coff;
-        indices[p] = idx;
-    }
-
-    if (n_new > 0) {  // the reference stores the mask only when the rebuild did not throw
-        for (int i = tid; i < I; i += kPlanThreads) cur_mask[i] = flag_l[i] & 1;
-    }
-    if (tid == 0) {
-        state[ST_STATE_N_ACTIVE] = n_new;
-        state[ST_STATE_N_CHANGED] = (int)n_changed;
-        state[ST_STATE_N_ADDED] = na;
-        state[ST_STATE_N_REMOVED] = nr;
-        state[ST_STATE_SERIAL] += 1;
-        if (n_new > 0) {
-            state[ST_STATE_STATUS] = 0;
-            state[ST_STATE_VALID] = 1;
-        } else {
-            state[ST_STATE_STATUS] = ST_ERR_NO_ACTIVE;
-        }
-    }
-}
-
-struct CopyPlan {
-    const unsigned char *pool[3];
-    unsigned char *active[3];
-    int nmat;
-    int row_bytes;
-};
-
-constexpr int kCopyThreads = 256;
-constexpr int kCopyUnroll = 4;  // 16-byte chunks per thread issued together
-
-// One block per (changed position, matrix): active[m][p] <- pool[m][source].
-// The work item is read speculatively together with the count, so a block
-// needs two memory round trips: (count, position, source), then the row.
-__global__ __launch_bounds__(kCopyThreads) void cache_copy_kernel(CopyPlan cp, const int32_t *__restrict__ state,
-                                                                  const int32_t *__restrict__ changed,
-                                                                  const int32_t *__restrict__ source, int I)
-{
-    const int nmat = cp.nmat;
-    const int cap = I * nmat;
-    int w = blockIdx.x;
-    if (w >= cap) return;
-    // the lists have I entries, so reading entry w / nmat is safe before the count is known
-    int p = changed[w / nmat];
-    int idx = source[w / nmat];
-    const int work = state[ST_STATE_N_CHANGED] * nmat;
-    for (; w < work; w += gridDim.x) {
-        const int j = w / nmat, m = w - j * nmat;
-        if (w != (int)blockIdx.x) {
-            p = changed[j];
-            idx = source[j];
-        }
-        const unsigned char *src = cp.pool[m] + (size_t)idx * cp.row_bytes;
-        unsigned char *dst = cp.active[m] + (size_t)p * cp.row_bytes;
-        for (int o0 = 0; o0 < cp.row_bytes; o0 += kCopyThreads * kCopyUnroll * 16) {
-            uint4 v[kCopyUnroll];
-#pragma unroll
-            for (int u = 0; u < kCopyUnroll; ++u) {
-                const int o = o0 + (u * kCopyThreads + (int)threadIdx.x) * 16;
-                if (o < cp.row_bytes) v[u] = ld16(src + o);
+    if (fast) {
+        n_new = n + (na - pairs);
+        if (n_new > I) n_new = I;
+        n_changed = (uint32_t)na;
+        ST_TL(4);
+    } else {
+        // ---- phase 3: surplus removals, sequential by construction
+        if (tid == 0) {
+            int m = n;
+            for (int k = pairs; k < nr; ++k) {
+                const int e = lists[I - 1 - k];
+                const uint16_t p = pos_l[e];
+                if (p == kNone) continue;
+                if (m <= 0) break;
+                const int last = m - 1;
+                if ((int)p != last) {
+                    const uint16_t li = idx_l[last];
+                    idx_l[p] = li;
+                    pos_l[li] = p;
+                    dirty[p >> 5] |= 1u << (p & 31);
+                }
+                --m;
+                pos_l[e] = kNone;
             }
+            n_new_s = m;
+        }
+        __syncthreads();
+        ST_TL(4);
+        n_new = n_new_s;
+
+        // ---- compact the dirty positions below n_new into the copy list (in LDS, over the dead lists)
+        uint32_t word = 0;
+        if (tid < dirty_words) {
+            word = dirty[tid];
+            const int lo = tid << 5;
+            if (lo >= n_new) word = 0;
+            else if (lo + 32 > n_new) word &= (1u << (n_new - lo)) - 1u;
+        }
+        uint32_t coff = block_excl_scan((uint32_t)__popc(word), wave_tot, &n_changed);  // barrier: lists are dead now
+        while (word) {
+            const int bit = __ffs(word) - 1;
+            word &= word - 1;
+            lists[coff++] = (uint16_t)((tid << 5) + bit);
+        }
+        __syncthreads();
+    }
+
+    ST_TL(5);
+    // ---- copy this block's share of the changed rows: active[m][p] <- pool[m][index at p]
+    {
+        const int nmat = cp.nmat, row_bytes = cp.row_bytes, chunks = row_bytes >> 4;
+        const int GS = 1 << gs_log2, ngrp = kPlanThreads >> gs_log2;
+        const int grp = tid >> gs_log2, cc = tid & (GS - 1);
+        const int slots = gridDim.x * ngrp, slot = blockIdx.x * ngrp + grp;
+        const int work = (int)n_changed * nmat;
+        for (int w0 = slot; w0 < work; w0 += slots * kCopyUnroll) {
+            for (int c = cc; c < chunks; c += GS) {
+                uint4 v[kCopyUnroll];
+                unsigned char *dst[kCopyUnroll];
 #pragma unroll
-            for (int u = 0; u < kCopyUnroll; ++u) {
-                const int o = o0 + (u * kCopyThreads + (int)threadIdx.x) * 16;
-                if (o < cp.row_bytes) st16(dst + o, v[u]);
+                for (int u = 0; u < kCopyUnroll; ++u) {
+                    const int w = w0 + u * slots;
+                    dst[u] = nullptr;
+                    if (w < work) {
+                        const int j = w / nmat, m = w - j * nmat;
+                        const int p = lists[j];
+                        if (p == kNone) continue;  // a removed index that was not in the cache: nothing to copy
+                        const int idx = idx_l[p];
+                        const unsigned char *pool = m == 0 ? cp.pool[0] : (m == 1 ? cp.pool[1] : cp.pool[2]);
+                        unsigned char *act = m == 0 ? cp.active[0] : (m == 1 ? cp.active[1] : cp.active[2]);
+                        v[u] = ld16(pool + (size_t)idx * row_bytes + ((size_t)c << 4));
+                        dst[u] = act + (size_t)p * row_bytes + ((size_t)c << 4);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kCopyUnroll; ++u)
+                    if (dst[u]) st16(dst[u], v[u]);
             }
         }
     }
+
+    ST_TL(6);
+    // ---- publish: one block writes the other bookkeeping buffer, the last arrival flips the epoch
+    if (writer) {
+        int32_t *idx_out = indices2 + (size_t)(ep ^ 1) * I;
+        uint8_t *mask_out = cur_mask2 + (size_t)(ep ^ 1) * I;
+        for (int p = tid; p < n_new; p += kPlanThreads) idx_out[p] = idx_l[p];
+        // the reference stores the new mask only when the rebuild did not throw (n_new > 0)
+        for (int i = tid; i < I; i += kPlanThreads) mask_out[i] = n_new > 0 ? (flag_l[i] & 1) : (flag_l[i] >> 1);
+        if (tid == 0) {
+            state[ST_STATE_N_BUF0 + (ep ^ 1)] = n_new;
+            state[ST_STATE_N_ACTIVE] = n_new;
+            state[ST_STATE_N_CHANGED] = (int)n_changed;
+            state[ST_STATE_N_ADDED] = na;
+            state[ST_STATE_N_REMOVED] = nr;
+            state[ST_STATE_SERIAL] += 1;
+            state[ST_STATE_EPOCH] = ep ^ 1;
+            if (n_new > 0) {
+                state[ST_STATE_STATUS] = 0;
+                state[ST_STATE_VALID] = 1;
+            } else {
+                state[ST_STATE_STATUS] = ST_ERR_NO_ACTIVE;
+            }
+        }
+    }
+    if (last_arrival && tid == 0)
+        atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)(ep ^ 1) << 16);
+    ST_TL(7);
 }
 
 // in [R,C] -> out [C,R], 64x64 tiles through LDS.
@@ -274,12 +362,12 @@ __global__ __launch_bounds__(256) void transpose_kernel(const E *__restrict__ in
     }
 }
 
-__global__ void cache_reset_kernel(uint8_t *cur_mask, int32_t *indices, int32_t *state, int I)
+__global__ void cache_reset_kernel(uint8_t *cur_mask2, int32_t *indices2, int32_t *state, int I)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < I) {
-        cur_mask[i] = 0;
-        indices[i] = -1;
+    if (i < 2 * I) {
+        cur_mask2[i] = 0;
+        indices2[i] = -1;
     }
     if (i < ST_STATE_WORDS) state[i] = 0;
 }
@@ -306,7 +394,7 @@ extern "C" st_cache *st_cache_create(const st_cache_buffers *bufs, int64_t I, in
     if (I < 1 || I > kPlanMaxI) return fail("intermediate size out of range (see st_cache_max_intermediate)");
     if (H < 1 || (H * esz) % 16 != 0) return fail("rows are not 16-byte multiples");
     if (!bufs->up_pool || !bufs->downT_pool || !bufs->up_active || !bufs->down_active || !bufs->indices ||
-        !bufs->cur_mask || !bufs->state || !bufs->scratch)
+        !bufs->cur_mask || !bufs->state)
         return fail("null device buffer");
     if (has_gate && (!bufs->gate_pool || !bufs->gate_active)) return fail("has_gate set but gate buffers are null");
     const uintptr_t align = (uintptr_t)bufs->gate_pool | (uintptr_t)bufs->up_pool | (uintptr_t)bufs->downT_pool |
@@ -349,7 +437,7 @@ extern "C" int st_cache_load_weights(st_cache *c, const void *gate, const void *
         hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, s, static_cast<const uint16_t *>(down),
                            static_cast<uint16_t *>(c->b.downT_pool), (int)c->H, (int)c->I);
     ST_HIP(hipGetLastError());
-    hipLaunchKernelGGL(cache_reset_kernel, dim3((unsigned)((c->I + 255) / 256)), dim3(256), 0, s, c->b.cur_mask,
+    hipLaunchKernelGGL(cache_reset_kernel, dim3((unsigned)((2 * c->I + 255) / 256)), dim3(256), 0, s, c->b.cur_mask,
                        c->b.indices, c->b.state, (int)c->I);
     ST_HIP(hipGetLastError());
     return ST_OK;
@@ -361,19 +449,15 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     ST_REQUIRE(c && mask, "st_cache_update_async: null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int I = (int)c->I;
-    const size_t lds = (size_t)I * 6 + (I & 1) * 2 + (size_t)((I + 31) >> 5) * 4 + (size_t)I + 16;
+    const size_t lds = (size_t)I * 6 + (I & 1) * 2 + (size_t)((((I + 31) >> 5) + 1) & ~1) * 4 + (size_t)I + 16;
     static bool attr_set = false;
     if (!attr_set) {
-        ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(cache_plan_kernel),
+        ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(cache_update_kernel<true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+        ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(cache_update_kernel<false>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
         attr_set = true;
     }
-    {
-        ProfScope ps(ST_K_CACHE_PLAN, s);
-        hipLaunchKernelGGL(cache_plan_kernel, dim3(1), dim3(kPlanThreads), lds, s, mask, c->b.cur_mask, c->b.indices,
-                           c->b.state, c->b.scratch, I);
-    }
-    ST_HIP(hipGetLastError());
     CopyPlan cp;
     cp.nmat = 0;
     if (c->has_gate) {
@@ -384,13 +468,27 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.up_active);
     cp.pool[cp.nmat] = static_cast<const unsigned char *>(c->b.downT_pool);
     cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.down_active);
-    for (int k = cp.nmat; k < 3; ++k) { cp.pool[k] = nullptr; cp.active[k] = nullptr; }
+    for (int k = cp.nmat; k < 3; ++k) { cp.pool[k] = cp.pool[0]; cp.active[k] = cp.active[0]; }
     cp.row_bytes = (int)(c->H * c->esz);
-    const int grid = 8 * device_cu_count();
+    const int chunks = cp.row_bytes >> 4;
+    int gs_log2 = 6;
+    while ((1 << gs_log2) < chunks && (1 << gs_log2) < kPlanThreads) ++gs_log2;
+    static const int blocks = [] {
+        const char *v = getenv("ST_CACHE_BLOCKS");
+        const int b = v ? atoi(v) : 0;
+        return b >= 1 && b <= 1024 ? b : 0;
+    }();
+    const int grid = blocks ? blocks : device_cu_count() / 2;
     {
-        ProfScope ps(ST_K_CACHE_COPY, s);
-        hipLaunchKernelGGL(cache_copy_kernel, dim3(grid), dim3(kCopyThreads), 0, s, cp, c->b.state, c->b.scratch,
-                           c->b.scratch + c->I, (int)c->I);
+        ProfScope ps(ST_K_CACHE_UPDATE, s);
+        const bool vec = (I % 8 == 0) && ((uintptr_t)mask % 8 == 0) && ((uintptr_t)c->b.cur_mask % 8 == 0) &&
+                         ((uintptr_t)c->b.indices % 16 == 0) && I <= 8 * kPlanThreads * kPlanMaxWords;
+        if (vec)
+            hipLaunchKernelGGL(cache_update_kernel<true>, dim3(grid), dim3(kPlanThreads), lds, s, cp, mask,
+                               c->b.cur_mask, c->b.indices, c->b.state, I, gs_log2);
+        else
+            hipLaunchKernelGGL(cache_update_kernel<false>, dim3(grid), dim3(kPlanThreads), lds, s, cp, mask,
+                               c->b.cur_mask, c->b.indices, c->b.state, I, gs_log2);
     }
     ST_HIP(hipGetLastError());
     return ST_OK;

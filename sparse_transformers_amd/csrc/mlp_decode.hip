@@ -20,13 +20,6 @@
 
 #include <cstdlib>
 
-// Timeline hook: a build that defines ST_TL(i) before including this file can
-// record a timestamp at stage i of the decode kernel; the library build leaves
-// it empty.
-#ifndef ST_TL
-#define ST_TL(i)
-#endif
-
 namespace st {
 
 // T: storage type; NB: x rows per launch; RB: rows per group kept in flight;
@@ -82,9 +75,9 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
         for (int q = 0; q < CPT; ++q) {
             const bool ok = valid[q] && row < n_spec;
             const size_t o = (size_t)row * H + coff[q];
-            wg[k][q] = (ok && has_gate) ? ld16(gate + o) : zero4;
-            wu[k][q] = ok ? ld16(up + o) : zero4;
-            wd[k][q] = ok ? ld16(down + o) : zero4;
+            wg[k][q] = (ok && has_gate) ? ld16_stream(gate + o) : zero4;
+            wu[k][q] = ok ? ld16_stream(up + o) : zero4;
+            wd[k][q] = ok ? ld16_stream(down + o) : zero4;
         }
     }
 
@@ -113,9 +106,9 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
                 const bool ok = valid[q] && row < n;
                 const size_t o = (size_t)row * H + coff[q];
                 if (!have) {
-                    wg[k][q] = (ok && has_gate) ? ld16(gate + o) : zero4;
-                    wu[k][q] = ok ? ld16(up + o) : zero4;
-                    wd[k][q] = ok ? ld16(down + o) : zero4;
+                    wg[k][q] = (ok && has_gate) ? ld16_stream(gate + o) : zero4;
+                    wu[k][q] = ok ? ld16_stream(up + o) : zero4;
+                    wd[k][q] = ok ? ld16_stream(down + o) : zero4;
                 } else if (!ok) {
                     wg[k][q] = zero4; wu[k][q] = zero4; wd[k][q] = zero4;
                 }

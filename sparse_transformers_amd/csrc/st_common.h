@@ -7,6 +7,13 @@
 
 #include "../../include/sparse_mlp_amd.h"
 
+// Timeline hook: a build that defines ST_TL(i) before including the kernel
+// sources can record a timestamp at stage i of a kernel; the library build
+// leaves it empty.
+#ifndef ST_TL
+#define ST_TL(i)
+#endif
+
 namespace st {
 
 constexpr int kWave = 64;
@@ -74,6 +81,17 @@ template <> __device__ __forceinline__ float to_float<f16_t>(f16_t v) { return (
 template <> __device__ __forceinline__ float to_float<bf16_t>(bf16_t v) { return __uint_as_float((uint32_t)v.bits << 16); }
 
 __device__ __forceinline__ uint4 ld16(const void *p) { return *reinterpret_cast<const uint4 *>(p); }
+// Streaming variant for data that is read once per launch (weight rows): non-temporal hint.
+__device__ __forceinline__ uint4 ld16_stream(const void *p)
+{
+#ifdef ST_NO_NT_LOADS
+    return *reinterpret_cast<const uint4 *>(p);
+#else
+    typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+#endif
+}
 __device__ __forceinline__ void st16(void *p, const uint4 &v) { *reinterpret_cast<uint4 *>(p) = v; }
 
 // Sum over the 64 lanes of a wave; every lane receives the total.

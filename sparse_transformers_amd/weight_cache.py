@@ -57,17 +57,16 @@ class WeightCache:
         self.gate_active = wbuf() if self.has_gate else None
         self.up_active = wbuf()
         self.down_active = wbuf()
-        self.indices = torch.empty(I, dtype=torch.int32, device=dev)
-        self.cur_mask = torch.empty(I, dtype=torch.uint8, device=dev)
+        # bookkeeping is double-buffered on the device; state[STATE_EPOCH] says which half is current
+        self.indices = torch.empty(2, I, dtype=torch.int32, device=dev)
+        self.cur_mask = torch.empty(2, I, dtype=torch.uint8, device=dev)
         self.state = torch.empty(_lib.STATE_WORDS, dtype=torch.int32, device=dev)
-        self.scratch = torch.empty(2 * I, dtype=torch.int32, device=dev)
         self.n_active_dev = self.state[_lib.STATE_N_ACTIVE:_lib.STATE_N_ACTIVE + 1]
 
         bufs = _lib.CacheBuffers(
             self.gate_pool.data_ptr() if self.has_gate else None, self.up_pool.data_ptr(), self.downT_pool.data_ptr(),
             self.gate_active.data_ptr() if self.has_gate else None, self.up_active.data_ptr(),
-            self.down_active.data_ptr(), self.indices.data_ptr(), self.cur_mask.data_ptr(), self.state.data_ptr(),
-            self.scratch.data_ptr())
+            self.down_active.data_ptr(), self.indices.data_ptr(), self.cur_mask.data_ptr(), self.state.data_ptr())
         self._h = L.st_cache_create(C.byref(bufs), I, H, code, int(self.has_gate))
         if not self._h:
             raise ValueError(_lib.last_error())
@@ -122,7 +121,8 @@ class WeightCache:
         s = self._host_state
         return {"n_active": s[_lib.STATE_N_ACTIVE], "n_changed": s[_lib.STATE_N_CHANGED],
                 "status": s[_lib.STATE_STATUS], "valid": s[_lib.STATE_VALID], "n_added": s[_lib.STATE_N_ADDED],
-                "n_removed": s[_lib.STATE_N_REMOVED], "serial": s[_lib.STATE_SERIAL]}
+                "n_removed": s[_lib.STATE_N_REMOVED], "serial": s[_lib.STATE_SERIAL],
+                "epoch": s[_lib.STATE_EPOCH]}
 
     # ------------------------------------------------------------------ getters
     def get_num_active(self) -> int:
@@ -130,8 +130,8 @@ class WeightCache:
 
     def get_active_indices(self) -> torch.Tensor:
         """Ordered active list (the reference's ``active_indices``) as int64[n]."""
-        n = self.get_num_active()
-        return self.indices[:n].to(torch.int64)
+        st = self.sync_state()
+        return self.indices[int(st["epoch"]), : int(st["n_active"])].to(torch.int64)
 
     def _require_valid(self) -> dict:
         st = self.sync_state()
