@@ -43,6 +43,8 @@ def parse_args():
     ap.add_argument("--cpu-layers", type=int, default=2)
     ap.add_argument("--cpu-steps", type=int, default=24)
     ap.add_argument("--profile-steps", type=int, default=32)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (a known-size reference for rocprofv3 --pmc)")
     ap.add_argument("--seed", type=int, default=1236)
     return ap.parse_args()
 
@@ -191,6 +193,13 @@ def main():
     host_s = time.perf_counter() - t_host0
     ms_per_step = e0.elapsed_time(e1) / K
     tok_s = B * 1000.0 / ms_per_step
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)          # 268435456 bytes read + as many written by one copy kernel
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- second pass over the same masks (backwards, so every transition has the same churn) with
     # ---- per-kernel HIP events recorded on the launch stream

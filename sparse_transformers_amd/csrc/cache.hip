@@ -45,6 +45,7 @@ __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane)
 }
 
 // Exclusive scan of one uint32 per thread over the block; *total receives the sum.
+template <int WAVES>
 __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wave_tot, uint32_t *total)
 {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
@@ -53,7 +54,7 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wave_t
     if (lane == kWave - 1) wave_tot[wave] = incl;
     __syncthreads();
     uint32_t prefix = 0, tot = 0;
-    for (int w = 0; w < kPlanWaves; ++w) {
+    for (int w = 0; w < WAVES; ++w) {
         const uint32_t t = wave_tot[w];
         if (w < wave) prefix += t;
         tot += t;
@@ -82,8 +83,8 @@ __device__ __forceinline__ uint64_t nonzero_bytes(uint64_t x)
 // VEC: I % 8 == 0 and the mask is 8-byte aligned, so masks are read as 8-byte
 // words and indices as 16-byte vectors; both bookkeeping buffers are requested
 // together with the ticket, so the kernel front costs one memory round trip.
-template <bool VEC>
-__global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp, const uint8_t *__restrict__ new_mask,
+template <bool VEC, int TPB>
+__global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const uint8_t *__restrict__ new_mask,
                                                                     uint8_t *__restrict__ cur_mask2,
                                                                     int32_t *__restrict__ indices2,
                                                                     int32_t *__restrict__ state, int I, int gs_log2)
@@ -98,14 +99,14 @@ __global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp,
     uint32_t *dirty = reinterpret_cast<uint32_t *>(lists + I + (I & 1));  // bit per position
     const int dirty_words = (I + 31) >> 5;
     uint8_t *flag_l = reinterpret_cast<uint8_t *>(dirty + ((dirty_words + 1) & ~1));  // bit0 new, bit1 old; 8-byte aligned
-    __shared__ uint32_t wave_tot[kPlanWaves];
+    __shared__ uint32_t wave_tot[(TPB / kWave)];
     __shared__ int n_new_s;
     __shared__ uint32_t ticket_s;
 
     const int tid = threadIdx.x;
     ST_TL(0);
     // Elements per thread (a contiguous range, so the diff lists come out ascending).
-    const int E = VEC ? ((I + 8 * kPlanThreads - 1) / (8 * kPlanThreads)) * 8 : (I + kPlanThreads - 1) / kPlanThreads;
+    const int E = VEC ? ((I + 8 * TPB - 1) / (8 * TPB)) * 8 : (I + TPB - 1) / TPB;
     const int e0 = tid * E < I ? tid * E : I, e1 = e0 + E < I ? e0 + E : I;
 
     uint64_t v_new[kPlanMaxWords], v_cur[2][kPlanMaxWords];
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp,
     }
     // One atomic returns both the epoch (which buffer to read) and this block's ticket.
     if (tid == 0) ticket_s = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
-    for (int w = tid; w < dirty_words; w += kPlanThreads) dirty[w] = 0u;
+    for (int w = tid; w < dirty_words; w += TPB) dirty[w] = 0u;
     __syncthreads();
     const uint32_t ticket = ticket_s;
     const int ep = (int)((ticket >> 16) & 1u);
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp,
         const uint8_t *cur_mask = cur_mask2 + (size_t)ep * I;
         const int32_t *indices = indices2 + (size_t)ep * I;
         n = state[ST_STATE_N_BUF0 + ep];
-        for (int i = tid; i < I; i += kPlanThreads) {
+        for (int i = tid; i < I; i += TPB) {
             pos_l[i] = kNone;
             flag_l[i] = (new_mask[i] ? 1 : 0) | (cur_mask[i] ? 2 : 0);
             idx_l[i] = (uint16_t)indices[i];
@@ -169,7 +170,7 @@ __global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp,
     ST_TL(1);
     __syncthreads();
     ST_TL(2);
-    for (int p = tid; p < n; p += kPlanThreads) pos_l[idx_l[p]] = (uint16_t)p;
+    for (int p = tid; p < n; p += TPB) pos_l[idx_l[p]] = (uint16_t)p;
 
     // ---- diff: contiguous element range per thread keeps the lists ascending
     uint32_t cnt = 0;  // added in the low half, removed in the high half
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp,
         cnt += (f == 2) ? 0x10000u : 0u;
     }
     uint32_t total;
-    const uint32_t off = block_excl_scan(cnt, wave_tot, &total);  // contains __syncthreads
+    const uint32_t off = block_excl_scan<TPB / kWave>(cnt, wave_tot, &total);  // contains __syncthreads
     ST_TL(3);
     const int na = (int)(total & 0xffffu), nr = (int)(total >> 16);
     if (na == 0 && nr == 0) {  // unchanged mask: nothing is touched (weight_cache.h:237-240)
@@ -208,7 +209,7 @@ __global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp,
     // have run: they replace the added indices in `lists` in place and no compaction is needed.
     const bool fast = nr <= na;
     // ---- phase 1: paired replacement
-    for (int i = tid; i < pairs; i += kPlanThreads) {
+    for (int i = tid; i < pairs; i += TPB) {
         const int e = lists[I - 1 - i];
         const uint16_t p = pos_l[e];
         if (p != kNone) {
@@ -221,7 +222,7 @@ __global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp,
         if (fast) lists[i] = p;
     }
     // ---- phase 2: append surplus additions
-    for (int i = pairs + tid; i < na; i += kPlanThreads) {
+    for (int i = pairs + tid; i < na; i += TPB) {
         const int p = n + (i - pairs);
         if (p < I) {
             const int a = lists[i];
@@ -272,7 +273,7 @@ __global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp,
             if (lo >= n_new) word = 0;
             else if (lo + 32 > n_new) word &= (1u << (n_new - lo)) - 1u;
         }
-        uint32_t coff = block_excl_scan((uint32_t)__popc(word), wave_tot, &n_changed);  // barrier: lists are dead now
+        uint32_t coff = block_excl_scan<TPB / kWave>((uint32_t)__popc(word), wave_tot, &n_changed);  // barrier: lists are dead now
         while (word) {
             const int bit = __ffs(word) - 1;
             word &= word - 1;
@@ -285,7 +286,7 @@ __global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp,
     // ---- copy this block's share of the changed rows: active[m][p] <- pool[m][index at p]
     {
         const int nmat = cp.nmat, row_bytes = cp.row_bytes, chunks = row_bytes >> 4;
-        const int GS = 1 << gs_log2, ngrp = kPlanThreads >> gs_log2;
+        const int GS = 1 << gs_log2, ngrp = TPB >> gs_log2;
         const int grp = tid >> gs_log2, cc = tid & (GS - 1);
         const int slots = gridDim.x * ngrp, slot = blockIdx.x * ngrp + grp;
         const int work = (int)n_changed * nmat;
@@ -320,9 +321,9 @@ __global__ __launch_bounds__(kPlanThreads) void cache_update_kernel(CopyPlan cp,
     if (writer) {
         int32_t *idx_out = indices2 + (size_t)(ep ^ 1) * I;
         uint8_t *mask_out = cur_mask2 + (size_t)(ep ^ 1) * I;
-        for (int p = tid; p < n_new; p += kPlanThreads) idx_out[p] = idx_l[p];
+        for (int p = tid; p < n_new; p += TPB) idx_out[p] = idx_l[p];
         // the reference stores the new mask only when the rebuild did not throw (n_new > 0)
-        for (int i = tid; i < I; i += kPlanThreads) mask_out[i] = n_new > 0 ? (flag_l[i] & 1) : (flag_l[i] >> 1);
+        for (int i = tid; i < I; i += TPB) mask_out[i] = n_new > 0 ? (flag_l[i] & 1) : (flag_l[i] >> 1);
         if (tid == 0) {
             state[ST_STATE_N_BUF0 + (ep ^ 1)] = n_new;
             state[ST_STATE_N_ACTIVE] = n_new;
@@ -450,14 +451,6 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int I = (int)c->I;
     const size_t lds = (size_t)I * 6 + (I & 1) * 2 + (size_t)((((I + 31) >> 5) + 1) & ~1) * 4 + (size_t)I + 16;
-    static bool attr_set = false;
-    if (!attr_set) {
-        ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(cache_update_kernel<true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
-        ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(cache_update_kernel<false>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
-        attr_set = true;
-    }
     CopyPlan cp;
     cp.nmat = 0;
     if (c->has_gate) {
@@ -471,24 +464,43 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     for (int k = cp.nmat; k < 3; ++k) { cp.pool[k] = cp.pool[0]; cp.active[k] = cp.active[0]; }
     cp.row_bytes = (int)(c->H * c->esz);
     const int chunks = cp.row_bytes >> 4;
-    int gs_log2 = 6;
-    while ((1 << gs_log2) < chunks && (1 << gs_log2) < kPlanThreads) ++gs_log2;
     static const int blocks = [] {
         const char *v = getenv("ST_CACHE_BLOCKS");
         const int b = v ? atoi(v) : 0;
         return b >= 1 && b <= 1024 ? b : 0;
     }();
+    static const int want_tpb = [] {
+        const char *v = getenv("ST_CACHE_TPB");
+        return v ? atoi(v) : 0;
+    }();
     const int grid = blocks ? blocks : device_cu_count() / 2;
+    const bool aligned = (I % 8 == 0) && ((uintptr_t)mask % 8 == 0) && ((uintptr_t)c->b.cur_mask % 8 == 0) &&
+                         ((uintptr_t)c->b.indices % 16 == 0);
+    // 512-thread blocks (ST_CACHE_TPB=512) leave room on the CU for a kernel of another stream, but
+    // measure slower on their own; they cover I <= 12288 in the vector path.
+    const bool small = want_tpb == 512 && aligned && I <= 8 * 512 * kPlanMaxWords;
+    const int tpb = small ? 512 : 1024;
+    const bool vec = aligned && I <= 8 * tpb * kPlanMaxWords;
+    int gs_log2 = 6;
+    while ((1 << gs_log2) < chunks && (1 << gs_log2) < tpb) ++gs_log2;
     {
         ProfScope ps(ST_K_CACHE_UPDATE, s);
-        const bool vec = (I % 8 == 0) && ((uintptr_t)mask % 8 == 0) && ((uintptr_t)c->b.cur_mask % 8 == 0) &&
-                         ((uintptr_t)c->b.indices % 16 == 0) && I <= 8 * kPlanThreads * kPlanMaxWords;
-        if (vec)
-            hipLaunchKernelGGL(cache_update_kernel<true>, dim3(grid), dim3(kPlanThreads), lds, s, cp, mask,
-                               c->b.cur_mask, c->b.indices, c->b.state, I, gs_log2);
-        else
-            hipLaunchKernelGGL(cache_update_kernel<false>, dim3(grid), dim3(kPlanThreads), lds, s, cp, mask,
-                               c->b.cur_mask, c->b.indices, c->b.state, I, gs_log2);
+        auto launch = [&](auto kern) -> int {
+            static bool attr_set = false;
+            if (!attr_set) {
+                ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+                attr_set = true;
+            }
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(tpb), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state,
+                               I, gs_log2);
+            return ST_OK;
+        };
+        int rc;
+        if (small) rc = launch(cache_update_kernel<true, 512>);
+        else if (vec) rc = launch(cache_update_kernel<true, 1024>);
+        else rc = launch(cache_update_kernel<false, 1024>);
+        if (rc != ST_OK) return rc;
     }
     ST_HIP(hipGetLastError());
     return ST_OK;

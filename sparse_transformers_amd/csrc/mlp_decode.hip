@@ -1,11 +1,13 @@
 // Fused sparse-MLP decode kernel for gfx950 (small batch, HBM-bound).
 //
 // One launch streams the three packed active matrices exactly once.  A block
-// (one per CU, 512 threads, so each thread may hold up to 256 VGPRs) owns a
-// contiguous range of active rows.  Every thread owns one 16-byte column chunk
-// of the hidden dimension (two when the row has more than 512 chunks) and, for
-// each row of its group, issues the gate, up AND down loads of that chunk up
-// front, so a whole batch of rows is in flight before any arithmetic:
+// (one per CU) owns the active rows j with j % gridDim.x == blockIdx.x.  Every
+// thread owns one 16-byte column chunk of the hidden dimension (two for very
+// wide rows) and, for each row its thread group has in flight, issues the
+// gate, up AND down loads of that chunk together.  Rows are processed in
+// batches of RB per group through two register buffers: while one batch is
+// being computed the loads of the next are in flight, so the memory system is
+// kept busy through the reductions and barriers of the previous batch.
 //   phase 1  per-thread partial products <gate[j],x>, <up[j],x> on the chunk,
 //            DPP wave reduction, cross-wave sum through LDS,
 //            h[j] = act(g) * u  left in LDS
@@ -22,10 +24,16 @@
 
 namespace st {
 
-// T: storage type; NB: x rows per launch; RB: rows per group kept in flight;
-// CPT: 16-byte chunks per thread (2 only when one group spans the block);
-// TPB: threads per block (512 leaves 256 VGPRs per thread, 1024 leaves 128).
-template <typename T, int NB, int RB, int CPT, int TPB>
+template <int RB, int CPT> struct RowBatch {
+    uint4 g[RB][CPT], u[RB][CPT], d[RB][CPT];
+};
+
+// T: storage type; NB: x rows per launch; RB: rows per group in one register
+// buffer; CPT: 16-byte chunks per thread; TPB: threads per block (512 leaves
+// 256 VGPRs per thread, 1024 leaves 128); DB: two register buffers (the next
+// batch is in flight while one is computed) or one (a single deep batch, which
+// measures faster when all rows of a block fit in it).
+template <typename T, int NB, int RB, int CPT, int TPB, bool DB>
 __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
     const T *__restrict__ x, int B, int H, const T *__restrict__ gate, const T *__restrict__ up,
     const T *__restrict__ down, int n_host, const int *__restrict__ n_dev, int n_hint, T *__restrict__ combined,
@@ -33,17 +41,16 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
 {
     constexpr int VEC = Elem<T>::kVec;
     extern __shared__ __align__(16) unsigned char region[];  // group combine buffer
-    constexpr int kMlpThreads = TPB;
     __shared__ float red[TPB / kWave][RB][NB][2];             // per-wave partial (g,u)
-    __shared__ float hs[TPB / kWave][RB][NB];                 // h of the rows in flight
+    __shared__ float hs[TPB / kWave][RB][NB];                 // h of the rows being computed
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int G = gridDim.x, blk = blockIdx.x;
-    // Active count: requested first, consumed only after the first batch of
-    // weight loads has been issued.  Rows are dealt to blocks round-robin
-    // (row j belongs to block j % G), so which rows a block owns does not
-    // depend on the count, and rows below `n_spec` can be requested before
-    // the count has arrived (the active buffers hold I rows, so this is safe).
+    // Active count: requested first, consumed only after the first two batches
+    // of weight loads have been issued.  Rows are dealt to blocks round-robin,
+    // so which rows a block owns does not depend on the count, and rows below
+    // `n_spec` can be requested before the count has arrived (the active
+    // buffers hold I rows, so this is safe).
     ST_TL(0);
     const int nd_raw = n_dev ? *n_dev : n_host;
     const int n_spec = n_dev ? (n_hint < n_host ? n_hint : n_host) : n_host;
@@ -51,7 +58,7 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
 
     // groups of 2^gs_log2 threads each cover all chunks of a row
-    const int GS = 1 << gs_log2, ngrp = kMlpThreads >> gs_log2, wpg = GS >> 6;
+    const int GS = 1 << gs_log2, ngrp = TPB >> gs_log2, wpg = GS >> 6;
     const int grp = tid >> gs_log2, cc = tid & (GS - 1);
     bool valid[CPT];
     size_t coff[CPT];
@@ -67,20 +74,45 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
 #pragma unroll
         for (int q = 0; q < CPT; ++q) xr[b][q] = (valid[q] && b < B) ? ld16(x + (size_t)b * H + coff[q]) : zero4;
 
-    uint4 wg[RB][CPT], wu[RB][CPT], wd[RB][CPT];
+    // row of (batch, slot k) for this thread's group
+    auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
+    auto load_batch = [&](RowBatch<RB, CPT> &w, int bat, int limit) {
 #pragma unroll
-    for (int k = 0; k < RB; ++k) {
-        const int row = blk + G * (grp + ngrp * k);
+        for (int k = 0; k < RB; ++k) {
+            const int row = row_of(bat, k);
 #pragma unroll
-        for (int q = 0; q < CPT; ++q) {
-            const bool ok = valid[q] && row < n_spec;
-            const size_t o = (size_t)row * H + coff[q];
-            wg[k][q] = (ok && has_gate) ? ld16_stream(gate + o) : zero4;
-            wu[k][q] = ok ? ld16_stream(up + o) : zero4;
-            wd[k][q] = ok ? ld16_stream(down + o) : zero4;
+            for (int q = 0; q < CPT; ++q) {
+                const bool ok = valid[q] && row < limit;
+                const size_t o = (size_t)row * H + coff[q];
+                w.g[k][q] = (ok && has_gate) ? ld16_stream(gate + o) : zero4;
+                w.u[k][q] = ok ? ld16_stream(up + o) : zero4;
+                w.d[k][q] = ok ? ld16_stream(down + o) : zero4;
+            }
         }
-    }
+    };
+    // A batch requested with the host's guess: fetch what the guess missed, drop what it overshot.
+    auto fix_batch = [&](RowBatch<RB, CPT> &w, int bat, int n) {
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+            const int row = row_of(bat, k);
+            const bool have = row < n_spec, want = row < n;
+#pragma unroll
+            for (int q = 0; q < CPT; ++q) {
+                if (want && !have && valid[q]) {
+                    const size_t o = (size_t)row * H + coff[q];
+                    w.g[k][q] = has_gate ? ld16_stream(gate + o) : zero4;
+                    w.u[k][q] = ld16_stream(up + o);
+                    w.d[k][q] = ld16_stream(down + o);
+                } else if (have && !want) {
+                    w.g[k][q] = zero4; w.u[k][q] = zero4; w.d[k][q] = zero4;
+                }
+            }
+        }
+    };
 
+    RowBatch<RB, CPT> w0, w1;
+    load_batch(w0, 0, n_spec);
+    if constexpr (DB) load_batch(w1, 1, n_spec);
     ST_TL(1);
     int n = nd_raw < n_host ? nd_raw : n_host;
     if (n < 0) n = 0;
@@ -93,27 +125,7 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
 #pragma unroll
             for (int e = 0; e < VEC; ++e) acc[b][q][e] = 0.f;
 
-    const int jcount = n > blk ? (n - blk + G - 1) / G : 0;  // rows of this block
-    const int nbat = ((jcount + ngrp - 1) / ngrp + RB - 1) / RB;  // uniform over the block
-    for (int bat = 0; bat < nbat; ++bat) {
-#pragma unroll
-        for (int k = 0; k < RB; ++k) {
-            const int row = blk + G * (grp + ngrp * (bat * RB + k));
-            // batch 0 was requested speculatively; fetch what the guess missed, drop what it overshot
-            const bool have = bat == 0 && row < n_spec;
-#pragma unroll
-            for (int q = 0; q < CPT; ++q) {
-                const bool ok = valid[q] && row < n;
-                const size_t o = (size_t)row * H + coff[q];
-                if (!have) {
-                    wg[k][q] = (ok && has_gate) ? ld16_stream(gate + o) : zero4;
-                    wu[k][q] = ok ? ld16_stream(up + o) : zero4;
-                    wd[k][q] = ok ? ld16_stream(down + o) : zero4;
-                } else if (!ok) {
-                    wg[k][q] = zero4; wu[k][q] = zero4; wd[k][q] = zero4;
-                }
-            }
-        }
+    auto compute = [&](const RowBatch<RB, CPT> &w, int bat) {
         // ---- phase 1: partial dot products on this thread's chunk(s)
         float pg[RB][NB], pu[RB][NB];
 #pragma unroll
@@ -123,8 +135,8 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
 #pragma unroll
             for (int q = 0; q < CPT; ++q) {
                 float fg[VEC], fu[VEC];
-                unpack<T>(wg[k][q], fg);
-                unpack<T>(wu[k][q], fu);
+                unpack<T>(w.g[k][q], fg);
+                unpack<T>(w.u[k][q], fu);
 #pragma unroll
                 for (int b = 0; b < NB; ++b) {
                     float fx[VEC];
@@ -156,9 +168,9 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
             const int k_ = rem / NB, b_ = rem - k_ * NB;
             const int row = blk + G * (g_ + ngrp * (bat * RB + k_));
             float sg = 0.f, su = 0.f;
-            for (int w = g_ * wpg; w < (g_ + 1) * wpg; ++w) {
-                sg += red[w][k_][b_][0];
-                su += red[w][k_][b_][1];
+            for (int wv = g_ * wpg; wv < (g_ + 1) * wpg; ++wv) {
+                sg += red[wv][k_][b_][0];
+                su += red[wv][k_][b_][1];
             }
             const float hv = has_gate ? activate(sg, act) * su : activate(su, act);
             const bool ok = row < n;
@@ -176,7 +188,7 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
 #pragma unroll
             for (int q = 0; q < CPT; ++q) {
                 float fw[VEC];
-                unpack<T>(wd[k][q], fw);
+                unpack<T>(w.d[k][q], fw);
 #pragma unroll
                 for (int b = 0; b < NB; ++b) {
                     const float hv = hs[grp][k][b];
@@ -184,6 +196,28 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
                     for (int e = 0; e < VEC; ++e) acc[b][q][e] = fmaf(hv, fw[e], acc[b][q][e]);
                 }
             }
+    };
+
+    const int jcount = n > blk ? (n - blk + G - 1) / G : 0;      // rows of this block
+    const int nbat = ((jcount + ngrp - 1) / ngrp + RB - 1) / RB;  // uniform over the block
+    if (n_dev && nbat > 0) {
+        fix_batch(w0, 0, n);
+        if constexpr (DB) fix_batch(w1, 1, n);
+    }
+    if constexpr (DB) {
+        for (int bat = 0; bat < nbat; bat += 2) {
+            compute(w0, bat);
+            if (bat + 2 < nbat) load_batch(w0, bat + 2, n);
+            if (bat + 1 < nbat) {
+                compute(w1, bat + 1);
+                if (bat + 3 < nbat) load_batch(w1, bat + 3, n);
+            }
+        }
+    } else {
+        for (int bat = 0; bat < nbat; ++bat) {
+            if (bat > 0) load_batch(w0, bat, n);
+            compute(w0, bat);
+        }
     }
 
     ST_TL(5);
@@ -279,7 +313,7 @@ struct MlpLaunch {
     int G;
 };
 
-template <typename T, int NB, int RB, int CPT, int TPB>
+template <typename T, int NB, int RB, int CPT, int TPB, bool DB>
 static int launch_inst(const MlpLaunch &a, int b0, int bcount)
 {
     const int chunks = a.H / Elem<T>::kVec;
@@ -289,7 +323,7 @@ static int launch_inst(const MlpLaunch &a, int b0, int bcount)
     const int ngrp = TPB >> gs_log2;
     const size_t lds = (size_t)(ngrp - 1) * NB * a.H * 4;
     ST_REQUIRE(lds <= (size_t)kMaxLds - 8192, "st_mlp_forward: H=%d needs %zu bytes of LDS", a.H, lds);
-    auto kern = mlp_decode_kernel<T, NB, RB, CPT, TPB>;
+    auto kern = mlp_decode_kernel<T, NB, RB, CPT, TPB, DB>;
     static bool attr_set = false;
     if (!attr_set) {
         ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -326,7 +360,8 @@ static int env_int(const char *name)
 
 // The launch shape trades registers for loads in flight: measured on MI355X,
 // about 12-18 outstanding 16-byte loads per thread with 16 waves per CU
-// streams fastest; many more per thread is slower.
+// streams fastest; many more per thread is slower.  RB is the depth of ONE of
+// the two register buffers.
 template <typename T, int NB> static int launch_one(const MlpLaunch &a, int b0, int bcount)
 {
     static const int want_tpb = env_int("ST_MLP_TPB"), want_rb = env_int("ST_MLP_RB");
@@ -334,35 +369,43 @@ template <typename T, int NB> static int launch_one(const MlpLaunch &a, int b0, 
     ST_REQUIRE(chunks <= 2048, "st_mlp_forward: hidden size %d too large for this dtype (max %d)", a.H,
                2048 * Elem<T>::kVec);
     if constexpr (NB == 1) {
-        if (chunks > 1024) return launch_inst<T, 1, 3, 2, 1024>(a, b0, bcount);
-        if (want_tpb == 512 || (want_tpb == 0 && false)) {
-            if (chunks > 512) return want_rb == 4 ? launch_inst<T, 1, 4, 2, 512>(a, b0, bcount)
-                                                 : launch_inst<T, 1, 6, 2, 512>(a, b0, bcount);
+        if (chunks > 1024) return launch_inst<T, 1, 3, 2, 1024, false>(a, b0, bcount);
+        if (want_tpb == 512) {
+            if (chunks > 512) return launch_inst<T, 1, 6, 2, 512, false>(a, b0, bcount);
             switch (want_rb) {
-            case 4: return launch_inst<T, 1, 4, 1, 512>(a, b0, bcount);
-            case 8: return launch_inst<T, 1, 8, 1, 512>(a, b0, bcount);
-            case 12: return launch_inst<T, 1, 12, 1, 512>(a, b0, bcount);
-            default: return launch_inst<T, 1, 6, 1, 512>(a, b0, bcount);
+            case 3: return launch_inst<T, 1, 3, 1, 512, true>(a, b0, bcount);
+            case 4: return launch_inst<T, 1, 4, 1, 512, false>(a, b0, bcount);
+            case 12: return launch_inst<T, 1, 12, 1, 512, false>(a, b0, bcount);
+            default: return launch_inst<T, 1, 6, 1, 512, false>(a, b0, bcount);
             }
         }
-        if (want_rb == 4) return launch_inst<T, 1, 4, 1, 1024>(a, b0, bcount);
-        return launch_inst<T, 1, 6, 1, 1024>(a, b0, bcount);
+        if (want_rb == 3) return launch_inst<T, 1, 3, 1, 1024, true>(a, b0, bcount);
+        if (want_rb == 4) return launch_inst<T, 1, 4, 1, 1024, false>(a, b0, bcount);
+        return launch_inst<T, 1, 6, 1, 1024, false>(a, b0, bcount);
     } else if constexpr (NB == 2) {
-        if (chunks > 1024) return launch_inst<T, 2, 2, 2, 512>(a, b0, bcount);
-        return launch_inst<T, 2, 4, 1, 1024>(a, b0, bcount);
+        return launch_inst<T, 2, 2, 1, 1024, true>(a, b0, bcount);
+    } else if constexpr (NB == 4) {
+        if (chunks > 512) return launch_inst<T, 4, 1, 2, 512, true>(a, b0, bcount);
+        return launch_inst<T, 4, 3, 1, 512, true>(a, b0, bcount);
     } else {
-        if (chunks > 512) return launch_inst<T, 4, 2, 2, 512>(a, b0, bcount);
-        return launch_inst<T, 4, 4, 1, 512>(a, b0, bcount);
+        return launch_inst<T, 8, 2, 1, 512, true>(a, b0, bcount);  // chunks <= 512 only (see launch_nb)
     }
 }
 
 template <typename T> static int launch_nb(const MlpLaunch &a)
 {
+    const int chunks = a.H / Elem<T>::kVec;
     int b0 = 0;
     while (b0 < a.B) {
         const int left = a.B - b0;
         int rc;
-        if (left >= 3) {
+        if (chunks > 1024) {  // very wide rows: one row of x per pass
+            rc = launch_one<T, 1>(a, b0, 1);
+            b0 += 1;
+        } else if (left >= 5 && chunks <= 512) {
+            rc = launch_one<T, 8>(a, b0, left < 8 ? left : 8);
+            b0 += 8;
+        } else if (left >= 3) {
             rc = launch_one<T, 4>(a, b0, left < 4 ? left : 4);
             b0 += 4;
         } else if (left == 2) {
@@ -377,7 +420,7 @@ template <typename T> static int launch_nb(const MlpLaunch &a)
     return ST_OK;
 }
 
-constexpr int kMlpMaxBatchPerLaunch = 4;
+constexpr int kMlpMaxBatchPerLaunch = 8;
 
 // Blocks per launch: one per CU by default; ST_MLP_GMULT (1..4) multiplies it.
 int mlp_grid()

@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kWave) void predictor_up_mask_kernel(const float *_
 #pragma unroll
             for (int b = 0; b < kPredUpBTile; ++b) {
                 if (b0 + b < B) {  // uniform across the wave
-                    const float v = group_sum(s[it][b], LPR);
+                    const float v = group_sum_dpp<LPR>(s[it][b]);
                     any[it] = any[it] || (cmp_ge ? (v >= thr) : (v > thr));
                     if (scores && cl == 0 && row_ok) scores[(size_t)(b0 + b) * I + row] = v;
                 }

@@ -122,6 +122,22 @@ __device__ __forceinline__ float wave_sum_dpp(float v)
     return (r0 + r1) + (r2 + r3);
 }
 
+// Sum over aligned groups of WIDTH lanes (4, 8, 16, 32 or 64); every lane of a group receives it.
+template <int WIDTH> __device__ __forceinline__ float group_sum_dpp(float v)
+{
+    static_assert(WIDTH == 4 || WIDTH == 8 || WIDTH == 16 || WIDTH == 32 || WIDTH == 64, "unsupported group width");
+    if constexpr (WIDTH == 64) {
+        return wave_sum_dpp(v);
+    } else {
+        v = dpp_add<0xB1>(v);
+        v = dpp_add<0x4E>(v);
+        if constexpr (WIDTH >= 8) v = dpp_add<0x141>(v);
+        if constexpr (WIDTH >= 16) v = dpp_add<0x140>(v);
+        if constexpr (WIDTH == 32) v += __shfl_xor(v, 16, kWave);
+        return v;
+    }
+}
+
 // Sum over aligned groups of `width` lanes (power of two <= 64).
 __device__ __forceinline__ float group_sum(float v, int width)
 {
