@@ -26,6 +26,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of mlp_decode_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by
+# what the same counter reads for a 256 MiB copy; see profiles/mlp_decode_traffic_llama3b_stack_fp16.md
+MEASURED_TRAFFIC_BYTES = {"llama3b_stack_fp16": 53_040_000 + 3_145_728}
 
 
 def parse_args():
@@ -202,18 +205,30 @@ def main():
         del src, dst
 
     # ---- second pass over the same masks (backwards, so every transition has the same churn) with
-    # ---- per-kernel HIP events recorded on the launch stream
+    # ---- per-kernel HIP events recorded on the launch stream by the library.  With a graph the events
     L = _lib.lib()
-    cap = P * layers * 8
-    _lib.check(L.st_profile_enable(cap), "st_profile_enable")
+    per_step = layers * 8
+    kinds_all, ms_all = [], []
+    kinds = (C.c_int * per_step)()
+    ms = (C.c_float * per_step)()
+
+    def collect():
+        cnt = L.st_profile_collect(kinds, ms, per_step)
+        if cnt < 0:
+            _lib.check(cnt, "st_profile_collect")
+        kinds_all.append(np.frombuffer(kinds, dtype=np.int32)[:cnt].copy())
+        ms_all.append(np.frombuffer(ms, dtype=np.float32)[:cnt].copy())
+
+    # (Events recorded inside a captured graph cannot be read back with hipEventElapsedTime on this ROCm, so
+    # this pass launches eagerly; the GPU idles between launches and the events bracket dispatch overhead,
+    # which makes these durations about 2 us longer than rocprofv3's kernel times - see profiles/.)
     for t in range(W + K - 1, W + K - 1 - P, -1):
+        _lib.check(L.st_profile_enable(per_step), "st_profile_enable")
         stack.step_staged(x_in[t], x_pred[t], trace[t], replay=False)
-    torch.cuda.synchronize()
-    kinds = (C.c_int * cap)()
-    ms = (C.c_float * cap)()
-    cnt = L.st_profile_collect(kinds, ms, cap)
+        torch.cuda.synchronize()
+        collect()
     L.st_profile_disable()
-    kinds_np, ms_np = np.frombuffer(kinds, dtype=np.int32)[:cnt], np.frombuffer(ms, dtype=np.float32)[:cnt]
+    kinds_np, ms_np = np.concatenate(kinds_all), np.concatenate(ms_all)
     per_kernel = {}
     for k, name in enumerate(_lib.KERNEL_KINDS):
         sel = ms_np[kinds_np == k]
@@ -238,9 +253,11 @@ def main():
                    "batch": B, "act": wl.act, "has_gate": wl.has_gate, "n_active": n,
                    "churn": [wl.churn_lo, wl.churn_hi], "mask_source": "trace",
                    "launch": "hip_graph" if use_graph else "eager",
-                   "streams": 2 if args.overlap else 1},
+                   "streams": 2 if args.overlap else 1,
+                   "kernel_timing": "hip events, eager second pass"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "mlp_decode_kernel",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name), "kernel": "mlp_decode_kernel",
                      "bytes_per_launch": alg_bytes, "mean_us": mlp_us},
         "cache_update_us_per_layer": round(upd_us, 3),
         "stack_hbm_gbps": round(layers * alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),

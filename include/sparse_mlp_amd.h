@@ -192,8 +192,10 @@ typedef enum st_kernel_kind {
 
 int st_profile_enable(int max_samples); /* host; allocates the event pool */
 int st_profile_disable(void);
-/* host; kinds/ms: arrays of `cap` entries; returns the number of samples
- * written (or a negative st_status) and clears the sample list */
+/* host; kinds/ms: arrays of `cap` entries; waits for the recorded events and
+ * returns the number of samples written (or a negative st_status).  The
+ * sample list is kept (st_profile_enable starts a new one), so launches that
+ * were captured into a HIP graph can be read again after every replay. */
 int st_profile_collect(int *kinds, float *ms, int cap);
 
 #ifdef __cplusplus

@@ -96,7 +96,6 @@ extern "C" int st_profile_collect(int *kinds, float *ms, int cap)
         ms[nout] = t;
         ++nout;
     }
-    g_prof.used = 0;
     return nout;
 }
 
