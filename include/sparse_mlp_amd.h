@@ -73,7 +73,7 @@ const char *st_last_error(void);
  *   workspace          scratch of st_mlp_workspace_bytes(B,H,n) bytes
  * All rows must be 16-byte aligned (H*sizeof(dtype) % 16 == 0). B <= 4096.
  * B < 32 runs the streaming decode kernel (HBM-bound); B >= 32 in fp16 / bf16
- * with H % 32 == 0 runs the MFMA kernels (then only columns [0,n) of
+ * with H % 128 == 0 runs the MFMA kernels (then only columns [0,n) of
  * `combined` are written).
  * ------------------------------------------------------------------------ */
 int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n);

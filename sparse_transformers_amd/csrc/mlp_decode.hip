@@ -65,54 +65,57 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
 #pragma unroll
     for (int q = 0; q < CPT; ++q) {
         valid[q] = cc + q * GS < chunks;
-        coff[q] = (size_t)(cc + q * GS) * VEC;
+        coff[q] = valid[q] ? (size_t)(cc + q * GS) * VEC : 0;   // clamped: loads below are unconditional
     }
+
+    // a wave whose 64 chunks all lie past the row end (H/VEC not a power of two) loads nothing (scalar test)
+    const bool wave_live = __builtin_amdgcn_readfirstlane(cc & ~(kWave - 1)) < chunks;
 
     uint4 xr[NB][CPT];
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int q = 0; q < CPT; ++q) xr[b][q] = (valid[q] && b < B) ? ld16(x + (size_t)b * H + coff[q]) : zero4;
+        for (int q = 0; q < CPT; ++q) {
+            xr[b][q] = ld16(x + (size_t)(b < B ? b : 0) * H + coff[q]);
+            if (!(valid[q] && b < B)) xr[b][q] = zero4;
+        }
 
     // row of (batch, slot k) for this thread's group
     auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
-    auto load_batch = [&](RowBatch<RB, CPT> &w, int bat, int limit) {
+    // Loads are issued unconditionally from a clamped row / chunk: a branch around every load costs far
+    // more than a few duplicate (cache-hit) loads.  What a clamped load returns is never used: x is zero
+    // on chunks past the row end, h is forced to zero for rows >= n, and the down row is replaced by
+    // zeros where it is consumed.  limit >= 1.
+    auto load_batch = [&](RowBatch<RB, CPT> &w, int bat, int limit) __attribute__((always_inline)) {
+        if (!wave_live) return;
 #pragma unroll
         for (int k = 0; k < RB; ++k) {
             const int row = row_of(bat, k);
+            const size_t ro = (size_t)(row < limit ? row : limit - 1) * H;
 #pragma unroll
             for (int q = 0; q < CPT; ++q) {
-                const bool ok = valid[q] && row < limit;
-                const size_t o = (size_t)row * H + coff[q];
-                w.g[k][q] = (ok && has_gate) ? ld16_stream(gate + o) : zero4;
-                w.u[k][q] = ok ? ld16_stream(up + o) : zero4;
-                w.d[k][q] = ok ? ld16_stream(down + o) : zero4;
+                const size_t o = ro + coff[q];
+                w.u[k][q] = ld16_stream(up + o);
+                w.d[k][q] = ld16_stream(down + o);
+                w.g[k][q] = has_gate ? ld16_stream(gate + o) : zero4;
             }
         }
     };
-    // A batch requested with the host's guess: fetch what the guess missed, drop what it overshot.
-    auto fix_batch = [&](RowBatch<RB, CPT> &w, int bat, int n) {
+    auto zero_batch = [&](RowBatch<RB, CPT> &w) __attribute__((always_inline)) {
 #pragma unroll
-        for (int k = 0; k < RB; ++k) {
-            const int row = row_of(bat, k);
-            const bool have = row < n_spec, want = row < n;
+        for (int k = 0; k < RB; ++k)
 #pragma unroll
-            for (int q = 0; q < CPT; ++q) {
-                if (want && !have && valid[q]) {
-                    const size_t o = (size_t)row * H + coff[q];
-                    w.g[k][q] = has_gate ? ld16_stream(gate + o) : zero4;
-                    w.u[k][q] = ld16_stream(up + o);
-                    w.d[k][q] = ld16_stream(down + o);
-                } else if (have && !want) {
-                    w.g[k][q] = zero4; w.u[k][q] = zero4; w.d[k][q] = zero4;
-                }
-            }
-        }
+            for (int q = 0; q < CPT; ++q) { w.g[k][q] = zero4; w.u[k][q] = zero4; w.d[k][q] = zero4; }
     };
 
     RowBatch<RB, CPT> w0, w1;
-    load_batch(w0, 0, n_spec);
-    if constexpr (DB) load_batch(w1, 1, n_spec);
+    if (n_spec > 0 && wave_live) {
+        load_batch(w0, 0, n_spec);
+        if constexpr (DB) load_batch(w1, 1, n_spec);
+    } else {
+        zero_batch(w0);
+        if constexpr (DB) zero_batch(w1);
+    }
     ST_TL(1);
     int n = nd_raw < n_host ? nd_raw : n_host;
     if (n < 0) n = 0;
@@ -184,11 +187,12 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
         ST_TL(4);
         // ---- phase 2: down projection from the rows already in registers
 #pragma unroll
-        for (int k = 0; k < RB; ++k)
+        for (int k = 0; k < RB; ++k) {
+            const bool row_ok = row_of(bat, k) < n;
 #pragma unroll
             for (int q = 0; q < CPT; ++q) {
                 float fw[VEC];
-                unpack<T>(w.d[k][q], fw);
+                unpack<T>(row_ok ? w.d[k][q] : zero4, fw);   // rows past the count may hold anything
 #pragma unroll
                 for (int b = 0; b < NB; ++b) {
                     const float hv = hs[grp][k][b];
@@ -196,13 +200,14 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
                     for (int e = 0; e < VEC; ++e) acc[b][q][e] = fmaf(hv, fw[e], acc[b][q][e]);
                 }
             }
+        }
     };
 
     const int jcount = n > blk ? (n - blk + G - 1) / G : 0;      // rows of this block
     const int nbat = ((jcount + ngrp - 1) / ngrp + RB - 1) / RB;  // uniform over the block
-    if (n_dev && nbat > 0) {
-        fix_batch(w0, 0, n);
-        if constexpr (DB) fix_batch(w1, 1, n);
+    if (n != n_spec && nbat > 0) {  // the host's guess was off: request the first batches again with the true count
+        load_batch(w0, 0, n);
+        if constexpr (DB) load_batch(w1, 1, n);
     }
     if constexpr (DB) {
         for (int bat = 0; bat < nbat; bat += 2) {
@@ -462,7 +467,7 @@ extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *g
                             (uintptr_t)workspace;
     ST_REQUIRE((align & 15) == 0, "st_mlp_forward: pointers must be 16-byte aligned");
 
-    if (B >= kPrefillMinRows && dtype != ST_F32 && H % 32 == 0)
+    if (B >= kPrefillMinRows && dtype != ST_F32 && H % 128 == 0 && n >= 1)
         return launch_prefill(dtype, x, (int)B, (int)H, gate_rows, up_rows, down_rows, (int)n, n_dev, out, combined,
                               (long)ldc, workspace, act, has_gate ? 1 : 0, static_cast<hipStream_t>(stream));
 
