@@ -72,9 +72,11 @@ const char *st_last_error(void);
  *                      leaves in combined_proj_buffer
  *   workspace          scratch of st_mlp_workspace_bytes(B,H,n) bytes
  * All rows must be 16-byte aligned (H*sizeof(dtype) % 16 == 0). B <= 4096.
- * B < 32 runs the streaming decode kernel (HBM-bound); B >= 32 in fp16 / bf16
- * with H % 128 == 0 runs the MFMA kernels (then only columns [0,n) of
- * `combined` are written).
+ * B == 1 (and any B < 32 in fp32 or with a hidden size the MFMA kernels do not
+ * cover) runs the streaming decode kernel; 2 <= B < 32 in fp16 / bf16 with H in
+ * {2048, 3072, 4096} runs the MFMA batch kernels (still HBM-bound, one pass over
+ * the weights per 16 rows); B >= 32 in fp16 / bf16 with H % 128 == 0 runs the
+ * MFMA GEMM kernels (then only columns [0,n) of `combined` are written).
  * ------------------------------------------------------------------------ */
 int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n);
 int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
@@ -187,7 +189,9 @@ typedef enum st_kernel_kind {
     ST_K_PRED_UP_MASK = 5,
     ST_K_MLP_PREFILL_GATEUP = 6,
     ST_K_MLP_PREFILL_DOWN = 7,
-    ST_K_KINDS = 8
+    ST_K_MLP_BATCH_GATEUP = 8,
+    ST_K_MLP_BATCH_DOWN = 9,
+    ST_K_KINDS = 10
 } st_kernel_kind;
 
 int st_profile_enable(int max_samples); /* host; allocates the event pool */

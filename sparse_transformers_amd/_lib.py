@@ -54,7 +54,7 @@ SIGNATURES = {
 }
 
 KERNEL_KINDS = ["mlp_decode", "mlp_reduce", "cache_update", "reserved", "pred_down", "pred_up_mask",
-                "mlp_prefill_gateup", "mlp_prefill_down"]
+                "mlp_prefill_gateup", "mlp_prefill_down", "mlp_batch_gateup", "mlp_batch_down"]
 
 _lib = None
 

@@ -427,6 +427,14 @@ template <typename T> static int launch_nb(const MlpLaunch &a)
 
 constexpr int kMlpMaxBatchPerLaunch = 8;
 
+// Rows of x from which the MFMA batch kernels take over from the streaming kernel
+// (ST_MLP_BATCH_MIN overrides; 32 or more switches them off).
+int batch_min_rows()
+{
+    static const int v = [] { const int m = env_int("ST_MLP_BATCH_MIN"); return m >= 2 ? m : 2; }();
+    return v;
+}
+
 // Blocks per launch: one per CU by default; ST_MLP_GMULT (1..4) multiplies it.
 int mlp_grid()
 {
@@ -439,7 +447,11 @@ int mlp_grid()
 extern "C" int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n)
 {
     const int64_t G = st::mlp_grid();
-    const int64_t decode = G * st::kMlpMaxBatchPerLaunch * H * 4;
+    int64_t decode = G * st::kMlpMaxBatchPerLaunch * H * 4;
+    if (B >= st::batch_min_rows() && B < st::kPrefillMinRows) {   // dtype is not known here: size for both paths
+        const int64_t batch = st::batch_workspace_bytes(H, n);
+        decode = batch > decode ? batch : decode;
+    }
     if (B < st::kPrefillMinRows) return decode;
     const int64_t prefill = st::prefill_workspace_bytes(B, H, n);
     return prefill > decode ? prefill : decode;
@@ -470,6 +482,10 @@ extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *g
     if (B >= kPrefillMinRows && dtype != ST_F32 && H % 128 == 0 && n >= 1)
         return launch_prefill(dtype, x, (int)B, (int)H, gate_rows, up_rows, down_rows, (int)n, n_dev, out, combined,
                               (long)ldc, workspace, act, has_gate ? 1 : 0, static_cast<hipStream_t>(stream));
+
+    if (B >= batch_min_rows() && batch_supported(dtype, (int)H))
+        return launch_batch(dtype, x, (int)B, (int)H, gate_rows, up_rows, down_rows, (int)n, n_dev, out, combined,
+                            (long)ldc, workspace, act, has_gate ? 1 : 0, static_cast<hipStream_t>(stream));
 
     MlpLaunch a;
     a.x = x; a.B = (int)B; a.H = (int)H;

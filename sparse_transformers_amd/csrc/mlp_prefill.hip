@@ -17,29 +17,9 @@
 // The reference only runs the sparse path for decode (src/modeling_skip.py:236);
 // this is the same contraction as sparse_mlp_forward_cpu
 // (sparse_transformers/csrc/sparse_mlp_op.cpp:151-161) for B > 1 rows.
-#include "st_common.h"
+#include "st_mfma.h"
 
 namespace st {
-
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-
-template <typename T> struct Mfma;
-template <> struct Mfma<f16_t> {
-    static __device__ __forceinline__ f32x4_t run(const uint4 &a, const uint4 &b, f32x4_t c)
-    {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b),
-                                                      c, 0, 0, 0);
-    }
-};
-template <> struct Mfma<bf16_t> {
-    static __device__ __forceinline__ f32x4_t run(const uint4 &a, const uint4 &b, f32x4_t c)
-    {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                       __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-    }
-};
 
 constexpr int kPfThreads = 256;
 constexpr int kPfBM = 128;   // rows of x per block
@@ -48,17 +28,6 @@ constexpr int kPfBK = 128;   // K per stage = 4 MFMA steps; 256 contiguous bytes
 constexpr int kPfKB = kPfBK / 32;
 constexpr int kPfCh = kPfBK / 8;   // 16-byte chunks per row and stage
 constexpr int kPfLd = kPfCh + 1;   // LDS row stride in 16-byte units (one pad chunk spreads the banks)
-
-__device__ __forceinline__ int device_count(int n_host, const int *n_dev)
-{
-    int n = n_host;
-    if (n_dev) {
-        const int nd = *n_dev;
-        n = nd < n ? nd : n;
-        if (n < 0) n = 0;
-    }
-    return n;
-}
 
 constexpr int kXcds = 8;
 

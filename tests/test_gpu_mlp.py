@@ -167,3 +167,59 @@ def test_prefill_agrees_with_decode_kernel():
     for b0 in range(0, 40, 8):
         small, _, _ = _run(x[b0:b0 + 8], cw, dn, "silu", True)
         assert_close(small.float().cpu().numpy(), big[b0:b0 + 8].float().cpu().numpy(), "float16", f"rows {b0}")
+
+
+# ---- MFMA batch kernels (3 <= B < 32, fp16 / bf16, H in {2048, 3072, 4096}) ----
+@pytest.mark.parametrize("name,B,H,n,dtype,act,has_gate", [
+    ("cfg3 batch 4", 4, 3072, 4620, "bfloat16", "silu", True),
+    ("cfg3 batch 16", 16, 3072, 7660, "bfloat16", "silu", True),
+    ("cfg4 batch 8", 8, 4096, 3584, "bfloat16", "silu", True),
+    ("cfg4 batch 4 fp16 ungated relu", 4, 4096, 1100, "float16", "relu", False),
+    ("two passes of 16 + ragged tail", 19, 2048, 1237, "float16", "gelu_pytorch_tanh", True),
+    ("31 rows, fewer active rows than blocks", 31, 3072, 97, "bfloat16", "sigmoid", True),
+    ("one active row", 5, 2048, 1, "float16", "silu", True),
+    ("33 rows per block (two tiles)", 3, 2048, 8450, "float16", "silu", False),
+])
+def test_batch_mfma_vs_oracle(name, B, H, n, dtype, act, has_gate):
+    x, cw, dn = _case(4242 + B + n, B, H, n, dtype, has_gate)
+    out, db, cb = _run(x, cw, dn, act, has_gate)
+    want, wantc = oracle.mlp_forward(x.float().numpy(), cw.float().numpy(), dn.float().numpy().T, act, has_gate)
+    assert tuple(out.shape) == (B, H) and tuple(cb.shape) == (B, cw.shape[0])
+    assert_close(out.float().cpu().numpy(), want, dtype, name)
+    assert_close(cb.float().cpu().numpy(), wantc, dtype, name + " combined")
+
+
+def test_batch_mfma_device_count_and_determinism():
+    """The batch kernels take the active count from device memory (rows past it may hold anything, here NaN),
+    and repeat bit-identically."""
+    B, H, I, n = 8, 3072, 2000, 1333
+    x, cw, dn = _case(99, B, H, I, "float16", True)
+    gate, up = cw[:I].clone(), cw[I:].clone()
+    gate[n:], up[n:], dn[n:] = float("nan"), float("nan"), float("nan")
+    xg, gg, ug, dg = x.to(DEV), gate.to(DEV), up.to(DEV), dn.to(DEV)
+    n_dev = torch.tensor([n], dtype=torch.int32, device=DEV)
+    outs = []
+    for _ in range(3):
+        out = torch.full((B, H), float("nan"), dtype=torch.float16, device=DEV)
+        mlp_forward_rows(xg, gg, ug, dg, I, n_dev, out, None, "silu", True)
+        torch.cuda.synchronize()
+        outs.append(out.cpu())
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    want, _ = oracle.mlp_forward(x.float().numpy(), torch.cat([gate[:n], up[:n]]).float().numpy(),
+                                 dn[:n].float().numpy().T, "silu", True)
+    assert_close(outs[0].float().numpy(), want, "float16", "device count")
+    # an empty active set gives zeros
+    n_dev.zero_()
+    out = torch.full((B, H), float("nan"), dtype=torch.float16, device=DEV)
+    mlp_forward_rows(xg, gg, ug, dg, I, n_dev, out, None, "silu", True)
+    torch.cuda.synchronize()
+    assert torch.count_nonzero(out).item() == 0
+
+
+def test_batch_mfma_agrees_with_streaming_kernel():
+    """Same inputs through the MFMA batch kernels (4 rows at once) and the streaming kernel (row by row)."""
+    H, n = 3072, 2867
+    x, cw, dn = _case(7, 4, H, n, "bfloat16", True)
+    out4, _, _ = _run(x, cw, dn, "silu", True)
+    ref = torch.cat([_run(x[i:i + 1], cw, dn, "silu", True)[0].clone() for i in range(4)]).float().cpu().numpy()
+    assert_close(out4.float().cpu().numpy(), ref, "bfloat16", "batch vs streaming")
