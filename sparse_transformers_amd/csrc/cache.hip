@@ -139,14 +139,17 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     const bool writer = blockIdx.x == 0;
 
     int n;
+    // VEC: new / current mask words as 0x01 bytes, kept in registers for the diff and for publishing
+    uint64_t w_new[kPlanMaxWords], w_cur[kPlanMaxWords];
     if constexpr (VEC) {
         n = ep ? n_both[1] : n_both[0];
 #pragma unroll
         for (int w = 0; w < kPlanMaxWords; ++w) {
             const int e = e0 + 8 * w;
+            w_new[w] = w_cur[w] = 0;
             if (e < e1) {
-                const uint64_t nw = nonzero_bytes(v_new[w]), cw = nonzero_bytes(ep ? v_cur[1][w] : v_cur[0][w]);
-                *reinterpret_cast<uint64_t *>(flag_l + e) = nw | (cw << 1);
+                w_new[w] = nonzero_bytes(v_new[w]);
+                w_cur[w] = nonzero_bytes(ep ? v_cur[1][w] : v_cur[0][w]);
                 const int4 a = ep ? v_idx[1][w][0] : v_idx[0][w][0], b4 = ep ? v_idx[1][w][1] : v_idx[0][w][1];
                 uint4 packed;
                 packed.x = (uint32_t)(a.x & 0xffff) | ((uint32_t)a.y << 16);
@@ -174,10 +177,16 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
 
     // ---- diff: contiguous element range per thread keeps the lists ascending
     uint32_t cnt = 0;  // added in the low half, removed in the high half
-    for (int i = e0; i < e1; ++i) {
-        const uint8_t f = flag_l[i];
-        cnt += (f == 1) ? 1u : 0u;
-        cnt += (f == 2) ? 0x10000u : 0u;
+    if constexpr (VEC) {
+#pragma unroll
+        for (int w = 0; w < kPlanMaxWords; ++w)
+            cnt += (uint32_t)__popcll(w_new[w] & ~w_cur[w]) + ((uint32_t)__popcll(w_cur[w] & ~w_new[w]) << 16);
+    } else {
+        for (int i = e0; i < e1; ++i) {
+            const uint8_t f = flag_l[i];
+            cnt += (f == 1) ? 1u : 0u;
+            cnt += (f == 2) ? 0x10000u : 0u;
+        }
     }
     uint32_t total;
     const uint32_t off = block_excl_scan<TPB / kWave>(cnt, wave_tot, &total);  // contains __syncthreads
@@ -196,10 +205,26 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     }
     {
         int oa = (int)(off & 0xffffu), orr = (int)(off >> 16);
-        for (int i = e0; i < e1; ++i) {
-            const uint8_t f = flag_l[i];
-            if (f == 1) lists[oa++] = (uint16_t)i;
-            if (f == 2) lists[I - 1 - (orr++)] = (uint16_t)i;
+        if constexpr (VEC) {
+#pragma unroll
+            for (int w = 0; w < kPlanMaxWords; ++w) {
+                const int e = e0 + 8 * w;
+                uint64_t a = w_new[w] & ~w_cur[w], r = w_cur[w] & ~w_new[w];   // one 0x01 byte per element, ascending
+                while (a) {
+                    lists[oa++] = (uint16_t)(e + ((__ffsll((long long)a) - 1) >> 3));
+                    a &= a - 1;
+                }
+                while (r) {
+                    lists[I - 1 - (orr++)] = (uint16_t)(e + ((__ffsll((long long)r) - 1) >> 3));
+                    r &= r - 1;
+                }
+            }
+        } else {
+            for (int i = e0; i < e1; ++i) {
+                const uint8_t f = flag_l[i];
+                if (f == 1) lists[oa++] = (uint16_t)i;
+                if (f == 2) lists[I - 1 - (orr++)] = (uint16_t)i;
+            }
         }
     }
     __syncthreads();
@@ -288,9 +313,13 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
         const int nmat = cp.nmat, row_bytes = cp.row_bytes, chunks = row_bytes >> 4;
         const int GS = 1 << gs_log2, ngrp = TPB >> gs_log2;
         const int grp = tid >> gs_log2, cc = tid & (GS - 1);
-        const int slots = gridDim.x * ngrp, slot = blockIdx.x * ngrp + grp;
+        // the publishing block takes no copies when there are others to do them
+        const bool solo = gridDim.x == 1;
+        const bool copies = solo || !writer;
+        const int slots = (solo ? 1 : (int)gridDim.x - 1) * ngrp;
+        const int slot = (solo ? 0 : (int)blockIdx.x - 1) * ngrp + grp;   // >= 0 whenever `copies`
         const int work = (int)n_changed * nmat;
-        for (int w0 = slot; w0 < work; w0 += slots * kCopyUnroll) {
+        for (int w0 = copies ? slot : work; w0 < work; w0 += slots * kCopyUnroll) {
             for (int c = cc; c < chunks; c += GS) {
                 uint4 v[kCopyUnroll];
                 unsigned char *dst[kCopyUnroll];
@@ -323,7 +352,15 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
         uint8_t *mask_out = cur_mask2 + (size_t)(ep ^ 1) * I;
         for (int p = tid; p < n_new; p += TPB) idx_out[p] = idx_l[p];
         // the reference stores the new mask only when the rebuild did not throw (n_new > 0)
-        for (int i = tid; i < I; i += TPB) mask_out[i] = n_new > 0 ? (flag_l[i] & 1) : (flag_l[i] >> 1);
+        if constexpr (VEC) {
+#pragma unroll
+            for (int w = 0; w < kPlanMaxWords; ++w) {
+                const int e = e0 + 8 * w;
+                if (e < e1) *reinterpret_cast<uint64_t *>(mask_out + e) = n_new > 0 ? w_new[w] : w_cur[w];
+            }
+        } else {
+            for (int i = tid; i < I; i += TPB) mask_out[i] = n_new > 0 ? (flag_l[i] & 1) : (flag_l[i] >> 1);
+        }
         if (tid == 0) {
             state[ST_STATE_N_BUF0 + (ep ^ 1)] = n_new;
             state[ST_STATE_N_ACTIVE] = n_new;
