@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of mlp_decode_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by
 # what the same counter reads for a 256 MiB copy; see profiles/mlp_decode_traffic_llama3b_stack_fp16.md
-MEASURED_TRAFFIC_BYTES = {"llama3b_stack_fp16": 53_040_000 + 3_145_728}
+MEASURED_TRAFFIC_BYTES = {("llama3b_stack_fp16", "mlp_decode"): 53_040_000 + 3_145_728}
 
 
 def parse_args():
@@ -42,6 +42,8 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--overlap", action="store_true",
                     help="run predictor/cache update on a side stream (measured slower inside a graph; off by default)")
+    ap.add_argument("--no-fused", action="store_true",
+                    help="cache update and MLP as two kernels per layer instead of the fused update+decode kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=2)
     ap.add_argument("--cpu-steps", type=int, default=24)
@@ -174,7 +176,7 @@ def main():
         assert layer.cache.get_num_active() == n
 
     use_graph = not args.no_graph
-    stack.prepare(B, overlap=args.overlap)
+    stack.prepare(B, overlap=args.overlap, fused=not args.no_fused)
     if use_graph:
         stack.step_staged(x_in[0], x_pred[0], trace[0])     # first launches outside capture
         torch.cuda.synchronize()
@@ -222,26 +224,48 @@ def main():
     # (Events recorded inside a captured graph cannot be read back with hipEventElapsedTime on this ROCm, so
     # this pass launches eagerly; the GPU idles between launches and the events bracket dispatch overhead,
     # which makes these durations about 2 us longer than rocprofv3's kernel times - see profiles/.)
-    for t in range(W + K - 1, W + K - 1 - P, -1):
+    def summarise():
+        kinds_np, ms_np = np.concatenate(kinds_all), np.concatenate(ms_all)
+        out = {}
+        for k, name in enumerate(_lib.KERNEL_KINDS):
+            sel = ms_np[kinds_np == k]
+            if sel.size:
+                out[name] = {"launches": int(sel.size), "mean_us": round(float(sel.mean()) * 1e3, 3),
+                             "median_us": round(float(np.median(sel)) * 1e3, 3),
+                             "p10_us": round(float(np.percentile(sel, 10)) * 1e3, 3),
+                             "p90_us": round(float(np.percentile(sel, 90)) * 1e3, 3)}
+        kinds_all.clear()
+        ms_all.clear()
+        return out
+
+    t_lo = W + K - 1 - P
+    for t in range(W + K - 1, t_lo, -1):
         _lib.check(L.st_profile_enable(per_step), "st_profile_enable")
         stack.step_staged(x_in[t], x_pred[t], trace[t], replay=False)
         torch.cuda.synchronize()
         collect()
+    per_kernel = summarise()
+    # the cache update on its own (it has no kernel of its own in the fused path): a few more steps, forwards again
+    unfused = None
+    if stack.fused:
+        stack.fused = False
+        for t in range(t_lo + 2, min(t_lo + 2 + max(4, P // 4), W + K)):
+            _lib.check(L.st_profile_enable(per_step), "st_profile_enable")
+            stack.step_staged(x_in[t], x_pred[t], trace[t], replay=False)
+            torch.cuda.synchronize()
+            collect()
+        unfused = summarise()
+        stack.fused = True
     L.st_profile_disable()
-    kinds_np, ms_np = np.concatenate(kinds_all), np.concatenate(ms_all)
-    per_kernel = {}
-    for k, name in enumerate(_lib.KERNEL_KINDS):
-        sel = ms_np[kinds_np == k]
-        if sel.size:
-            per_kernel[name] = {"launches": int(sel.size), "mean_us": round(float(sel.mean()) * 1e3, 3),
-                                "median_us": round(float(np.median(sel)) * 1e3, 3),
-                                "p10_us": round(float(np.percentile(sel, 10)) * 1e3, 3),
-                                "p90_us": round(float(np.percentile(sel, 90)) * 1e3, 3)}
     mats = 3 if wl.has_gate else 2
     alg_bytes = mats * n * H * esz                      # active-weight bytes one launch streams
-    mlp_us = per_kernel["mlp_decode"]["mean_us"]
+    dom = "cache_update_decode" if "cache_update_decode" in per_kernel else \
+          ("mlp_decode" if "mlp_decode" in per_kernel else "mlp_batch_gateup")
+    mlp_us = per_kernel[dom]["mean_us"]
+    if dom == "mlp_batch_gateup":                        # the batch path streams the weights in two kernels
+        mlp_us += per_kernel["mlp_batch_down"]["mean_us"]
     achieved = alg_bytes / (mlp_us * 1e-6) / 1e9
-    upd_us = per_kernel["cache_update"]["mean_us"]
+    upd_us = (unfused or per_kernel).get("cache_update", {}).get("mean_us")
 
     churn_mean = 0.5 * (wl.churn_lo + wl.churn_hi)
     result = {
@@ -253,16 +277,19 @@ def main():
                    "batch": B, "act": wl.act, "has_gate": wl.has_gate, "n_active": n,
                    "churn": [wl.churn_lo, wl.churn_hi], "mask_source": "trace",
                    "launch": "hip_graph" if use_graph else "eager",
-                   "streams": 2 if args.overlap else 1,
+                   "streams": 2 if args.overlap else 1, "update_fused_into_decode": bool(stack.fused),
                    "kernel_timing": "hip events, eager second pass"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name), "kernel": "mlp_decode_kernel",
-                     "bytes_per_launch": alg_bytes, "mean_us": mlp_us},
-        "cache_update_us_per_layer": round(upd_us, 3),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((wl.name, dom)) if B == wl.batch else None,
+                     "kernel": dom + "_kernel", "bytes_per_launch": alg_bytes, "mean_us": mlp_us},
+        "cache_update_us_per_layer": upd_us,
+        "cache_update_note": ("standalone cache_update_kernel, measured in a short unfused pass; the timed path "
+                              "runs it fused into the decode kernel") if unfused else "standalone kernel",
         "stack_hbm_gbps": round(layers * alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
         "host_wall_ms_per_step": round(host_s * 1e3 / K, 5),
         "kernels_us": per_kernel,
+        "kernels_us_unfused": unfused,
         "churn_mean": churn_mean,
     }
     if not args.no_cpu_baseline:

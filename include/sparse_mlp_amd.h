@@ -165,6 +165,22 @@ int st_cache_update_async(st_cache *c, const uint8_t *mask, void *stream);
  * state_out: host int32[ST_STATE_WORDS], may be NULL. */
 int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream);
 
+/* update_active_weights(mask) immediately followed by the sparse MLP on the
+ * updated cache -- weight_cache.h:229-359 then sparse_mlp_op.cpp:53-192 /
+ * src/modeling_skip.py:114-117, i.e. what SkipDecoderLayer.forward does per
+ * layer (src/modeling_skip.py:234-261) -- enqueued as one call.  For B == 1
+ * (16-byte aligned rows, 8-byte aligned mask, I % 8 == 0) this is ONE kernel
+ * that replays the bookkeeping and streams the active rows, taking rows whose
+ * index changed from the pool and writing them back on the way; otherwise it
+ * is st_cache_update_async followed by st_mlp_forward.  Either way the cache
+ * ends in the same state and `out` holds the same bits as the two separate
+ * calls.  x, out: [B,H] in the cache's dtype; combined: [B,ldc] or NULL;
+ * workspace: st_mlp_workspace_bytes(B, H, I) bytes.  An update that empties
+ * the cache leaves status ST_ERR_NO_ACTIVE in the state words (reported by
+ * st_cache_sync_state) and zeros in `out`. */
+int st_cache_update_forward(st_cache *c, const uint8_t *mask, const void *x, int64_t B, void *out, void *combined,
+                            int64_t ldc, void *workspace, int64_t workspace_bytes, int act, void *stream);
+
 /* get_concat_weight(): weight_cache.h:113-145,362-366.  Writes the contiguous
  * [2n,H] (gate rows then up rows; [n,H] when ungated) tensor into dst, for
  * callers that need the reference's tensor; n is the host's count from the
@@ -191,7 +207,8 @@ typedef enum st_kernel_kind {
     ST_K_MLP_PREFILL_DOWN = 7,
     ST_K_MLP_BATCH_GATEUP = 8,
     ST_K_MLP_BATCH_DOWN = 9,
-    ST_K_KINDS = 10
+    ST_K_CACHE_UPDATE_DECODE = 10,
+    ST_K_KINDS = 11
 } st_kernel_kind;
 
 int st_profile_enable(int max_samples); /* host; allocates the event pool */

@@ -46,6 +46,7 @@ SIGNATURES = {
     "st_cache_destroy": (None, [_vp]),
     "st_cache_load_weights": (_ci, [_vp, _vp, _vp, _vp, _vp]),
     "st_cache_update_async": (_ci, [_vp, _vp, _vp]),
+    "st_cache_update_forward": (_ci, [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _ci, _vp]),
     "st_cache_sync_state": (_ci, [_vp, _vp, _vp]),
     "st_cache_materialize_concat": (_ci, [_vp, _vp, _i64, _vp]),
     "st_profile_enable": (_ci, [_ci]),
@@ -54,7 +55,8 @@ SIGNATURES = {
 }
 
 KERNEL_KINDS = ["mlp_decode", "mlp_reduce", "cache_update", "reserved", "pred_down", "pred_up_mask",
-                "mlp_prefill_gateup", "mlp_prefill_down", "mlp_batch_gateup", "mlp_batch_down"]
+                "mlp_prefill_gateup", "mlp_prefill_down", "mlp_batch_gateup", "mlp_batch_down",
+                "cache_update_decode"]
 
 _lib = None
 

@@ -80,16 +80,36 @@ __device__ __forceinline__ uint64_t nonzero_bytes(uint64_t x)
     return x & 0x0101010101010101ull;
 }
 
-// VEC: I % 8 == 0 and the mask is 8-byte aligned, so masks are read as 8-byte
-// words and indices as 16-byte vectors; both bookkeeping buffers are requested
-// together with the ticket, so the kernel front costs one memory round trip.
-template <bool VEC, int TPB>
-__global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const uint8_t *__restrict__ new_mask,
-                                                                    uint8_t *__restrict__ cur_mask2,
-                                                                    int32_t *__restrict__ indices2,
-                                                                    int32_t *__restrict__ state, int I, int gs_log2)
+// The plan as every block computes it, and the LDS arrays that hold it.
+struct PlanView {
+    uint16_t *pos_l;    // index -> position (kNone when absent)
+    uint16_t *idx_l;    // position -> index, after the update
+    uint16_t *lists;    // positions to rewrite: [0, n_changed)
+    uint32_t *dirty;    // bit per position whose index changed (complete only with MARK, or on the slow path)
+    int ep;             // bookkeeping buffer this launch read
+    bool last_arrival;  // this block took the last ticket
+    bool writer;        // this block publishes
+    bool changed;       // false: the mask equals the remembered one, nothing was touched
+    int n_old, n_new, na, nr;
+    uint32_t n_changed;
+};
+
+constexpr size_t plan_lds_bytes(int I)
 {
-    extern __shared__ __align__(16) unsigned char smem[];
+    return (size_t)I * 6 + (size_t)(I & 1) * 2 + (size_t)((((I + 31) >> 5) + 1) & ~1) * 4 + (size_t)I + 16;
+}
+
+// Replays the bookkeeping of one update in LDS and publishes it (block 0 writes the other bookkeeping
+// buffer, the last block to arrive flips the epoch).  Called by all threads of the block; contains
+// barriers.  VEC: I % 8 == 0 and the mask is 8-byte aligned, so masks are read as 8-byte words and
+// indices as 16-byte vectors; both bookkeeping buffers are requested together with the ticket, so the
+// front costs one memory round trip.  MARK: the dirty bitmap is kept on the fast path too.
+// `after_issue` runs right after the front loads have been issued (a place to start other loads).
+template <bool VEC, int TPB, bool MARK, typename F>
+__device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, const uint8_t *__restrict__ new_mask,
+                                           uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
+                                           int32_t *__restrict__ state, int I, F after_issue)
+{
     uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);  // index -> position
     uint16_t *idx_l = pos_l + I;                           // position -> index
     // added indices ascending from the front, removed indices ascending from the
@@ -102,6 +122,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     __shared__ uint32_t wave_tot[(TPB / kWave)];
     __shared__ int n_new_s;
     __shared__ uint32_t ticket_s;
+    pv.pos_l = pos_l; pv.idx_l = idx_l; pv.lists = lists; pv.dirty = dirty;
 
     const int tid = threadIdx.x;
     ST_TL(0);
@@ -131,12 +152,14 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     }
     // One atomic returns both the epoch (which buffer to read) and this block's ticket.
     if (tid == 0) ticket_s = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
+    after_issue();
     for (int w = tid; w < dirty_words; w += TPB) dirty[w] = 0u;
     __syncthreads();
     const uint32_t ticket = ticket_s;
     const int ep = (int)((ticket >> 16) & 1u);
     const bool last_arrival = (ticket & 0xffffu) == gridDim.x - 1;
     const bool writer = blockIdx.x == 0;
+    pv.ep = ep; pv.last_arrival = last_arrival; pv.writer = writer;
 
     int n;
     // VEC: new / current mask words as 0x01 bytes, kept in registers for the diff and for publishing
@@ -201,6 +224,8 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
                 state[ST_STATE_N_REMOVED] = 0;
             }
         }
+        pv.changed = false;
+        pv.n_old = pv.n_new = n; pv.na = pv.nr = 0; pv.n_changed = 0;
         return;
     }
     {
@@ -242,7 +267,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
             idx_l[p] = (uint16_t)a;
             pos_l[a] = p;
             pos_l[e] = kNone;
-            if (!fast) atomicOr(&dirty[p >> 5], 1u << (p & 31));
+            if (MARK || !fast) atomicOr(&dirty[p >> 5], 1u << (p & 31));
         }
         if (fast) lists[i] = p;
     }
@@ -308,6 +333,59 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     }
 
     ST_TL(5);
+    // ---- publish: one block writes the other bookkeeping buffer, the last arrival flips the epoch
+    if (writer) {
+        int32_t *idx_out = indices2 + (size_t)(ep ^ 1) * I;
+        uint8_t *mask_out = cur_mask2 + (size_t)(ep ^ 1) * I;
+        for (int p = tid; p < n_new; p += TPB) idx_out[p] = idx_l[p];
+        // the reference stores the new mask only when the rebuild did not throw (n_new > 0)
+        if constexpr (VEC) {
+#pragma unroll
+            for (int w = 0; w < kPlanMaxWords; ++w) {
+                const int e = e0 + 8 * w;
+                if (e < e1) *reinterpret_cast<uint64_t *>(mask_out + e) = n_new > 0 ? w_new[w] : w_cur[w];
+            }
+        } else {
+            for (int i = tid; i < I; i += TPB) mask_out[i] = n_new > 0 ? (flag_l[i] & 1) : (flag_l[i] >> 1);
+        }
+        if (tid == 0) {
+            state[ST_STATE_N_BUF0 + (ep ^ 1)] = n_new;
+            state[ST_STATE_N_ACTIVE] = n_new;
+            state[ST_STATE_N_CHANGED] = (int)n_changed;
+            state[ST_STATE_N_ADDED] = na;
+            state[ST_STATE_N_REMOVED] = nr;
+            state[ST_STATE_SERIAL] += 1;
+            state[ST_STATE_EPOCH] = ep ^ 1;
+            if (n_new > 0) {
+                state[ST_STATE_STATUS] = 0;
+                state[ST_STATE_VALID] = 1;
+            } else {
+                state[ST_STATE_STATUS] = ST_ERR_NO_ACTIVE;
+            }
+        }
+    }
+    if (last_arrival && tid == 0)
+        atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)(ep ^ 1) << 16);
+    pv.changed = true;
+    pv.n_old = n; pv.n_new = n_new; pv.na = na; pv.nr = nr; pv.n_changed = n_changed;
+}
+
+
+// update = plan + this block's share of the row copies
+template <bool VEC, int TPB>
+__global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const uint8_t *__restrict__ new_mask,
+                                                                    uint8_t *__restrict__ cur_mask2,
+                                                                    int32_t *__restrict__ indices2,
+                                                                    int32_t *__restrict__ state, int I, int gs_log2)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x;
+    PlanView pv;
+    cache_plan<VEC, TPB, false>(pv, smem, new_mask, cur_mask2, indices2, state, I, [] {});
+    if (!pv.changed) return;
+    const uint16_t *lists = pv.lists, *idx_l = pv.idx_l;
+    const uint32_t n_changed = pv.n_changed;
+    const bool writer = pv.writer;
     // ---- copy this block's share of the changed rows: active[m][p] <- pool[m][index at p]
     {
         const int nmat = cp.nmat, row_bytes = cp.row_bytes, chunks = row_bytes >> 4;
@@ -346,40 +424,166 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     }
 
     ST_TL(6);
-    // ---- publish: one block writes the other bookkeeping buffer, the last arrival flips the epoch
-    if (writer) {
-        int32_t *idx_out = indices2 + (size_t)(ep ^ 1) * I;
-        uint8_t *mask_out = cur_mask2 + (size_t)(ep ^ 1) * I;
-        for (int p = tid; p < n_new; p += TPB) idx_out[p] = idx_l[p];
-        // the reference stores the new mask only when the rebuild did not throw (n_new > 0)
-        if constexpr (VEC) {
+}
+
+// ---------------------------------------------------------------------------
+// update + sparse MLP for one row of x in ONE kernel.
+//
+// Every block replays the plan (as above) and then streams its share of the
+// active rows exactly like mlp_decode_kernel does -- except that a position
+// whose index changed is read from the POOL row of its new index instead of
+// the active buffer, and written back to the active buffer from the registers
+// it already sits in.  The separate copy pass, its launch and its memory round
+// trips disappear; the cache ends in the same state as after
+// cache_update_kernel, and the arithmetic (row -> block dealing, summation
+// order) is that of mlp_decode_kernel, so the result is bit-identical to
+// update followed by forward.
+// Rows are dealt to blocks round-robin: row(bat, k) = blk + G * (grp + ngrp * (bat * RB + k)).
+// ---------------------------------------------------------------------------
+template <typename T, int RB, int TPB>
+__global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
+    CopyPlan cp, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
+    int32_t *__restrict__ state, int I, const T *__restrict__ x, int H, T *__restrict__ combined, long ldc,
+    float *__restrict__ partials, int act, int gs_log2, int plan_bytes)
+{
+    constexpr int VEC = Elem<T>::kVec;
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float red[TPB / kWave][RB][2];  // per-wave partial (g,u)
+    __shared__ float hs[TPB / kWave][RB];      // h of the rows being computed
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int G = gridDim.x, blk = blockIdx.x;
+    const int chunks = H / VEC;
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+    const int GS = 1 << gs_log2, ngrp = TPB >> gs_log2, wpg = GS >> 6;
+    const int grp = tid >> gs_log2, cc = tid & (GS - 1);
+    const bool valid = cc < chunks;
+    const size_t coff = valid ? (size_t)cc * 16 : 0;   // byte offset of this thread's chunk (clamped)
+    const bool wave_live = __builtin_amdgcn_readfirstlane(cc & ~(kWave - 1)) < chunks;
+    const bool has_gate = cp.nmat == 3;
+    const int iu = has_gate ? 1 : 0, id = iu + 1;
+    const int row_bytes = cp.row_bytes;
+
+    uint4 xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff);
+    if (!valid) xr = zero4;
+
+    PlanView pv;
+    cache_plan<true, TPB, true>(pv, smem, new_mask, cur_mask2, indices2, state, I, [] {});
+    const int n = pv.n_new, n_old = pv.n_old;
+
+    auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
+
+    float acc[VEC];
 #pragma unroll
-            for (int w = 0; w < kPlanMaxWords; ++w) {
-                const int e = e0 + 8 * w;
-                if (e < e1) *reinterpret_cast<uint64_t *>(mask_out + e) = n_new > 0 ? w_new[w] : w_cur[w];
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+
+    const int jcount = n > blk ? (n - blk + G - 1) / G : 0;      // rows of this block
+    const int nbat = ((jcount + ngrp - 1) / ngrp + RB - 1) / RB;  // uniform over the block
+    for (int bat = 0; bat < nbat; ++bat) {
+        uint4 wg[RB], wu[RB], wd[RB];
+        bool fresh[RB];   // row comes from the pool and has to be written back
+        if (wave_live) {
+#pragma unroll
+            for (int k = 0; k < RB; ++k) {
+                const int p = row_of(bat, k);
+                const bool ok = p < n;
+                const int pc = ok ? p : n - 1;   // clamped; rows past the count are neutralised below
+                const bool moved = pc >= n_old || ((pv.dirty[pc >> 5] >> (pc & 31)) & 1u);
+                fresh[k] = ok && moved && pv.changed;
+                const size_t ro = (size_t)(fresh[k] ? (int)pv.idx_l[pc] : pc) * row_bytes + coff;
+                wu[k] = ld16_stream((fresh[k] ? cp.pool[iu] : cp.active[iu]) + ro);
+                wd[k] = ld16_stream((fresh[k] ? cp.pool[id] : cp.active[id]) + ro);
+                wg[k] = has_gate ? ld16_stream((fresh[k] ? cp.pool[0] : cp.active[0]) + ro) : zero4;
             }
         } else {
-            for (int i = tid; i < I; i += TPB) mask_out[i] = n_new > 0 ? (flag_l[i] & 1) : (flag_l[i] >> 1);
+#pragma unroll
+            for (int k = 0; k < RB; ++k) { wg[k] = wu[k] = wd[k] = zero4; fresh[k] = false; }
         }
-        if (tid == 0) {
-            state[ST_STATE_N_BUF0 + (ep ^ 1)] = n_new;
-            state[ST_STATE_N_ACTIVE] = n_new;
-            state[ST_STATE_N_CHANGED] = (int)n_changed;
-            state[ST_STATE_N_ADDED] = na;
-            state[ST_STATE_N_REMOVED] = nr;
-            state[ST_STATE_SERIAL] += 1;
-            state[ST_STATE_EPOCH] = ep ^ 1;
-            if (n_new > 0) {
-                state[ST_STATE_STATUS] = 0;
-                state[ST_STATE_VALID] = 1;
-            } else {
-                state[ST_STATE_STATUS] = ST_ERR_NO_ACTIVE;
+
+        // ---- phase 1: partial dot products on this thread's chunk
+        float fx[VEC];
+        unpack<T>(xr, fx);
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+            float fg[VEC], fu[VEC], pg = 0.f, pu = 0.f;
+            unpack<T>(wg[k], fg);
+            unpack<T>(wu[k], fu);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                pg = fmaf(fg[e], fx[e], pg);
+                pu = fmaf(fu[e], fx[e], pu);
+            }
+            const float sg = wave_sum_dpp(pg), su = wave_sum_dpp(pu);
+            if (lane == 0) {
+                red[wave][k][0] = sg;
+                red[wave][k][1] = su;
             }
         }
+        // write the fresh rows back while the reductions settle
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+            if (fresh[k] && valid) {
+                const size_t ro = (size_t)row_of(bat, k) * row_bytes + coff;
+                st16(cp.active[iu] + ro, wu[k]);
+                st16(cp.active[id] + ro, wd[k]);
+                if (has_gate) st16(cp.active[0] + ro, wg[k]);
+            }
+        }
+        __syncthreads();
+        if (tid < ngrp * RB) {
+            const int g_ = tid / RB, k_ = tid - g_ * RB;
+            const int row = blk + G * (g_ + ngrp * (bat * RB + k_));
+            float sg = 0.f, su = 0.f;
+            for (int wv = g_ * wpg; wv < (g_ + 1) * wpg; ++wv) {
+                sg += red[wv][k_][0];
+                su += red[wv][k_][1];
+            }
+            const float hv = has_gate ? activate(sg, act) * su : activate(su, act);
+            const bool ok = row < n;
+            hs[g_][k_] = ok ? hv : 0.f;
+            if (ok && combined) {
+                combined[row] = from_float<T>(hv);
+                if (has_gate) combined[n + row] = from_float<T>(su);
+            }
+        }
+        __syncthreads();
+        // ---- phase 2: down projection from the rows already in registers
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+            const bool row_ok = row_of(bat, k) < n;
+            float fw[VEC];
+            unpack<T>(row_ok ? wd[k] : zero4, fw);
+            const float hv = hs[grp][k];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] = fmaf(hv, fw[e], acc[e]);
+        }
     }
-    if (last_arrival && tid == 0)
-        atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)(ep ^ 1) << 16);
-    ST_TL(7);
+
+    // ---- combine the thread groups through LDS (behind the plan arrays), one fp32 partial row per block
+    if (ngrp > 1) {
+        float *redc = reinterpret_cast<float *>(smem + plan_bytes);  // [ngrp-1][H]
+        if (grp > 0 && valid) {
+#pragma unroll
+            for (int e = 0; e < VEC; e += 4)
+                *reinterpret_cast<float4 *>(redc + (size_t)(grp - 1) * H + (size_t)cc * VEC + e) =
+                    make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
+        }
+        __syncthreads();
+        if (grp == 0 && valid) {
+            for (int gq = 1; gq < ngrp; ++gq)
+#pragma unroll
+                for (int e = 0; e < VEC; e += 4) {
+                    const float4 v = *reinterpret_cast<const float4 *>(redc + (size_t)(gq - 1) * H + (size_t)cc * VEC + e);
+                    acc[e] += v.x; acc[e + 1] += v.y; acc[e + 2] += v.z; acc[e + 3] += v.w;
+                }
+        }
+    }
+    if (grp == 0 && valid) {
+#pragma unroll
+        for (int e = 0; e < VEC; e += 4)
+            *reinterpret_cast<float4 *>(partials + (size_t)blk * H + (size_t)cc * VEC + e) =
+                make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
+    }
 }
 
 // in [R,C] -> out [C,R], 64x64 tiles through LDS.
@@ -487,7 +691,7 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     ST_REQUIRE(c && mask, "st_cache_update_async: null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int I = (int)c->I;
-    const size_t lds = (size_t)I * 6 + (I & 1) * 2 + (size_t)((((I + 31) >> 5) + 1) & ~1) * 4 + (size_t)I + 16;
+    const size_t lds = plan_lds_bytes(I);
     CopyPlan cp;
     cp.nmat = 0;
     if (c->has_gate) {
@@ -541,6 +745,82 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     }
     ST_HIP(hipGetLastError());
     return ST_OK;
+}
+
+extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const void *x, int64_t B, void *out,
+                                       void *combined, int64_t ldc, void *workspace, int64_t workspace_bytes, int act,
+                                       void *stream)
+{
+    using namespace st;
+    ST_REQUIRE(c && mask && x && out && workspace, "st_cache_update_forward: null pointer");
+    ST_REQUIRE(B >= 1 && B <= 4096, "st_cache_update_forward: B=%lld out of range [1,4096]", (long long)B);
+    ST_REQUIRE(act >= ST_ACT_RELU && act <= ST_ACT_IDENTITY, "st_cache_update_forward: unknown activation %d", act);
+    ST_REQUIRE(workspace_bytes >= st_mlp_workspace_bytes(B, c->H, c->I),
+               "st_cache_update_forward: workspace too small (%lld < %lld)", (long long)workspace_bytes,
+               (long long)st_mlp_workspace_bytes(B, c->H, c->I));
+    ST_REQUIRE((((uintptr_t)x | (uintptr_t)workspace) & 15) == 0, "st_cache_update_forward: pointers must be 16-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int I = (int)c->I, H = (int)c->H;
+    const int row_bytes = (int)(c->H * c->esz), chunks = row_bytes >> 4;
+    constexpr int TPB = 1024, RB = 6;
+    int gs_log2 = 6;
+    while ((1 << gs_log2) < chunks && (1 << gs_log2) < TPB) ++gs_log2;
+    const int ngrp = TPB >> gs_log2;
+    const size_t plan_bytes = (plan_lds_bytes(I) + 15) & ~(size_t)15;
+    const size_t lds = plan_bytes + (size_t)(ngrp - 1) * H * 4;
+    const bool aligned = (I % 8 == 0) && ((uintptr_t)mask % 8 == 0) && ((uintptr_t)c->b.cur_mask % 8 == 0) &&
+                         ((uintptr_t)c->b.indices % 16 == 0);
+    static const bool fused_off = [] { const char *v = getenv("ST_CACHE_FUSED"); return v && atoi(v) == 0; }();
+    const bool fused = !fused_off && B == 1 && aligned && I <= 8 * TPB * kPlanMaxWords && chunks <= TPB &&
+                       row_bytes % 16 == 0 && lds <= (size_t)(156 * 1024);
+    if (!fused) {   // two launches: update, then the forward that reads the count on the device
+        const int rc = st_cache_update_async(c, mask, stream);
+        if (rc != ST_OK) return rc;
+        return st_mlp_forward(x, B, c->H, c->b.gate_active, c->b.up_active, c->b.down_active, c->I,
+                              c->b.state + ST_STATE_N_ACTIVE, 0, out, combined, ldc, workspace, workspace_bytes, act,
+                              c->dtype, c->has_gate, stream);
+    }
+    CopyPlan cp;
+    cp.nmat = 0;
+    if (c->has_gate) {
+        cp.pool[cp.nmat] = static_cast<const unsigned char *>(c->b.gate_pool);
+        cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.gate_active);
+    }
+    cp.pool[cp.nmat] = static_cast<const unsigned char *>(c->b.up_pool);
+    cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.up_active);
+    cp.pool[cp.nmat] = static_cast<const unsigned char *>(c->b.downT_pool);
+    cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.down_active);
+    for (int k = cp.nmat; k < 3; ++k) { cp.pool[k] = cp.pool[0]; cp.active[k] = cp.active[0]; }
+    cp.row_bytes = row_bytes;
+    const int G = mlp_grid();
+    float *partials = static_cast<float *>(workspace);
+    {
+        ProfScope ps(ST_K_CACHE_UPDATE_DECODE, s);
+        auto launch = [&](auto kern, auto *xt, auto *ct) -> int {
+            static bool attr_set = false;
+            if (!attr_set) {
+                ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+                attr_set = true;
+            }
+            hipLaunchKernelGGL(kern, dim3(G), dim3(TPB), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state, I,
+                               xt, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes);
+            return ST_OK;
+        };
+        int rc;
+        if (c->dtype == ST_F32)
+            rc = launch(cache_update_decode_kernel<float, RB, TPB>, static_cast<const float *>(x),
+                        static_cast<float *>(combined));
+        else if (c->dtype == ST_F16)
+            rc = launch(cache_update_decode_kernel<f16_t, RB, TPB>, static_cast<const f16_t *>(x),
+                        static_cast<f16_t *>(combined));
+        else
+            rc = launch(cache_update_decode_kernel<bf16_t, RB, TPB>, static_cast<const bf16_t *>(x),
+                        static_cast<bf16_t *>(combined));
+        if (rc != ST_OK) return rc;
+    }
+    ST_HIP(hipGetLastError());
+    return launch_mlp_reduce(c->dtype, partials, G, 1, 1, H, out, s);
 }
 
 extern "C" int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream)

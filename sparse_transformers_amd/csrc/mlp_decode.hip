@@ -442,6 +442,24 @@ int mlp_grid()
     return device_cu_count() * mult;
 }
 
+int launch_mlp_reduce(int dtype, const float *partials, int G, int NB, int bcount, int H, void *out,
+                      hipStream_t stream)
+{
+    ProfScope ps(ST_K_MLP_REDUCE, stream);
+    const dim3 grid((H + 63) / 64, bcount);
+    if (dtype == ST_F32)
+        hipLaunchKernelGGL(mlp_reduce_kernel<float>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+                           static_cast<float *>(out));
+    else if (dtype == ST_F16)
+        hipLaunchKernelGGL(mlp_reduce_kernel<f16_t>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+                           static_cast<f16_t *>(out));
+    else
+        hipLaunchKernelGGL(mlp_reduce_kernel<bf16_t>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+                           static_cast<bf16_t *>(out));
+    ST_HIP(hipGetLastError());
+    return ST_OK;
+}
+
 }  // namespace st
 
 extern "C" int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n)

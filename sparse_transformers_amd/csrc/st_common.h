@@ -179,6 +179,12 @@ int hip_fail(hipError_t e, const char *what);
 
 int device_cu_count();
 
+// Blocks of the streaming decode kernels (one per CU by default) and the fixed-order sum of their
+// fp32 partial rows [G][NB][H] into out[bcount][H].
+int mlp_grid();
+int launch_mlp_reduce(int dtype, const float *partials, int G, int NB, int bcount, int H, void *out,
+                      hipStream_t stream);
+
 // Rows of x from which st_mlp_forward switches from the streaming decode
 // kernel to the MFMA kernels (fp16 / bf16 only).
 constexpr int kPrefillMinRows = 32;

@@ -120,6 +120,13 @@ class SparseDecodeLayer:
     def mlp(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         return self.cache.forward(x, self.act, out=out)
 
+    def step(self, x_pred: torch.Tensor, x: torch.Tensor, mask_override: Optional[torch.Tensor] = None,
+             out: Optional[torch.Tensor] = None, t_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Predictor mask, then cache update and MLP in one call (``WeightCache.update_and_forward``)."""
+        self.predictor.mask(x_pred, "threshold", self.thr, self.ge, out=self.mask, t_ws=t_ws)
+        return self.cache.update_and_forward(self.mask if mask_override is None else mask_override, x, self.act,
+                                             out=out)
+
 
 class SparseMLPStack:
     """A stack of sparse layers stepped one token at a time (the decode loop of the reference,
@@ -129,7 +136,7 @@ class SparseMLPStack:
         self.layers: List[SparseDecodeLayer] = list(layers)
 
     # ---- staged / graph-replayed stepping: fixed device buffers, no allocation, no host reads ----
-    def prepare(self, batch: int, overlap: bool = False) -> None:
+    def prepare(self, batch: int, overlap: bool = False, fused: bool = True) -> None:
         c0 = self.layers[0].cache
         dev, dt, H, I = c0.device, c0.dtype, c0.hidden_size, c0.intermediate_size
         L = len(self.layers)
@@ -143,6 +150,7 @@ class SparseMLPStack:
         self.graph = None
         self.use_trace_masks = True
         self.overlap = overlap
+        self.fused = fused and not overlap   # update + MLP as one call per layer
         self._side = torch.cuda.Stream(device=dev) if overlap else None   # default priority
         self._ev_fork = torch.cuda.Event()
         self._ev_upd = [torch.cuda.Event() for _ in range(L)]
@@ -160,6 +168,11 @@ class SparseMLPStack:
             side.wait_event(self._ev_fork)
         for l, layer in enumerate(self.layers):
             mask = self.mask_stage[l] if self.use_trace_masks else None
+            if self.fused:
+                out = self._pingpong[l & 1]
+                layer.step(self.xp_stage[l], x, mask, out=out, t_ws=self._t_ws)
+                x = out
+                continue
             if side is not None:
                 with torch.cuda.stream(side):
                     layer.compute_mask_and_update(self.xp_stage[l], mask, t_ws=self._t_ws)
@@ -202,6 +215,5 @@ class SparseMLPStack:
         sees the previous layer's output."""
         for l, layer in enumerate(self.layers):
             xp = x if x_pred is None else x_pred[l]
-            layer.compute_mask_and_update(xp, None if mask_override is None else mask_override[l])
-            x = layer.mlp(x)
+            x = layer.step(xp, x, None if mask_override is None else mask_override[l])
         return x

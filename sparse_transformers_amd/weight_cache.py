@@ -13,7 +13,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .ops import current_stream_ptr, dtype_code, mlp_forward_rows, require_gpu
+from .ops import current_stream_ptr, dtype_code, mlp_forward_rows, mlp_workspace, require_gpu
 
 
 class WeightCache:
@@ -158,6 +158,33 @@ class WeightCache:
         return self.down_active[: int(st["n_active"])].t()
 
     # ---------------------------------------------------------------- fast path
+    def update_and_forward(self, mask: torch.Tensor, x: torch.Tensor, act: str = "silu",
+                           out: Optional[torch.Tensor] = None, combined: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``update_active_weights(mask)`` followed by the sparse MLP on x, enqueued as one call and never
+        touching the host.  For one row of x this is a single kernel that takes the rows whose index
+        changed straight from the pool (and writes them back to the active buffers on the way); the
+        cache state and the result equal those of the two separate calls bit for bit."""
+        m = self._mask_arg(mask)
+        H = self.hidden_size
+        x2 = x.reshape(-1, H)
+        if not x2.is_contiguous():
+            x2 = x2.contiguous()
+        if x2.dtype != self.dtype or x2.device != self.device:
+            raise TypeError(f"x must be {self.dtype} on {self.device}")
+        B = x2.size(0)
+        if out is None:
+            out = torch.empty_like(x2)
+        ws = mlp_workspace(self.device, B, H, self.intermediate_size)
+        if act not in _lib.ACT_CODES:
+            raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
+        rc = _lib.lib().st_cache_update_forward(
+            self._h, m.data_ptr(), x2.data_ptr(), B, out.data_ptr(),
+            combined.data_ptr() if combined is not None else None, combined.stride(0) if combined is not None else 0,
+            ws.data_ptr(), ws.numel(), _lib.ACT_CODES[act], current_stream_ptr(self.device))
+        _lib.check(rc, "st_cache_update_forward")
+        self._dirty = True
+        return out.view(x.shape)
+
     def forward(self, x: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor] = None,
                 combined: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Sparse MLP on the cache's packed rows; the active count is read on the device."""

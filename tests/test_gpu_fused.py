@@ -1,0 +1,131 @@
+"""Cache update fused into the decode kernel (st_cache_update_forward) vs the two separate calls.
+
+The fused kernel takes the rows whose index changed from the pool and writes them back on the way, so the
+cache must end in exactly the state update_active_weights leaves (ordered list, counts, active rows), and its
+arithmetic is that of the decode kernel, so the output must carry the same bits."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import sparse_transformers_amd as st
+from sparse_transformers_amd import synthetic as syn
+from conftest import assert_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _pair(I, H, dtype, has_gate, seed, init_mask):
+    g = torch.Generator().manual_seed(seed)
+    tdt = getattr(torch, dtype)
+    gate = (torch.randn(I, H, generator=g) * 0.05).to(tdt)
+    up = (torch.randn(I, H, generator=g) * 0.05).to(tdt)
+    down = (torch.randn(H, I, generator=g) * 0.05).to(tdt)
+    mk = lambda: st.WeightCache(init_mask.to(DEV), H, gate.to(DEV) if has_gate else None, up.to(DEV), down.to(DEV),
+                                has_gate)
+    return mk(), mk(), (gate, up, down), g
+
+
+def _same_state(a, b, step):
+    sa, sb = a.sync_state(), b.sync_state()
+    for key in ("n_active", "n_changed", "n_added", "n_removed", "status", "valid"):
+        assert sa[key] == sb[key], (step, key, sa, sb)
+    n = sa["n_active"]
+    assert torch.equal(a.get_active_indices(), b.get_active_indices()), step
+    assert torch.equal(a.up_active[:n], b.up_active[:n]) and torch.equal(a.down_active[:n], b.down_active[:n]), step
+    if a.has_gate:
+        assert torch.equal(a.gate_active[:n], b.gate_active[:n]), step
+    ea, eb = int(sa["epoch"]), int(sb["epoch"])
+    assert torch.equal(a.cur_mask[ea], b.cur_mask[eb]), step
+
+
+@pytest.mark.parametrize("dtype,H", [("float16", 3072), ("bfloat16", 1024), ("float32", 2048), ("float16", 4096)])
+@pytest.mark.parametrize("has_gate", [True, False])
+def test_fused_equals_update_then_forward(dtype, H, has_gate):
+    I = 1536
+    rng = np.random.default_rng(5)
+    trace = syn.ragged_mask_trace(11 + H, I, 40)      # growth, shrinkage (sequential removals), no-ops, tiny sets
+    fused, plain, (gate, up, down), g = _pair(I, H, dtype, has_gate, 3, torch.from_numpy(trace[0]))
+    tdt = getattr(torch, dtype)
+    for t in range(1, len(trace)):
+        if not trace[t].any():
+            continue
+        m = torch.from_numpy(trace[t]).to(DEV)
+        x = torch.randn(1, H, generator=g).to(tdt).to(DEV)
+        comb_f = torch.zeros(1, 2 * I, dtype=tdt, device=DEV)
+        comb_p = torch.zeros_like(comb_f)
+        yf = fused.update_and_forward(m, x, "silu", combined=comb_f)
+        plain.update_active_weights_async(m)
+        yp = plain.forward(x, "silu", combined=comb_p)
+        torch.cuda.synchronize()
+        assert torch.equal(yf, yp), (t, (yf.float() - yp.float()).abs().max().item())
+        assert torch.equal(comb_f, comb_p), t
+        _same_state(fused, plain, t)
+    # and against the oracle at the end: order, then the MLP on the final active set
+    oc = oracle.OracleWeightCache(trace[0], H, gate.float().numpy() if has_gate else None, up.float().numpy(),
+                                  down.float().numpy(), has_gate)
+    for t in range(1, len(trace)):
+        if trace[t].any():
+            oc.update_active_weights(trace[t])
+    assert fused.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist()
+    want, _ = oracle.mlp_forward(x.float().cpu().numpy(), oc.get_concat_weight(), oc.get_active_down_weight(), "silu",
+                                 has_gate)
+    assert_close(yf.float().cpu().numpy(), want, dtype, "fused output vs oracle")
+
+
+def test_fused_full_size_trace_and_errors():
+    """BASELINE config 2 shape with its churn, then the corner cases: unchanged mask, an update that empties the
+    cache (status reported at the next sync, zeros out), recovery from empty."""
+    H, I, n = 3072, 8192, 2867
+    trace = syn.mask_trace(21, 1, I, n, 12, 0.05, 0.15)[:, 0]
+    fused, plain, _, g = _pair(I, H, "float16", True, 9, torch.from_numpy(trace[0]))
+    x = torch.randn(1, H, generator=g).half().to(DEV)
+    for t in range(1, len(trace)):
+        m = torch.from_numpy(trace[t]).to(DEV)
+        yf = fused.update_and_forward(m, x, "silu")
+        plain.update_active_weights_async(m)
+        yp = plain.forward(x, "silu")
+        assert torch.equal(yf, yp), t
+    _same_state(fused, plain, "trace end")
+    # unchanged mask: nothing moves, same output again
+    y2 = fused.update_and_forward(m, x, "silu")
+    assert torch.equal(y2, yf) and fused.sync_state()["n_changed"] == 0
+    # all-false mask: reference raises "No active weights" (weight_cache.h:117-118); here at the next sync
+    none = torch.zeros(I, dtype=torch.bool, device=DEV)
+    y0 = fused.update_and_forward(none, x, "silu")
+    with pytest.raises(RuntimeError, match="No active weights"):
+        fused.sync_state()
+    assert torch.count_nonzero(y0).item() == 0
+    with pytest.raises(RuntimeError, match="No active weights"):
+        plain.update_active_weights(none)
+    # the remembered mask survives the failed update (weight_cache.h:356-358 is never reached), so the same
+    # mask again is "unchanged" and the cache stays empty; a different mask re-adds only what differs from it
+    y0 = fused.update_and_forward(m, x, "silu")
+    with pytest.raises(RuntimeError, match="No active weights"):
+        fused.sync_state()
+    assert torch.count_nonzero(y0).item() == 0
+    m2 = m.clone()
+    m2[(~m).nonzero().flatten()[:100]] = True       # 100 additions, no removals
+    yf = fused.update_and_forward(m2, x, "silu")
+    plain.update_active_weights_async(m2)
+    yp = plain.forward(x, "silu")
+    assert torch.equal(yf, yp)
+    _same_state(fused, plain, "after recovery")
+    assert fused.get_num_active() == 100
+
+
+def test_fused_call_with_several_rows_takes_the_two_kernel_path():
+    H, I = 2048, 1024
+    trace = syn.ragged_mask_trace(3, I, 6)
+    fused, plain, _, g = _pair(I, H, "bfloat16", True, 1, torch.from_numpy(trace[0]))
+    x = torch.randn(4, H, generator=g).bfloat16().to(DEV)
+    for t in range(1, len(trace)):
+        if not trace[t].any():
+            continue
+        m = torch.from_numpy(trace[t]).to(DEV)
+        yf = fused.update_and_forward(m, x, "relu")
+        plain.update_active_weights_async(m)
+        yp = plain.forward(x, "relu")
+        assert torch.equal(yf, yp), t
+    _same_state(fused, plain, "end")
