@@ -34,6 +34,15 @@ constexpr uint16_t kNone = 0xffffu;
 // LDS per intermediate element: pos(2) + idx(2) + added/removed lists(2) + flags(1) + dirty(1/8)
 constexpr int64_t kPlanMaxI = 22000;
 
+// Block barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global
+// load, which would serialise loads that are meant to stay in flight across the bookkeeping phases.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane)
 {
 #pragma unroll
@@ -50,9 +59,9 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wave_t
 {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t incl = wave_incl_scan(v, lane);
-    __syncthreads();  // protect wave_tot from the previous use
+    lds_barrier();  // protect wave_tot from the previous use
     if (lane == kWave - 1) wave_tot[wave] = incl;
-    __syncthreads();
+    lds_barrier();
     uint32_t prefix = 0, tot = 0;
     for (int w = 0; w < WAVES; ++w) {
         const uint32_t t = wave_tot[w];
@@ -104,11 +113,12 @@ constexpr size_t plan_lds_bytes(int I)
 // barriers.  VEC: I % 8 == 0 and the mask is 8-byte aligned, so masks are read as 8-byte words and
 // indices as 16-byte vectors; both bookkeeping buffers are requested together with the ticket, so the
 // front costs one memory round trip.  MARK: the dirty bitmap is kept on the fast path too.
-// `after_issue` runs right after the front loads have been issued (a place to start other loads).
+// `after_front(n_old)` runs once the front loads have arrived and been put into LDS, before the
+// bookkeeping phases: the place to start other loads that should be in flight meanwhile.
 template <bool VEC, int TPB, bool MARK, typename F>
 __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, const uint8_t *__restrict__ new_mask,
                                            uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
-                                           int32_t *__restrict__ state, int I, F after_issue)
+                                           int32_t *__restrict__ state, int I, F after_front)
 {
     uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);  // index -> position
     uint16_t *idx_l = pos_l + I;                           // position -> index
@@ -152,9 +162,8 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
     }
     // One atomic returns both the epoch (which buffer to read) and this block's ticket.
     if (tid == 0) ticket_s = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
-    after_issue();
     for (int w = tid; w < dirty_words; w += TPB) dirty[w] = 0u;
-    __syncthreads();
+    lds_barrier();
     const uint32_t ticket = ticket_s;
     const int ep = (int)((ticket >> 16) & 1u);
     const bool last_arrival = (ticket & 0xffffu) == gridDim.x - 1;
@@ -194,7 +203,8 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
         }
     }
     ST_TL(1);
-    __syncthreads();
+    after_front(n);
+    lds_barrier();
     ST_TL(2);
     for (int p = tid; p < n; p += TPB) pos_l[idx_l[p]] = (uint16_t)p;
 
@@ -252,7 +262,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
             }
         }
     }
-    __syncthreads();
+    lds_barrier();
 
     const int pairs = na < nr ? na : nr;
     // Without surplus removals (nr <= na) the rewritten positions are known as soon as phases 1 and 2
@@ -281,7 +291,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
         }
         lists[i] = p < I ? (uint16_t)p : kNone;
     }
-    __syncthreads();
+    lds_barrier();
 
     int n_new;
     uint32_t n_changed;
@@ -311,7 +321,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
             }
             n_new_s = m;
         }
-        __syncthreads();
+        lds_barrier();
         ST_TL(4);
         n_new = n_new_s;
 
@@ -329,7 +339,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
             word &= word - 1;
             lists[coff++] = (uint16_t)((tid << 5) + bit);
         }
-        __syncthreads();
+        lds_barrier();
     }
 
     ST_TL(5);
@@ -381,7 +391,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     PlanView pv;
-    cache_plan<VEC, TPB, false>(pv, smem, new_mask, cur_mask2, indices2, state, I, [] {});
+    cache_plan<VEC, TPB, false>(pv, smem, new_mask, cur_mask2, indices2, state, I, [](int) {});
     if (!pv.changed) return;
     const uint16_t *lists = pv.lists, *idx_l = pv.idx_l;
     const uint32_t n_changed = pv.n_changed;
@@ -440,7 +450,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
 // update followed by forward.
 // Rows are dealt to blocks round-robin: row(bat, k) = blk + G * (grp + ngrp * (bat * RB + k)).
 // ---------------------------------------------------------------------------
-template <typename T, int RB, int TPB>
+template <typename T, int RB, int RBS, int TPB>
 __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     CopyPlan cp, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
     int32_t *__restrict__ state, int I, const T *__restrict__ x, int H, T *__restrict__ combined, long ldc,
@@ -461,17 +471,35 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     const size_t coff = valid ? (size_t)cc * 16 : 0;   // byte offset of this thread's chunk (clamped)
     const bool wave_live = __builtin_amdgcn_readfirstlane(cc & ~(kWave - 1)) < chunks;
     const bool has_gate = cp.nmat == 3;
-    const int iu = has_gate ? 1 : 0, id = iu + 1;
     const int row_bytes = cp.row_bytes;
+    // matrix pointers picked with constant subscripts, so that they stay in scalar registers
+    const unsigned char *const pool_g = cp.pool[0], *const pool_u = has_gate ? cp.pool[1] : cp.pool[0];
+    const unsigned char *const pool_d = has_gate ? cp.pool[2] : cp.pool[1];
+    unsigned char *const act_g = cp.active[0], *const act_u = has_gate ? cp.active[1] : cp.active[0];
+    unsigned char *const act_d = has_gate ? cp.active[2] : cp.active[1];
 
     uint4 xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff);
     if (!valid) xr = zero4;
 
-    PlanView pv;
-    cache_plan<true, TPB, true>(pv, smem, new_mask, cur_mask2, indices2, state, I, [] {});
-    const int n = pv.n_new, n_old = pv.n_old;
-
     auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
+
+    // The first RBS rows of the first batch are requested from the active buffers as soon as the old
+    // count is known, i.e. while the plan is still being worked out; most of them are unchanged.
+    uint4 wg[RB], wu[RB], wd[RB];
+    auto speculate = [&](int n_old) __attribute__((always_inline)) {
+        if (RBS == 0 || !wave_live || n_old <= 0) return;
+#pragma unroll
+        for (int k = 0; k < RBS; ++k) {
+            const int p = row_of(0, k);
+            const size_t ro = (size_t)(p < n_old ? p : n_old - 1) * row_bytes + coff;
+            wu[k] = ld16_stream(act_u + ro);
+            wd[k] = ld16_stream(act_d + ro);
+            if (has_gate) wg[k] = ld16_stream(act_g + ro);
+        }
+    };
+    PlanView pv;
+    cache_plan<true, TPB, true>(pv, smem, new_mask, cur_mask2, indices2, state, I, speculate);
+    const int n = pv.n_new, n_old = pv.n_old;
 
     float acc[VEC];
 #pragma unroll
@@ -480,25 +508,39 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     const int jcount = n > blk ? (n - blk + G - 1) / G : 0;      // rows of this block
     const int nbat = ((jcount + ngrp - 1) / ngrp + RB - 1) / RB;  // uniform over the block
     for (int bat = 0; bat < nbat; ++bat) {
-        uint4 wg[RB], wu[RB], wd[RB];
         bool fresh[RB];   // row comes from the pool and has to be written back
+        // (rows, source) of slot k; issues the loads unless the speculative request already covers them
+        auto request = [&](int k, bool speculated) __attribute__((always_inline)) {
+            const int p = row_of(bat, k);
+            const bool ok = p < n;
+            const int pc = ok ? p : n - 1;   // clamped; rows past the count are neutralised below
+            const bool moved = pc >= n_old || ((pv.dirty[pc >> 5] >> (pc & 31)) & 1u);
+            fresh[k] = ok && moved && pv.changed;
+            if (speculated && !fresh[k]) return;
+            const size_t ro = (size_t)(fresh[k] ? (int)pv.idx_l[pc] : pc) * row_bytes + coff;
+            wu[k] = ld16_stream((fresh[k] ? pool_u : act_u) + ro);
+            wd[k] = ld16_stream((fresh[k] ? pool_d : act_d) + ro);
+            wg[k] = has_gate ? ld16_stream((fresh[k] ? pool_g : act_g) + ro) : zero4;
+        };
         if (wave_live) {
+            const bool spec = RBS > 0 && bat == 0 && n_old > 0;
+            // rows nobody has asked for yet go first, then the corrections of the speculative ones
 #pragma unroll
-            for (int k = 0; k < RB; ++k) {
-                const int p = row_of(bat, k);
-                const bool ok = p < n;
-                const int pc = ok ? p : n - 1;   // clamped; rows past the count are neutralised below
-                const bool moved = pc >= n_old || ((pv.dirty[pc >> 5] >> (pc & 31)) & 1u);
-                fresh[k] = ok && moved && pv.changed;
-                const size_t ro = (size_t)(fresh[k] ? (int)pv.idx_l[pc] : pc) * row_bytes + coff;
-                wu[k] = ld16_stream((fresh[k] ? cp.pool[iu] : cp.active[iu]) + ro);
-                wd[k] = ld16_stream((fresh[k] ? cp.pool[id] : cp.active[id]) + ro);
-                wg[k] = has_gate ? ld16_stream((fresh[k] ? cp.pool[0] : cp.active[0]) + ro) : zero4;
+            for (int k = 0; k < RB; ++k)
+                if (k >= RBS || !spec) request(k, false);   // static slot numbers keep the rows in registers
+            if (spec) {
+#pragma unroll
+                for (int k = 0; k < RBS; ++k) request(k, true);
+                if (!has_gate) {
+#pragma unroll
+                    for (int k = 0; k < RBS; ++k) wg[k] = zero4;
+                }
             }
         } else {
 #pragma unroll
             for (int k = 0; k < RB; ++k) { wg[k] = wu[k] = wd[k] = zero4; fresh[k] = false; }
         }
+        ST_TL(6);
 
         // ---- phase 1: partial dot products on this thread's chunk
         float fx[VEC];
@@ -524,9 +566,9 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
         for (int k = 0; k < RB; ++k) {
             if (fresh[k] && valid) {
                 const size_t ro = (size_t)row_of(bat, k) * row_bytes + coff;
-                st16(cp.active[iu] + ro, wu[k]);
-                st16(cp.active[id] + ro, wd[k]);
-                if (has_gate) st16(cp.active[0] + ro, wg[k]);
+                st16(act_u + ro, wu[k]);
+                st16(act_d + ro, wd[k]);
+                if (has_gate) st16(act_g + ro, wg[k]);
             }
         }
         __syncthreads();
@@ -584,6 +626,7 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
             *reinterpret_cast<float4 *>(partials + (size_t)blk * H + (size_t)cc * VEC + e) =
                 make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
     }
+    ST_TL(7);
 }
 
 // in [R,C] -> out [C,R], 64x64 tiles through LDS.
@@ -808,14 +851,17 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
             return ST_OK;
         };
         int rc;
+        static const int spec_rows = [] { const char *v = getenv("ST_FUSED_SPEC"); return v ? atoi(v) : 0; }();
         if (c->dtype == ST_F32)
-            rc = launch(cache_update_decode_kernel<float, RB, TPB>, static_cast<const float *>(x),
+            rc = launch(cache_update_decode_kernel<float, RB, 0, TPB>, static_cast<const float *>(x),
                         static_cast<float *>(combined));
         else if (c->dtype == ST_F16)
-            rc = launch(cache_update_decode_kernel<f16_t, RB, TPB>, static_cast<const f16_t *>(x),
-                        static_cast<f16_t *>(combined));
+            rc = spec_rows ? launch(cache_update_decode_kernel<f16_t, RB, RB / 2, TPB>, static_cast<const f16_t *>(x),
+                                    static_cast<f16_t *>(combined))
+                           : launch(cache_update_decode_kernel<f16_t, RB, 0, TPB>, static_cast<const f16_t *>(x),
+                                    static_cast<f16_t *>(combined));
         else
-            rc = launch(cache_update_decode_kernel<bf16_t, RB, TPB>, static_cast<const bf16_t *>(x),
+            rc = launch(cache_update_decode_kernel<bf16_t, RB, 0, TPB>, static_cast<const bf16_t *>(x),
                         static_cast<bf16_t *>(combined));
         if (rc != ST_OK) return rc;
     }
