@@ -26,9 +26,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of mlp_decode_kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by
-# what the same counter reads for a 256 MiB copy; see profiles/mlp_decode_traffic_llama3b_stack_fp16.md
-MEASURED_TRAFFIC_BYTES = {("llama3b_stack_fp16", "mlp_decode"): 53_040_000 + 3_145_728}
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by
+# what the same counter reads for a 256 MiB copy; see profiles/decode_traffic_llama3b_stack_fp16.md
+MEASURED_TRAFFIC_BYTES = {("llama3b_stack_fp16", "mlp_decode"): 53_040_000 + 3_145_728,
+                          ("llama3b_stack_fp16", "cache_update_decode"): 54_056_960 + 8_297_779}
 
 
 def parse_args():
@@ -222,8 +223,8 @@ def main():
         ms_all.append(np.frombuffer(ms, dtype=np.float32)[:cnt].copy())
 
     # (Events recorded inside a captured graph cannot be read back with hipEventElapsedTime on this ROCm, so
-    # this pass launches eagerly; the GPU idles between launches and the events bracket dispatch overhead,
-    # which makes these durations about 2 us longer than rocprofv3's kernel times - see profiles/.)
+    # this pass launches eagerly.  The library launches with hipExtLaunchKernelGGL, whose start / stop events are
+    # stamped at the kernel's own begin and end, so these are execution times, as rocprofv3 reports them.)
     def summarise():
         kinds_np, ms_np = np.concatenate(kinds_all), np.concatenate(ms_all)
         out = {}
@@ -278,7 +279,7 @@ def main():
                    "churn": [wl.churn_lo, wl.churn_hi], "mask_source": "trace",
                    "launch": "hip_graph" if use_graph else "eager",
                    "streams": 2 if args.overlap else 1, "update_fused_into_decode": bool(stack.fused),
-                   "kernel_timing": "hip events, eager second pass"},
+                   "kernel_timing": "hip events stamped at kernel begin/end (hipExtLaunchKernelGGL), eager second pass"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get((wl.name, dom)) if B == wl.batch else None,

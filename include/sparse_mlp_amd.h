@@ -175,11 +175,14 @@ int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream);
  * is st_cache_update_async followed by st_mlp_forward.  Either way the cache
  * ends in the same state and `out` holds the same bits as the two separate
  * calls.  x, out: [B,H] in the cache's dtype; combined: [B,ldc] or NULL;
- * workspace: st_mlp_workspace_bytes(B, H, I) bytes.  An update that empties
+ * workspace: st_mlp_workspace_bytes(B, H, I) bytes.  n_hint: the active count
+ * the host last saw (0 = unknown); it only decides which rows are requested
+ * before the plan is known and never affects results.  An update that empties
  * the cache leaves status ST_ERR_NO_ACTIVE in the state words (reported by
  * st_cache_sync_state) and zeros in `out`. */
-int st_cache_update_forward(st_cache *c, const uint8_t *mask, const void *x, int64_t B, void *out, void *combined,
-                            int64_t ldc, void *workspace, int64_t workspace_bytes, int act, void *stream);
+int st_cache_update_forward(st_cache *c, const uint8_t *mask, const void *x, int64_t B, int64_t n_hint, void *out,
+                            void *combined, int64_t ldc, void *workspace, int64_t workspace_bytes, int act,
+                            void *stream);
 
 /* get_concat_weight(): weight_cache.h:113-145,362-366.  Writes the contiguous
  * [2n,H] (gate rows then up rows; [n,H] when ungated) tensor into dst, for

@@ -46,7 +46,7 @@ SIGNATURES = {
     "st_cache_destroy": (None, [_vp]),
     "st_cache_load_weights": (_ci, [_vp, _vp, _vp, _vp, _vp]),
     "st_cache_update_async": (_ci, [_vp, _vp, _vp]),
-    "st_cache_update_forward": (_ci, [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _ci, _vp]),
+    "st_cache_update_forward": (_ci, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _vp, _i64, _ci, _vp]),
     "st_cache_sync_state": (_ci, [_vp, _vp, _vp]),
     "st_cache_materialize_concat": (_ci, [_vp, _vp, _i64, _vp]),
     "st_profile_enable": (_ci, [_ci]),

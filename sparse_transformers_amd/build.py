@@ -24,6 +24,9 @@ FLAGS = [
     "-std=c++17",
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the pass that aggregates uniform atomics per wave reads their result back at once; the cache kernels
+    # issue one atomic per block and look at its result much later on purpose
+    "-mllvm", "-amdgpu-atomic-optimizer-strategy=None",
     "-Wall",
     "-Wno-unused-command-line-argument",
 ]

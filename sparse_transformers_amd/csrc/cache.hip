@@ -96,8 +96,9 @@ struct PlanView {
     uint16_t *lists;    // positions to rewrite: [0, n_changed)
     uint32_t *dirty;    // bit per position whose index changed (complete only with MARK, or on the slow path)
     int ep;             // bookkeeping buffer this launch read
-    bool last_arrival;  // this block took the last ticket
     bool writer;        // this block publishes
+    uint32_t arrival;   // thread 0 only: ticket word before this block's arrival (requested, not yet looked at)
+    int next_epoch;     // epoch the last arrival leaves behind
     bool changed;       // false: the mask equals the remembered one, nothing was touched
     int n_old, n_new, na, nr;
     uint32_t n_changed;
@@ -113,12 +114,13 @@ constexpr size_t plan_lds_bytes(int I)
 // barriers.  VEC: I % 8 == 0 and the mask is 8-byte aligned, so masks are read as 8-byte words and
 // indices as 16-byte vectors; both bookkeeping buffers are requested together with the ticket, so the
 // front costs one memory round trip.  MARK: the dirty bitmap is kept on the fast path too.
-// `after_front(n_old)` runs once the front loads have arrived and been put into LDS, before the
-// bookkeeping phases: the place to start other loads that should be in flight meanwhile.
+// `after_issue()` runs right after the front loads have been issued: loads started there travel together
+// with them (the compiler makes every later loop or branch wait for all outstanding loads, so this is
+// the one window in which other loads can overlap the front's memory round trip).
 template <bool VEC, int TPB, bool MARK, typename F>
 __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, const uint8_t *__restrict__ new_mask,
                                            uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
-                                           int32_t *__restrict__ state, int I, F after_front)
+                                           int32_t *__restrict__ state, int I, F after_issue)
 {
     uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);  // index -> position
     uint16_t *idx_l = pos_l + I;                           // position -> index
@@ -131,7 +133,6 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
     uint8_t *flag_l = reinterpret_cast<uint8_t *>(dirty + ((dirty_words + 1) & ~1));  // bit0 new, bit1 old; 8-byte aligned
     __shared__ uint32_t wave_tot[(TPB / kWave)];
     __shared__ int n_new_s;
-    __shared__ uint32_t ticket_s;
     pv.pos_l = pos_l; pv.idx_l = idx_l; pv.lists = lists; pv.dirty = dirty;
 
     const int tid = threadIdx.x;
@@ -139,6 +140,12 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
     // Elements per thread (a contiguous range, so the diff lists come out ascending).
     const int E = VEC ? ((I + 8 * TPB - 1) / (8 * TPB)) * 8 : (I + TPB - 1) / TPB;
     const int e0 = tid * E < I ? tid * E : I, e1 = e0 + E < I ? e0 + E : I;
+
+    // The ticket word holds the epoch (bit 16: which buffer to read) and the arrivals so far.  Every thread
+    // reads it with a plain load, together with the rest of the front; the epoch cannot flip before every
+    // block has arrived, and a block arrives (one atomic, at the end of the plan) only after all its
+    // threads have consumed this load, so they all see the same epoch.
+    const uint32_t tword = *reinterpret_cast<const volatile uint32_t *>(&state[ST_STATE_TICKET]);
 
     uint64_t v_new[kPlanMaxWords], v_cur[2][kPlanMaxWords];
     int4 v_idx[2][kPlanMaxWords][2];
@@ -160,15 +167,11 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
         n_both[0] = state[ST_STATE_N_BUF0];
         n_both[1] = state[ST_STATE_N_BUF1];
     }
-    // One atomic returns both the epoch (which buffer to read) and this block's ticket.
-    if (tid == 0) ticket_s = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
+    after_issue();
     for (int w = tid; w < dirty_words; w += TPB) dirty[w] = 0u;
-    lds_barrier();
-    const uint32_t ticket = ticket_s;
-    const int ep = (int)((ticket >> 16) & 1u);
-    const bool last_arrival = (ticket & 0xffffu) == gridDim.x - 1;
+    const int ep = (int)((tword >> 16) & 1u);
     const bool writer = blockIdx.x == 0;
-    pv.ep = ep; pv.last_arrival = last_arrival; pv.writer = writer;
+    pv.ep = ep; pv.writer = writer;
 
     int n;
     // VEC: new / current mask words as 0x01 bytes, kept in registers for the diff and for publishing
@@ -203,7 +206,6 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
         }
     }
     ST_TL(1);
-    after_front(n);
     lds_barrier();
     ST_TL(2);
     for (int p = tid; p < n; p += TPB) pos_l[idx_l[p]] = (uint16_t)p;
@@ -226,14 +228,13 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
     ST_TL(3);
     const int na = (int)(total & 0xffffu), nr = (int)(total >> 16);
     if (na == 0 && nr == 0) {  // unchanged mask: nothing is touched (weight_cache.h:237-240)
-        if (tid == 0) {
-            if (last_arrival) atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)ep << 16);
-            if (writer) {
-                state[ST_STATE_N_CHANGED] = 0;
-                state[ST_STATE_N_ADDED] = 0;
-                state[ST_STATE_N_REMOVED] = 0;
-            }
+        if (tid == 0 && writer) {
+            state[ST_STATE_N_CHANGED] = 0;
+            state[ST_STATE_N_ADDED] = 0;
+            state[ST_STATE_N_REMOVED] = 0;
         }
+        pv.next_epoch = ep;
+        if (tid == 0) pv.arrival = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
         pv.changed = false;
         pv.n_old = pv.n_new = n; pv.na = pv.nr = 0; pv.n_changed = 0;
         return;
@@ -374,12 +375,24 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
             }
         }
     }
-    if (last_arrival && tid == 0)
-        atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)(ep ^ 1) << 16);
+    pv.next_epoch = ep ^ 1;
+    if (tid == 0) pv.arrival = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
     pv.changed = true;
     pv.n_old = n; pv.n_new = n_new; pv.na = na; pv.nr = nr; pv.n_changed = n_changed;
 }
 
+
+// Last step of a kernel that ran cache_plan: the block that arrived last resets the arrivals and sets the
+// epoch.  Looking at the atomic's result only here keeps its round trip off the critical path.
+__device__ __forceinline__ void plan_finish(const PlanView &pv, int32_t *__restrict__ state)
+{
+    if (threadIdx.x == 0) {
+        uint32_t arrival = pv.arrival;
+        asm volatile("" : "+v"(arrival));   // the result is first looked at here, not where it was requested
+        if ((arrival & 0xffffu) == gridDim.x - 1)
+            atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)pv.next_epoch << 16);
+    }
+}
 
 // update = plan + this block's share of the row copies
 template <bool VEC, int TPB>
@@ -391,8 +404,11 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     PlanView pv;
-    cache_plan<VEC, TPB, false>(pv, smem, new_mask, cur_mask2, indices2, state, I, [](int) {});
-    if (!pv.changed) return;
+    cache_plan<VEC, TPB, false>(pv, smem, new_mask, cur_mask2, indices2, state, I, [] {});
+    if (!pv.changed) {
+        plan_finish(pv, state);
+        return;
+    }
     const uint16_t *lists = pv.lists, *idx_l = pv.idx_l;
     const uint32_t n_changed = pv.n_changed;
     const bool writer = pv.writer;
@@ -433,6 +449,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
         }
     }
 
+    plan_finish(pv, state);
     ST_TL(6);
 }
 
@@ -454,7 +471,7 @@ template <typename T, int RB, int RBS, int TPB>
 __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     CopyPlan cp, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
     int32_t *__restrict__ state, int I, const T *__restrict__ x, int H, T *__restrict__ combined, long ldc,
-    float *__restrict__ partials, int act, int gs_log2, int plan_bytes)
+    float *__restrict__ partials, int act, int gs_log2, int plan_bytes, int n_hint)
 {
     constexpr int VEC = Elem<T>::kVec;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -483,15 +500,17 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
 
     auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
 
-    // The first RBS rows of the first batch are requested from the active buffers as soon as the old
-    // count is known, i.e. while the plan is still being worked out; most of them are unchanged.
+    // The first RBS rows of the first batch are requested from the active buffers together with the
+    // plan's own loads, on the host's guess of the active count (most rows are unchanged; the others are
+    // requested again from the right place once the plan is known).
     uint4 wg[RB], wu[RB], wd[RB];
-    auto speculate = [&](int n_old) __attribute__((always_inline)) {
-        if (RBS == 0 || !wave_live || n_old <= 0) return;
+    const int n_spec = RBS > 0 ? (n_hint < I ? n_hint : I) : 0;
+    auto speculate = [&]() __attribute__((always_inline)) {
+        if (RBS == 0 || !wave_live || n_spec <= 0) return;
 #pragma unroll
         for (int k = 0; k < RBS; ++k) {
             const int p = row_of(0, k);
-            const size_t ro = (size_t)(p < n_old ? p : n_old - 1) * row_bytes + coff;
+            const size_t ro = (size_t)(p < n_spec ? p : n_spec - 1) * row_bytes + coff;
             wu[k] = ld16_stream(act_u + ro);
             wd[k] = ld16_stream(act_d + ro);
             if (has_gate) wg[k] = ld16_stream(act_g + ro);
@@ -516,14 +535,14 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
             const int pc = ok ? p : n - 1;   // clamped; rows past the count are neutralised below
             const bool moved = pc >= n_old || ((pv.dirty[pc >> 5] >> (pc & 31)) & 1u);
             fresh[k] = ok && moved && pv.changed;
-            if (speculated && !fresh[k]) return;
+            if (speculated && !fresh[k] && p < n_spec) return;
             const size_t ro = (size_t)(fresh[k] ? (int)pv.idx_l[pc] : pc) * row_bytes + coff;
             wu[k] = ld16_stream((fresh[k] ? pool_u : act_u) + ro);
             wd[k] = ld16_stream((fresh[k] ? pool_d : act_d) + ro);
             wg[k] = has_gate ? ld16_stream((fresh[k] ? pool_g : act_g) + ro) : zero4;
         };
         if (wave_live) {
-            const bool spec = RBS > 0 && bat == 0 && n_old > 0;
+            const bool spec = RBS > 0 && bat == 0 && n_spec > 0;
             // rows nobody has asked for yet go first, then the corrections of the speculative ones
 #pragma unroll
             for (int k = 0; k < RB; ++k)
@@ -626,6 +645,7 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
             *reinterpret_cast<float4 *>(partials + (size_t)blk * H + (size_t)cc * VEC + e) =
                 make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
     }
+    plan_finish(pv, state);
     ST_TL(7);
 }
 
@@ -776,7 +796,7 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
                 attr_set = true;
             }
-            hipLaunchKernelGGL(kern, dim3(grid), dim3(tpb), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state,
+            ST_LAUNCH(ps, kern, dim3(grid), dim3(tpb), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state,
                                I, gs_log2);
             return ST_OK;
         };
@@ -790,9 +810,9 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     return ST_OK;
 }
 
-extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const void *x, int64_t B, void *out,
-                                       void *combined, int64_t ldc, void *workspace, int64_t workspace_bytes, int act,
-                                       void *stream)
+extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const void *x, int64_t B, int64_t n_hint,
+                                       void *out, void *combined, int64_t ldc, void *workspace,
+                                       int64_t workspace_bytes, int act, void *stream)
 {
     using namespace st;
     ST_REQUIRE(c && mask && x && out && workspace, "st_cache_update_forward: null pointer");
@@ -837,6 +857,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
     cp.row_bytes = row_bytes;
     const int G = mlp_grid();
     float *partials = static_cast<float *>(workspace);
+    const int hint = (int)(n_hint < 0 ? 0 : (n_hint > c->I ? c->I : n_hint));
     {
         ProfScope ps(ST_K_CACHE_UPDATE_DECODE, s);
         auto launch = [&](auto kern, auto *xt, auto *ct) -> int {
@@ -846,8 +867,8 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
                 attr_set = true;
             }
-            hipLaunchKernelGGL(kern, dim3(G), dim3(TPB), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state, I,
-                               xt, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes);
+            ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state, I,
+                               xt, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint);
             return ST_OK;
         };
         int rc;

@@ -45,16 +45,13 @@ struct ProfState {
 };
 static ProfState g_prof;
 
-ProfScope::ProfScope(int kind, hipStream_t s) : slot(-1), stream(s)
+ProfScope::ProfScope(int kind, hipStream_t) : slot(-1), start(nullptr), stop(nullptr)
 {
     if (!g_prof.on || g_prof.used >= g_prof.cap) return;
     slot = g_prof.used++;
     g_prof.kind[slot] = kind;
-    (void)hipEventRecord(g_prof.start[slot], stream);
-}
-ProfScope::~ProfScope()
-{
-    if (slot >= 0) (void)hipEventRecord(g_prof.stop[slot], stream);
+    start = g_prof.start[slot];
+    stop = g_prof.stop[slot];
 }
 
 }  // namespace st

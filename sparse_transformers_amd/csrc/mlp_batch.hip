@@ -360,7 +360,7 @@ static int launch_gateup(const T *x, int B, const T *gate, const T *up, int n, c
         attr_set = true;
     }
     ProfScope ps(ST_K_MLP_BATCH_GATEUP, stream);
-    hipLaunchKernelGGL(kern, dim3(device_cu_count()), dim3(kBtThreads), lds, stream, x, B, gate, up, n, n_dev, hbuf,
+    ST_LAUNCH(ps, kern, dim3(device_cu_count()), dim3(kBtThreads), lds, stream, x, B, gate, up, n, n_dev, hbuf,
                        ldh, comb, ldc, act);
     return ST_OK;
 }
@@ -379,7 +379,7 @@ static int launch_down(const T *hbuf, int ldh, int B, const T *down, int H, int 
         attr_set = true;
     }
     ProfScope ps(ST_K_MLP_BATCH_DOWN, stream);
-    hipLaunchKernelGGL(kern, dim3(s.cg * s.rs), dim3(kBtThreads), lds, stream, hbuf, ldh, B, down, H, n, n_dev, partial,
+    ST_LAUNCH(ps, kern, dim3(s.cg * s.rs), dim3(kBtThreads), lds, stream, hbuf, ldh, B, down, H, n, n_dev, partial,
                        s.cg, s.rs);
     return ST_OK;
 }
@@ -418,7 +418,7 @@ static int launch_batch_t(const void *x_, int B, int H, const void *gate_, const
         ST_HIP(hipGetLastError());
         {
             ProfScope ps(ST_K_MLP_REDUCE, stream);
-            hipLaunchKernelGGL(batch_reduce_kernel<T>, dim3((H / 4 + 255) / 256, bc), dim3(256), 0, stream, partial,
+            ST_LAUNCH(ps, batch_reduce_kernel<T>, dim3((H / 4 + 255) / 256, bc), dim3(256), 0, stream, partial,
                                s.rs, bc, H, out);
         }
         ST_HIP(hipGetLastError());

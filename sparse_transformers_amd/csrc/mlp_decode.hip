@@ -339,7 +339,7 @@ static int launch_inst(const MlpLaunch &a, int b0, int bcount)
     T *comb = a.combined ? static_cast<T *>(a.combined) + (size_t)b0 * a.ldc : nullptr;
     {
         ProfScope ps(ST_K_MLP_DECODE, a.stream);
-        hipLaunchKernelGGL(kern, dim3(a.G), dim3(TPB), lds, a.stream, x, bcount, a.H,
+        ST_LAUNCH(ps, kern, dim3(a.G), dim3(TPB), lds, a.stream, x, bcount, a.H,
                            static_cast<const T *>(a.gate), static_cast<const T *>(a.up),
                            static_cast<const T *>(a.down), a.n, a.n_dev, a.n_hint, comb, a.ldc, a.partials, a.act,
                            a.has_gate, gs_log2);
@@ -348,7 +348,7 @@ static int launch_inst(const MlpLaunch &a, int b0, int bcount)
     T *out = static_cast<T *>(a.out) + (size_t)b0 * a.H;
     {
         ProfScope ps(ST_K_MLP_REDUCE, a.stream);
-        hipLaunchKernelGGL(mlp_reduce_kernel<T>, dim3((a.H + 63) / 64, bcount), dim3(256), 0, a.stream, a.partials,
+        ST_LAUNCH(ps, mlp_reduce_kernel<T>, dim3((a.H + 63) / 64, bcount), dim3(256), 0, a.stream, a.partials,
                            a.G, NB, bcount, a.H, out);
     }
     ST_HIP(hipGetLastError());
@@ -448,13 +448,13 @@ int launch_mlp_reduce(int dtype, const float *partials, int G, int NB, int bcoun
     ProfScope ps(ST_K_MLP_REDUCE, stream);
     const dim3 grid((H + 63) / 64, bcount);
     if (dtype == ST_F32)
-        hipLaunchKernelGGL(mlp_reduce_kernel<float>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+        ST_LAUNCH(ps, mlp_reduce_kernel<float>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
                            static_cast<float *>(out));
     else if (dtype == ST_F16)
-        hipLaunchKernelGGL(mlp_reduce_kernel<f16_t>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+        ST_LAUNCH(ps, mlp_reduce_kernel<f16_t>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
                            static_cast<f16_t *>(out));
     else
-        hipLaunchKernelGGL(mlp_reduce_kernel<bf16_t>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+        ST_LAUNCH(ps, mlp_reduce_kernel<bf16_t>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
                            static_cast<bf16_t *>(out));
     ST_HIP(hipGetLastError());
     return ST_OK;

@@ -335,7 +335,7 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         ProfScope ps(ST_K_MLP_PREFILL_GATEUP, stream);
         const int jt = (int)(ldh / 64), mt = (M + kPfBM - 1) / kPfBM;
         const int grid = (jt * mt + kXcds - 1) / kXcds * kXcds;
-        hipLaunchKernelGGL(prefill_gateup_kernel<T>, dim3(grid), dim3(kPfThreads), 0, stream,
+        ST_LAUNCH(ps, prefill_gateup_kernel<T>, dim3(grid), dim3(kPfThreads), 0, stream,
                            static_cast<const T *>(x), M, H, static_cast<const T *>(gate), static_cast<const T *>(up), n,
                            n_dev, Hh, ldh, static_cast<T *>(comb), ldc, act, has_gate, jt, mt);
     }
@@ -344,14 +344,14 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         ProfScope ps(ST_K_MLP_PREFILL_DOWN, stream);
         const int ct = (H + kPfBN - 1) / kPfBN, mt = (M + kPfBM - 1) / kPfBM;
         const int grid = (ct * mt * split_k + kXcds - 1) / kXcds * kXcds;
-        hipLaunchKernelGGL(prefill_down_kernel<T>, dim3(grid), dim3(kPfThreads), 0, stream, Hh, ldh, M,
+        ST_LAUNCH(ps, prefill_down_kernel<T>, dim3(grid), dim3(kPfThreads), 0, stream, Hh, ldh, M,
                            static_cast<const T *>(down), H, n, n_dev, static_cast<T *>(out), partial, split_k, ct, mt);
     }
     ST_HIP(hipGetLastError());
     if (split_k > 1) {
         ProfScope ps(ST_K_MLP_REDUCE, stream);
         const size_t quads = ((size_t)M * H + 3) / 4;
-        hipLaunchKernelGGL(prefill_reduce_kernel<T>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
+        ST_LAUNCH(ps, prefill_reduce_kernel<T>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
                            partial, split_k, M, H, static_cast<T *>(out));
         ST_HIP(hipGetLastError());
     }

@@ -163,12 +163,12 @@ __global__ __launch_bounds__(kWave) void predictor_up_mask_kernel(const float *_
 }
 
 template <typename T, int LPR>
-static void launch_up(const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge, float *scores,
-                      uint8_t *mask, hipStream_t stream)
+static void launch_up(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
+                      float *scores, uint8_t *mask, hipStream_t stream)
 {
     const size_t lds = (size_t)B * r * sizeof(float);
-    hipLaunchKernelGGL((predictor_up_mask_kernel<T, LPR>), dim3((I + kPredRowsPerWave - 1) / kPredRowsPerWave),
-                       dim3(kWave), lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask);
+    ST_LAUNCH(ps, (predictor_up_mask_kernel<T, LPR>), dim3((I + kPredRowsPerWave - 1) / kPredRowsPerWave),
+              dim3(kWave), lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask);
 }
 
 template <typename T>
@@ -178,18 +178,18 @@ static int launch_predictor(const void *x, int B, int H, const void *A, int r, c
     constexpr int VEC = Elem<T>::kVec;
     {
         ProfScope ps(ST_K_PRED_DOWN, stream);
-        hipLaunchKernelGGL(predictor_down_kernel<T>, dim3(r), dim3(kPredDownThreads), 0, stream,
+        ST_LAUNCH(ps, predictor_down_kernel<T>, dim3(r), dim3(kPredDownThreads), 0, stream,
                            static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
     }
     ST_HIP(hipGetLastError());
     const int chunks = r / VEC;
     {
         ProfScope ps(ST_K_PRED_UP_MASK, stream);
-        if (chunks <= 4) launch_up<T, 4>(t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
-        else if (chunks <= 8) launch_up<T, 8>(t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
-        else if (chunks <= 16) launch_up<T, 16>(t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
-        else if (chunks <= 32) launch_up<T, 32>(t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
-        else launch_up<T, 64>(t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+        if (chunks <= 4) launch_up<T, 4>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+        else if (chunks <= 8) launch_up<T, 8>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+        else if (chunks <= 16) launch_up<T, 16>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+        else if (chunks <= 32) launch_up<T, 32>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+        else launch_up<T, 64>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
     }
     ST_HIP(hipGetLastError());
     return ST_OK;

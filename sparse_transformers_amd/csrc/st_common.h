@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "../../include/sparse_mlp_amd.h"
@@ -201,12 +202,21 @@ int launch_batch(int dtype, const void *x, int B, int H, const void *gate, const
                  const int *n_dev, void *out, void *comb, long ldc, void *workspace, int act, int has_gate,
                  hipStream_t stream);
 
-// Event bracket around one kernel launch; a no-op unless profiling is enabled.
+// Timing slot for one kernel launch; inert unless profiling is enabled.  ST_LAUNCH hands the slot's
+// events to hipExtLaunchKernelGGL, which stamps them at the kernel's own begin and end (so the elapsed
+// time is the kernel's execution time, without dispatch latency).
 struct ProfScope {
     int slot;
-    hipStream_t stream;
+    hipEvent_t start, stop;
     ProfScope(int kind, hipStream_t s);
-    ~ProfScope();
 };
+
+#define ST_LAUNCH(ps, kern, grid, block, lds, stream, ...)                                              \
+    do {                                                                                                \
+        if ((ps).slot >= 0)                                                                             \
+            hipExtLaunchKernelGGL(kern, grid, block, lds, stream, (ps).start, (ps).stop, 0, __VA_ARGS__); \
+        else                                                                                            \
+            hipLaunchKernelGGL(kern, grid, block, lds, stream, __VA_ARGS__);                             \
+    } while (0)
 
 }  // namespace st

@@ -178,7 +178,7 @@ class WeightCache:
         if act not in _lib.ACT_CODES:
             raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
         rc = _lib.lib().st_cache_update_forward(
-            self._h, m.data_ptr(), x2.data_ptr(), B, out.data_ptr(),
+            self._h, m.data_ptr(), x2.data_ptr(), B, int(self._host_state[_lib.STATE_N_ACTIVE]), out.data_ptr(),
             combined.data_ptr() if combined is not None else None, combined.stride(0) if combined is not None else 0,
             ws.data_ptr(), ws.numel(), _lib.ACT_CODES[act], current_stream_ptr(self.device))
         _lib.check(rc, "st_cache_update_forward")
