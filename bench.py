@@ -265,7 +265,11 @@ def main():
     mlp_us = per_kernel[dom]["mean_us"]
     if dom == "mlp_batch_gateup":                        # the batch path streams the weights in two kernels
         mlp_us += per_kernel["mlp_batch_down"]["mean_us"]
-    achieved = alg_bytes / (mlp_us * 1e-6) / 1e9
+    # changed rows per update over the timed steps (the trace swaps as many rows in as out)
+    k_changed = float((trace[W + 1:W + K + 1] & ~trace[W:W + K]).sum(dim=-1).float().mean())
+    upd_bytes = int(2 * mats * k_changed * H * esz)      # cache update: changed rows read + written
+    launch_bytes = alg_bytes + (upd_bytes if dom == "cache_update_decode" else 0)
+    achieved = launch_bytes / (mlp_us * 1e-6) / 1e9
     upd_us = (unfused or per_kernel).get("cache_update", {}).get("mean_us")
 
     churn_mean = 0.5 * (wl.churn_lo + wl.churn_hi)
@@ -283,7 +287,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get((wl.name, dom)) if B == wl.batch else None,
-                     "kernel": dom + "_kernel", "bytes_per_launch": alg_bytes, "mean_us": mlp_us},
+                     "kernel": dom + "_kernel", "bytes_per_launch": launch_bytes, "mean_us": mlp_us,
+                     "bytes_mlp": alg_bytes, "bytes_cache_update": upd_bytes if dom == "cache_update_decode" else 0,
+                     "frac_mlp_bytes_only": round(alg_bytes / (mlp_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)},
         "cache_update_us_per_layer": upd_us,
         "cache_update_note": ("standalone cache_update_kernel, measured in a short unfused pass; the timed path "
                               "runs it fused into the decode kernel") if unfused else "standalone kernel",
