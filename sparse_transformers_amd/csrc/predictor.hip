@@ -13,25 +13,26 @@ namespace st {
 
 constexpr int kPredBTile = 8;
 constexpr int kPredDownThreads = 256;
-constexpr int kPredDownUnroll = 4;  // chunks per thread issued together
+constexpr int kPredDownUnroll = 2;  // chunks per thread issued together
 
 // One block per rank row k: all loads of the row (and of x) are issued before
 // any arithmetic, so the kernel costs one memory round trip.
-template <typename T>
+// BT = rows of x per pass (1 for single-row decode, so that nothing is requested twice).
+template <typename T, int BT>
 __global__ __launch_bounds__(kPredDownThreads) void predictor_down_kernel(const T *__restrict__ x, int B, int H,
                                                                           const T *__restrict__ A, int r,
                                                                           float *__restrict__ t)
 {
     constexpr int VEC = Elem<T>::kVec;
-    __shared__ float red[kPredDownThreads / kWave][kPredBTile];
+    __shared__ float red[kPredDownThreads / kWave][BT];
     const int k = blockIdx.x, tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int chunks = H / VEC;
     const T *row = A + (size_t)k * H;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
-    for (int b0 = 0; b0 < B; b0 += kPredBTile) {
-        float acc[kPredBTile];
+    for (int b0 = 0; b0 < B; b0 += BT) {
+        float acc[BT];
 #pragma unroll
-        for (int b = 0; b < kPredBTile; ++b) acc[b] = 0.f;
+        for (int b = 0; b < BT; ++b) acc[b] = 0.f;
         for (int c0 = 0; c0 < chunks; c0 += kPredDownThreads * kPredDownUnroll) {
             uint4 w[kPredDownUnroll];
 #pragma unroll
@@ -39,33 +40,37 @@ __global__ __launch_bounds__(kPredDownThreads) void predictor_down_kernel(const 
                 const int c = c0 + u * kPredDownThreads + tid;
                 w[u] = c < chunks ? ld16(row + (size_t)c * VEC) : zero4;
             }
+            // x for every row of the tile is requested together (clamped row: the surplus sums are dropped)
+            uint4 xv[BT][kPredDownUnroll];
 #pragma unroll
-            for (int b = 0; b < kPredBTile; ++b) {
-                if (b0 + b < B) {
-                    uint4 xv[kPredDownUnroll];
+            for (int b = 0; b < BT; ++b) {
+                const int bb = b0 + b < B ? b0 + b : B - 1;
 #pragma unroll
-                    for (int u = 0; u < kPredDownUnroll; ++u) {
-                        const int c = c0 + u * kPredDownThreads + tid;
-                        xv[u] = c < chunks ? ld16(x + (size_t)(b0 + b) * H + (size_t)c * VEC) : zero4;
-                    }
+                for (int u = 0; u < kPredDownUnroll; ++u) {
+                    const int c = c0 + u * kPredDownThreads + tid;
+                    xv[b][u] = ld16(x + (size_t)bb * H + (size_t)(c < chunks ? c : 0) * VEC);
+                }
+            }
 #pragma unroll
-                    for (int u = 0; u < kPredDownUnroll; ++u) {
-                        float fw[VEC], fx[VEC];
-                        unpack<T>(w[u], fw);
-                        unpack<T>(xv[u], fx);
+            for (int u = 0; u < kPredDownUnroll; ++u) {
+                float fw[VEC];
+                unpack<T>(w[u], fw);   // zeros past the row end
 #pragma unroll
-                        for (int e = 0; e < VEC; ++e) acc[b] = fmaf(fw[e], fx[e], acc[b]);
-                    }
+                for (int b = 0; b < BT; ++b) {
+                    float fx[VEC];
+                    unpack<T>(xv[b][u], fx);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[b] = fmaf(fw[e], fx[e], acc[b]);
                 }
             }
         }
 #pragma unroll
-        for (int b = 0; b < kPredBTile; ++b) {
+        for (int b = 0; b < BT; ++b) {
             const float s = wave_sum_dpp(acc[b]);
             if (lane == 0) red[wave][b] = s;
         }
         __syncthreads();
-        if (tid < kPredBTile && b0 + tid < B) {
+        if (tid < BT && b0 + tid < B) {
             float s = 0.f;
 #pragma unroll
             for (int w2 = 0; w2 < kPredDownThreads / kWave; ++w2) s += red[w2][tid];
@@ -75,27 +80,29 @@ __global__ __launch_bounds__(kPredDownThreads) void predictor_down_kernel(const 
     }
 }
 
-constexpr int kPredRowsPerWave = 16;
-constexpr int kPredUpBTile = 4;
+constexpr int kPredUpThreads = 256;
+// rows of Bm a wave owns: fewer when a whole wave is needed per row, to keep the accumulators in registers
+constexpr int pred_rows_per_wave(int lpr) { return lpr >= 64 ? 8 : 16; }
+constexpr int kPredUpBTile = 8;
 
 // LPR lanes share one row of Bm (LPR >= r/VEC unless the row needs several
 // passes); a wave owns 16 consecutive rows and issues the loads of all of them
 // before the rank-r intermediate is staged in LDS.
-template <typename T, int LPR>
-__global__ __launch_bounds__(kWave) void predictor_up_mask_kernel(const float *__restrict__ t, int B, int r,
+template <typename T, int LPR, int RPW>
+__global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_kernel(const float *__restrict__ t, int B, int r,
                                                                   const T *__restrict__ Bm, int I, float thr,
                                                                   int cmp_ge, float *__restrict__ scores,
                                                                   uint8_t *__restrict__ mask)
 {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int RPI = kWave / LPR;                                          // rows per iteration
-    constexpr int NIT = kPredRowsPerWave / RPI > 0 ? kPredRowsPerWave / RPI : 1;  // iterations per tile
+    constexpr int NIT = RPW / RPI > 0 ? RPW / RPI : 1;  // iterations per tile
     extern __shared__ __align__(16) unsigned char smem[];
     float *ts = reinterpret_cast<float *>(smem);  // [B][r]
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int chunks = r / VEC;
     const int cl = lane & (LPR - 1), gidx = lane / LPR;
-    const int tile = blockIdx.x * kPredRowsPerWave;
+    const int tile = (blockIdx.x * (kPredUpThreads / kWave) + wave) * RPW;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
 
     float s[NIT][kPredUpBTile];
@@ -114,11 +121,26 @@ __global__ __launch_bounds__(kWave) void predictor_up_mask_kernel(const float *_
             for (int it = 0; it < NIT; ++it) {
                 const int ro = it * RPI + gidx;
                 const int row = tile + ro;
-                w[it] = (c < chunks && ro < kPredRowsPerWave && row < I) ? ld16(Bm + (size_t)row * r + (size_t)c * VEC)
+                w[it] = (c < chunks && ro < RPW && row < I) ? ld16(Bm + (size_t)row * r + (size_t)c * VEC)
                                                                         : zero4;
             }
             if (b0 == 0 && c == cl) {  // stage t after the row loads are in flight
-                for (int i = lane; i < B * r; i += kWave) ts[i] = t[i];
+                // 16-byte pieces, two per thread requested together: one memory round trip per 8 KB
+                // (a scalar copy loop pays one round trip per 256 bytes)
+                const float4 *t4 = reinterpret_cast<const float4 *>(t);
+                float4 *ts4 = reinterpret_cast<float4 *>(ts);
+                const int n4 = (B * r) >> 2;
+                for (int i0 = 0; i0 < n4; i0 += kPredUpThreads * 2) {
+                    float4 v[2];
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        const int i = i0 + u * kPredUpThreads + tid;
+                        v[u] = t4[i < n4 ? i : n4 - 1];
+                    }
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)   // unconditional: the staging buffer is padded to whole batches
+                        ts4[i0 + u * kPredUpThreads + tid] = v[u];
+                }
                 __syncthreads();
             }
             if (c < chunks) {
@@ -142,7 +164,7 @@ __global__ __launch_bounds__(kWave) void predictor_up_mask_kernel(const float *_
         for (int it = 0; it < NIT; ++it) {
             const int ro = it * RPI + gidx;
             const int row = tile + ro;
-            const bool row_ok = ro < kPredRowsPerWave && row < I;
+            const bool row_ok = ro < RPW && row < I;
 #pragma unroll
             for (int b = 0; b < kPredUpBTile; ++b) {
                 if (b0 + b < B) {  // uniform across the wave
@@ -158,17 +180,29 @@ __global__ __launch_bounds__(kWave) void predictor_up_mask_kernel(const float *_
     for (int it = 0; it < NIT; ++it) {
         const int ro = it * RPI + gidx;
         const int row = tile + ro;
-        if (cl == 0 && ro < kPredRowsPerWave && row < I) mask[row] = any[it] ? 1 : 0;
+        if (cl == 0 && ro < RPW && row < I) mask[row] = any[it] ? 1 : 0;
     }
 }
 
+template <typename T, int LPR, int RPW>
+static void launch_up_rpw(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
+                          float *scores, uint8_t *mask, hipStream_t stream)
+{
+    // padded to whole staging batches of 256 threads x 2 x 16 bytes
+    const size_t lds = ((size_t)B * r * sizeof(float) + 8191) / 8192 * 8192;
+    constexpr int rows = RPW * (kPredUpThreads / kWave);
+    ST_LAUNCH(ps, (predictor_up_mask_kernel<T, LPR, RPW>), dim3((I + rows - 1) / rows), dim3(kPredUpThreads), lds,
+              stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask);
+}
+
+// One row of x: 16 rows per wave (8 when a whole wave shares a row).  Several rows of x: 4 rows per wave,
+// so that four times as many waves hide each other's latencies.
 template <typename T, int LPR>
 static void launch_up(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
                       float *scores, uint8_t *mask, hipStream_t stream)
 {
-    const size_t lds = (size_t)B * r * sizeof(float);
-    ST_LAUNCH(ps, (predictor_up_mask_kernel<T, LPR>), dim3((I + kPredRowsPerWave - 1) / kPredRowsPerWave),
-              dim3(kWave), lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask);
+    if (B == 1) launch_up_rpw<T, LPR, pred_rows_per_wave(LPR)>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+    else launch_up_rpw<T, LPR, 4>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
 }
 
 template <typename T>
@@ -178,8 +212,12 @@ static int launch_predictor(const void *x, int B, int H, const void *A, int r, c
     constexpr int VEC = Elem<T>::kVec;
     {
         ProfScope ps(ST_K_PRED_DOWN, stream);
-        ST_LAUNCH(ps, predictor_down_kernel<T>, dim3(r), dim3(kPredDownThreads), 0, stream,
-                           static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
+        if (B == 1)
+            ST_LAUNCH(ps, (predictor_down_kernel<T, 1>), dim3(r), dim3(kPredDownThreads), 0, stream,
+                      static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
+        else
+            ST_LAUNCH(ps, (predictor_down_kernel<T, kPredBTile>), dim3(r), dim3(kPredDownThreads), 0, stream,
+                      static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
     }
     ST_HIP(hipGetLastError());
     const int chunks = r / VEC;
@@ -211,7 +249,7 @@ extern "C" int st_predictor_mask(const void *x, int64_t B, int64_t H, const void
     ST_REQUIRE(r >= 1 && (r * esz) % 16 == 0, "st_predictor_mask: rank %lld rows are not 16-byte multiples",
                (long long)r);
     ST_REQUIRE(I >= 1 && I <= (1 << 24), "st_predictor_mask: I=%lld out of range", (long long)I);
-    ST_REQUIRE(B * r * 4 <= 64 * 1024, "st_predictor_mask: B*r=%lld too large for the LDS staging buffer",
+    ST_REQUIRE(B * r * 4 <= 56 * 1024, "st_predictor_mask: B*r=%lld too large for the LDS staging buffer",
                (long long)(B * r));
     const uintptr_t align = (uintptr_t)x | (uintptr_t)A | (uintptr_t)Bm;
     ST_REQUIRE((align & 15) == 0, "st_predictor_mask: pointers must be 16-byte aligned");
