@@ -82,7 +82,7 @@ __global__ __launch_bounds__(kPredDownThreads) void predictor_down_kernel(const 
 
 constexpr int kPredUpThreads = 256;
 // rows of Bm a wave owns: fewer when a whole wave is needed per row, to keep the accumulators in registers
-constexpr int pred_rows_per_wave(int lpr) { return lpr >= 64 ? 8 : 16; }
+constexpr int pred_rows_per_wave(int lpr) { return lpr >= 64 ? 4 : (lpr >= 32 ? 8 : 16); }
 constexpr int kPredUpBTile = 8;
 
 // LPR lanes share one row of Bm (LPR >= r/VEC unless the row needs several
