@@ -53,15 +53,16 @@ __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane)
     return v;
 }
 
-// Exclusive scan of one uint32 per thread over the block; *total receives the sum.
-template <int WAVES>
-__device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wave_tot, uint32_t *total)
+// Exclusive scan of one uint32 per thread over WAVES waves; *total receives the sum.  `sync` is the
+// barrier of exactly those waves.
+template <int WAVES, typename S>
+__device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wave_tot, uint32_t *total, int tid, S sync)
 {
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
     const uint32_t incl = wave_incl_scan(v, lane);
-    lds_barrier();  // protect wave_tot from the previous use
+    sync();  // protect wave_tot from the previous use
     if (lane == kWave - 1) wave_tot[wave] = incl;
-    lds_barrier();
+    sync();
     uint32_t prefix = 0, tot = 0;
     for (int w = 0; w < WAVES; ++w) {
         const uint32_t t = wave_tot[w];
@@ -70,6 +71,23 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wave_t
     }
     *total = tot;
     return prefix + incl - v;
+}
+
+// Barrier among a subset of the block's waves (all of which are resident together), through a counter in
+// LDS that only grows: each wave adds one and waits until all `waves` have.  The wait is bounded, so a
+// wave can never hang the GPU; running out of spins would mean a broken launch, not a slow one.
+__device__ __forceinline__ void sub_barrier(uint32_t *counter, uint32_t &target, int waves, int tid)
+{
+    target += (uint32_t)waves;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    if ((tid & (kWave - 1)) == 0) atomicAdd(counter, 1u);
+    for (uint32_t spins = 0; spins < (1u << 22); ++spins) {
+        // (an atomic load rather than a volatile one: the latter is emitted as a flat load, which queues
+        // behind the block's global memory traffic)
+        if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= target) break;
+        __builtin_amdgcn_s_sleep(1);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 struct CopyPlan {
@@ -81,7 +99,7 @@ struct CopyPlan {
 
 constexpr int kCopyUnroll = 4;  // rows a thread group keeps in flight
 
-constexpr int kPlanMaxWords = 3;  // 8-element words per thread in the vector path: I <= 24576
+constexpr int kPlanMaxWords = 3;  // 8-element words per thread in the vector path: I <= 32 * threads
 
 __device__ __forceinline__ uint64_t nonzero_bytes(uint64_t x)
 {
@@ -97,7 +115,8 @@ struct PlanView {
     uint32_t *dirty;    // bit per position whose index changed (complete only with MARK, or on the slow path)
     int ep;             // bookkeeping buffer this launch read
     bool writer;        // this block publishes
-    uint32_t arrival;   // thread 0 only: ticket word before this block's arrival (requested, not yet looked at)
+    bool arriver;       // this thread issued the block's arrival
+    uint32_t arrival;   // arriver only: ticket word before this block's arrival (requested, not yet looked at)
     int next_epoch;     // epoch the last arrival leaves behind
     bool changed;       // false: the mask equals the remembered one, nothing was touched
     int n_old, n_new, na, nr;
@@ -109,19 +128,34 @@ constexpr size_t plan_lds_bytes(int I)
     return (size_t)I * 6 + (size_t)(I & 1) * 2 + (size_t)((((I + 31) >> 5) + 1) & ~1) * 4 + (size_t)I + 16;
 }
 
+// Small block-wide scalars of the plan (static LDS, declared by the kernel so that waves which do not take
+// part in the plan can read them).
+struct PlanShared {
+    uint32_t wave_tot[kPlanWaves];
+    int n_new_s;   // count after the sequential removals (slow path)
+    uint32_t sub_count;          // sub_barrier counter
+    int out_n_old, out_n_new, out_changed;   // the finished plan, for waves that did not take part
+};
+
 // Replays the bookkeeping of one update in LDS and publishes it (block 0 writes the other bookkeeping
-// buffer, the last block to arrive flips the epoch).  Called by all threads of the block; contains
-// barriers.  VEC: I % 8 == 0 and the mask is 8-byte aligned, so masks are read as 8-byte words and
-// indices as 16-byte vectors; both bookkeeping buffers are requested together with the ticket, so the
-// front costs one memory round trip.  MARK: the dirty bitmap is kept on the fast path too.
-// `after_issue()` runs right after the front loads have been issued: loads started there travel together
-// with them (the compiler makes every later loop or branch wait for all outstanding loads, so this is
-// the one window in which other loads can overlap the front's memory round trip).
-template <bool VEC, int TPB, bool MARK, typename F>
-__device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, const uint8_t *__restrict__ new_mask,
-                                           uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
-                                           int32_t *__restrict__ state, int I, F after_issue)
+// buffer, the last block to arrive flips the epoch).  Called by PT threads of the block (tid = 0..PT-1)
+// that are exactly the threads executing block barriers at that time, or by all of them together with
+// the rest of the block waiting at a block barrier (SUB); contains barriers.  VEC: I % 8 == 0 and the mask is
+// 8-byte aligned, so masks are read as 8-byte words and indices as 16-byte vectors; both bookkeeping
+// buffers are requested together with the ticket, so the front costs one memory round trip.  MARK: the
+// dirty bitmap is kept on the fast path too.  `after_issue()` runs right after the front loads have
+// been issued.
+//
+// Barrier sequence: 1 after the LDS fill; 2 in the diff scan;
+// [unchanged mask: done]; 1 after the lists; 1 after phases 1 and 2; [surplus removals: 1 after phase 3,
+// 2 in the compaction scan, 1 after the compaction].
+template <bool VEC, int PT, bool MARK, bool SUB, typename F>
+__device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, PlanShared *ps,
+                                           const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2,
+                                           int32_t *__restrict__ indices2, int32_t *__restrict__ state, int I,
+                                           const int tid, F after_issue)
 {
+    constexpr int TPB = PT;
     uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);  // index -> position
     uint16_t *idx_l = pos_l + I;                           // position -> index
     // added indices ascending from the front, removed indices ascending from the
@@ -131,11 +165,17 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
     uint32_t *dirty = reinterpret_cast<uint32_t *>(lists + I + (I & 1));  // bit per position
     const int dirty_words = (I + 31) >> 5;
     uint8_t *flag_l = reinterpret_cast<uint8_t *>(dirty + ((dirty_words + 1) & ~1));  // bit0 new, bit1 old; 8-byte aligned
-    __shared__ uint32_t wave_tot[(TPB / kWave)];
-    __shared__ int n_new_s;
+    uint32_t *wave_tot = ps->wave_tot;
+    int &n_new_s = ps->n_new_s;
+    // SUB: the PT threads are only part of the block and synchronise among themselves
+    uint32_t sub_target = 0;
+    auto sync = [&]() __attribute__((always_inline)) {
+        if constexpr (SUB) sub_barrier(&ps->sub_count, sub_target, PT / kWave, tid);
+        else lds_barrier();
+    };
     pv.pos_l = pos_l; pv.idx_l = idx_l; pv.lists = lists; pv.dirty = dirty;
+    pv.arriver = tid == 0;
 
-    const int tid = threadIdx.x;
     ST_TL(0);
     // Elements per thread (a contiguous range, so the diff lists come out ascending).
     const int E = VEC ? ((I + 8 * TPB - 1) / (8 * TPB)) * 8 : (I + TPB - 1) / TPB;
@@ -145,7 +185,8 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
     // reads it with a plain load, together with the rest of the front; the epoch cannot flip before every
     // block has arrived, and a block arrives (one atomic, at the end of the plan) only after all its
     // threads have consumed this load, so they all see the same epoch.
-    const uint32_t tword = *reinterpret_cast<const volatile uint32_t *>(&state[ST_STATE_TICKET]);
+    const uint32_t tword = __hip_atomic_load(reinterpret_cast<const uint32_t *>(&state[ST_STATE_TICKET]), __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
 
     uint64_t v_new[kPlanMaxWords], v_cur[2][kPlanMaxWords];
     int4 v_idx[2][kPlanMaxWords][2];
@@ -206,7 +247,11 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
         }
     }
     ST_TL(1);
-    lds_barrier();
+    // SUB: this one barrier is a block barrier -- the rest of the block holds its memory requests back
+    // until the plan's own loads have arrived (under a saturated memory system they would take several
+    // times longer, and the whole plan hangs on them)
+    if constexpr (SUB) lds_barrier();
+    else sync();
     ST_TL(2);
     for (int p = tid; p < n; p += TPB) pos_l[idx_l[p]] = (uint16_t)p;
 
@@ -224,7 +269,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
         }
     }
     uint32_t total;
-    const uint32_t off = block_excl_scan<TPB / kWave>(cnt, wave_tot, &total);  // contains __syncthreads
+    const uint32_t off = block_excl_scan<TPB / kWave>(cnt, wave_tot, &total, tid, sync);  // contains __syncthreads
     ST_TL(3);
     const int na = (int)(total & 0xffffu), nr = (int)(total >> 16);
     if (na == 0 && nr == 0) {  // unchanged mask: nothing is touched (weight_cache.h:237-240)
@@ -263,7 +308,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
             }
         }
     }
-    lds_barrier();
+    sync();
 
     const int pairs = na < nr ? na : nr;
     // Without surplus removals (nr <= na) the rewritten positions are known as soon as phases 1 and 2
@@ -292,7 +337,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
         }
         lists[i] = p < I ? (uint16_t)p : kNone;
     }
-    lds_barrier();
+    sync();
 
     int n_new;
     uint32_t n_changed;
@@ -322,7 +367,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
             }
             n_new_s = m;
         }
-        lds_barrier();
+        sync();
         ST_TL(4);
         n_new = n_new_s;
 
@@ -334,13 +379,13 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
             if (lo >= n_new) word = 0;
             else if (lo + 32 > n_new) word &= (1u << (n_new - lo)) - 1u;
         }
-        uint32_t coff = block_excl_scan<TPB / kWave>((uint32_t)__popc(word), wave_tot, &n_changed);  // barrier: lists are dead now
+        uint32_t coff = block_excl_scan<TPB / kWave>((uint32_t)__popc(word), wave_tot, &n_changed, tid, sync);  // barrier: lists are dead now
         while (word) {
             const int bit = __ffs(word) - 1;
             word &= word - 1;
             lists[coff++] = (uint16_t)((tid << 5) + bit);
         }
-        lds_barrier();
+        sync();
     }
 
     ST_TL(5);
@@ -382,11 +427,31 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, co
 }
 
 
+// The finished plan as seen by waves that did not take part in it (after the block barrier that follows
+// plan_publish).
+__device__ __forceinline__ void plan_publish(const PlanView &pv, PlanShared *ps)
+{
+    if (pv.arriver) {
+        ps->out_n_old = pv.n_old;
+        ps->out_n_new = pv.n_new;
+        ps->out_changed = pv.changed ? 1 : 0;
+    }
+}
+__device__ __forceinline__ void plan_adopt(PlanView &pv, unsigned char *smem, const PlanShared *ps, int I)
+{
+    uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);
+    pv.pos_l = pos_l; pv.idx_l = pos_l + I; pv.lists = pos_l + 2 * I;
+    pv.dirty = reinterpret_cast<uint32_t *>(pv.lists + I + (I & 1));
+    pv.arriver = false; pv.writer = false; pv.arrival = 0; pv.next_epoch = 0; pv.ep = 0; pv.n_changed = 0;
+    pv.na = pv.nr = 0;
+    pv.n_old = ps->out_n_old; pv.n_new = ps->out_n_new; pv.changed = ps->out_changed != 0;
+}
+
 // Last step of a kernel that ran cache_plan: the block that arrived last resets the arrivals and sets the
 // epoch.  Looking at the atomic's result only here keeps its round trip off the critical path.
 __device__ __forceinline__ void plan_finish(const PlanView &pv, int32_t *__restrict__ state)
 {
-    if (threadIdx.x == 0) {
+    if (pv.arriver) {
         uint32_t arrival = pv.arrival;
         asm volatile("" : "+v"(arrival));   // the result is first looked at here, not where it was requested
         if ((arrival & 0xffffu) == gridDim.x - 1)
@@ -402,9 +467,10 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
                                                                     int32_t *__restrict__ state, int I, int gs_log2)
 {
     extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ PlanShared ps;
     const int tid = threadIdx.x;
     PlanView pv;
-    cache_plan<VEC, TPB, false>(pv, smem, new_mask, cur_mask2, indices2, state, I, [] {});
+    cache_plan<VEC, TPB, false, false>(pv, smem, &ps, new_mask, cur_mask2, indices2, state, I, tid, [] {});
     if (!pv.changed) {
         plan_finish(pv, state);
         return;
@@ -467,7 +533,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
 // update followed by forward.
 // Rows are dealt to blocks round-robin: row(bat, k) = blk + G * (grp + ngrp * (bat * RB + k)).
 // ---------------------------------------------------------------------------
-template <typename T, int RB, int RBS, int TPB>
+template <typename T, int RB, bool SPLIT, int TPB>
 __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     CopyPlan cp, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
     int32_t *__restrict__ state, int I, const T *__restrict__ x, int H, T *__restrict__ combined, long ldc,
@@ -500,24 +566,42 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
 
     auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
 
-    // The first RBS rows of the first batch are requested from the active buffers together with the
-    // plan's own loads, on the host's guess of the active count (most rows are unchanged; the others are
-    // requested again from the right place once the plan is known).
+    // SPLIT: the upper half of the waves works out the plan while the lower half -- whole row groups --
+    // already streams its first batch of rows from the active buffers, on the host's guess of the count
+    // (most rows are unchanged; the others are requested again from the right place once the plan is
+    // known).
     uint4 wg[RB], wu[RB], wd[RB];
-    const int n_spec = RBS > 0 ? (n_hint < I ? n_hint : I) : 0;
-    auto speculate = [&]() __attribute__((always_inline)) {
-        if (RBS == 0 || !wave_live || n_spec <= 0) return;
-#pragma unroll
-        for (int k = 0; k < RBS; ++k) {
-            const int p = row_of(0, k);
-            const size_t ro = (size_t)(p < n_spec ? p : n_spec - 1) * row_bytes + coff;
-            wu[k] = ld16_stream(act_u + ro);
-            wd[k] = ld16_stream(act_d + ro);
-            if (has_gate) wg[k] = ld16_stream(act_g + ro);
-        }
-    };
+    constexpr int PT = SPLIT ? TPB / 2 : TPB;
+    const bool streams_ahead = SPLIT && tid < TPB / 2;
+    const int n_spec = SPLIT ? (n_hint < I ? n_hint : I) : 0;
+    __shared__ PlanShared plan_shared;
     PlanView pv;
-    cache_plan<true, TPB, true>(pv, smem, new_mask, cur_mask2, indices2, state, I, speculate);
+    if (SPLIT && tid == 0) plan_shared.sub_count = 0;
+    if (streams_ahead) {
+        lds_barrier();   // (A) the plan's own loads have arrived (inside cache_plan, after the LDS fill)
+        if (wave_live && n_spec > 0) {
+#pragma unroll
+            for (int k = 0; k < RB; ++k) {
+                const int p = row_of(0, k);
+                const size_t ro = (size_t)(p < n_spec ? p : n_spec - 1) * row_bytes + coff;
+                wu[k] = ld16_stream(act_u + ro);
+                wd[k] = ld16_stream(act_d + ro);
+                if (has_gate) wg[k] = ld16_stream(act_g + ro);
+            }
+        }
+        lds_barrier();   // (B) the plan is finished
+        plan_adopt(pv, smem, &plan_shared, I);
+    } else {
+        // block barrier (A) sits inside the plan, where its loads have arrived; after it the planning
+        // waves synchronise among themselves, so the streaming waves are free to stall on their own
+        // memory requests
+        cache_plan<true, PT, true, SPLIT>(pv, smem, &plan_shared, new_mask, cur_mask2, indices2, state, I,
+                                          SPLIT ? tid - TPB / 2 : tid, [] {});
+        if (SPLIT) {
+            plan_publish(pv, &plan_shared);
+            lds_barrier();   // (B)
+        }
+    }
     const int n = pv.n_new, n_old = pv.n_old;
 
     float acc[VEC];
@@ -542,18 +626,12 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
             wg[k] = has_gate ? ld16_stream((fresh[k] ? pool_g : act_g) + ro) : zero4;
         };
         if (wave_live) {
-            const bool spec = RBS > 0 && bat == 0 && n_spec > 0;
-            // rows nobody has asked for yet go first, then the corrections of the speculative ones
+            const bool spec = streams_ahead && bat == 0 && n_spec > 0;   // uniform over the wave
 #pragma unroll
-            for (int k = 0; k < RB; ++k)
-                if (k >= RBS || !spec) request(k, false);   // static slot numbers keep the rows in registers
-            if (spec) {
+            for (int k = 0; k < RB; ++k) request(k, spec);   // static slot numbers keep the rows in registers
+            if (spec && !has_gate) {
 #pragma unroll
-                for (int k = 0; k < RBS; ++k) request(k, true);
-                if (!has_gate) {
-#pragma unroll
-                    for (int k = 0; k < RBS; ++k) wg[k] = zero4;
-                }
+                for (int k = 0; k < RB; ++k) wg[k] = zero4;
             }
         } else {
 #pragma unroll
@@ -872,18 +950,20 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
             return ST_OK;
         };
         int rc;
-        static const int spec_rows = [] { const char *v = getenv("ST_FUSED_SPEC"); return v ? atoi(v) : 0; }();
-        if (c->dtype == ST_F32)
-            rc = launch(cache_update_decode_kernel<float, RB, 0, TPB>, static_cast<const float *>(x),
-                        static_cast<float *>(combined));
-        else if (c->dtype == ST_F16)
-            rc = spec_rows ? launch(cache_update_decode_kernel<f16_t, RB, RB / 2, TPB>, static_cast<const f16_t *>(x),
-                                    static_cast<f16_t *>(combined))
-                           : launch(cache_update_decode_kernel<f16_t, RB, 0, TPB>, static_cast<const f16_t *>(x),
-                                    static_cast<f16_t *>(combined));
-        else
-            rc = launch(cache_update_decode_kernel<bf16_t, RB, 0, TPB>, static_cast<const bf16_t *>(x),
-                        static_cast<bf16_t *>(combined));
+        // split roles need whole row groups for each half and the plan done by half the threads
+        static const bool split_off = [] { const char *v = getenv("ST_FUSED_SPLIT"); return v && atoi(v) == 0; }();
+        // (only the fp16 instantiation of the split kernel fits the register file without spilling)
+        const bool split = !split_off && c->dtype == ST_F16 && ngrp >= 2 && (ngrp & 1) == 0 && hint > 0 &&
+                           I <= 8 * (TPB / 2) * kPlanMaxWords;
+#define ST_FUSED_LAUNCH(TYPE)                                                                                       \
+    rc = split ? launch(cache_update_decode_kernel<TYPE, RB, true, TPB>, static_cast<const TYPE *>(x),              \
+                        static_cast<TYPE *>(combined))                                                              \
+               : launch(cache_update_decode_kernel<TYPE, RB, false, TPB>, static_cast<const TYPE *>(x),             \
+                        static_cast<TYPE *>(combined))
+        if (c->dtype == ST_F32) ST_FUSED_LAUNCH(float);
+        else if (c->dtype == ST_F16) ST_FUSED_LAUNCH(f16_t);
+        else ST_FUSED_LAUNCH(bf16_t);
+#undef ST_FUSED_LAUNCH
         if (rc != ST_OK) return rc;
     }
     ST_HIP(hipGetLastError());
