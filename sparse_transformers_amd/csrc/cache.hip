@@ -99,7 +99,7 @@ struct CopyPlan {
 
 constexpr int kCopyUnroll = 4;  // rows a thread group keeps in flight
 
-constexpr int kPlanMaxWords = 3;  // 8-element words per thread in the vector path: I <= 32 * threads
+constexpr int kPlanMaxWords = 4;  // 8-element words per thread in the vector path: I <= 32 * threads
 
 __device__ __forceinline__ uint64_t nonzero_bytes(uint64_t x)
 {
@@ -188,8 +188,10 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
     const uint32_t tword = __hip_atomic_load(reinterpret_cast<const uint32_t *>(&state[ST_STATE_TICKET]), __ATOMIC_RELAXED,
                                              __HIP_MEMORY_SCOPE_AGENT);
 
-    uint64_t v_new[kPlanMaxWords], v_cur[2][kPlanMaxWords];
-    int4 v_idx[2][kPlanMaxWords][2];
+    // (several small arrays rather than one big one: each has to stay below the size up to which the
+    // compiler keeps a private array in registers)
+    uint64_t v_new[kPlanMaxWords], v_cur0[kPlanMaxWords], v_cur1[kPlanMaxWords];
+    int4 v_i0a[kPlanMaxWords], v_i0b[kPlanMaxWords], v_i1a[kPlanMaxWords], v_i1b[kPlanMaxWords];
     int n_both[2];
     if constexpr (VEC) {
 #pragma unroll
@@ -197,12 +199,12 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
             const int e = e0 + 8 * w;
             if (e < e1) {
                 v_new[w] = *reinterpret_cast<const uint64_t *>(new_mask + e);
-#pragma unroll
-                for (int b = 0; b < 2; ++b) {
-                    v_cur[b][w] = *reinterpret_cast<const uint64_t *>(cur_mask2 + (size_t)b * I + e);
-                    v_idx[b][w][0] = *reinterpret_cast<const int4 *>(indices2 + (size_t)b * I + e);
-                    v_idx[b][w][1] = *reinterpret_cast<const int4 *>(indices2 + (size_t)b * I + e + 4);
-                }
+                v_cur0[w] = *reinterpret_cast<const uint64_t *>(cur_mask2 + e);
+                v_cur1[w] = *reinterpret_cast<const uint64_t *>(cur_mask2 + (size_t)I + e);
+                v_i0a[w] = *reinterpret_cast<const int4 *>(indices2 + e);
+                v_i0b[w] = *reinterpret_cast<const int4 *>(indices2 + e + 4);
+                v_i1a[w] = *reinterpret_cast<const int4 *>(indices2 + (size_t)I + e);
+                v_i1b[w] = *reinterpret_cast<const int4 *>(indices2 + (size_t)I + e + 4);
             }
         }
         n_both[0] = state[ST_STATE_N_BUF0];
@@ -225,8 +227,8 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
             w_new[w] = w_cur[w] = 0;
             if (e < e1) {
                 w_new[w] = nonzero_bytes(v_new[w]);
-                w_cur[w] = nonzero_bytes(ep ? v_cur[1][w] : v_cur[0][w]);
-                const int4 a = ep ? v_idx[1][w][0] : v_idx[0][w][0], b4 = ep ? v_idx[1][w][1] : v_idx[0][w][1];
+                w_cur[w] = nonzero_bytes(ep ? v_cur1[w] : v_cur0[w]);
+                const int4 a = ep ? v_i1a[w] : v_i0a[w], b4 = ep ? v_i1b[w] : v_i0b[w];
                 uint4 packed;
                 packed.x = (uint32_t)(a.x & 0xffff) | ((uint32_t)a.y << 16);
                 packed.y = (uint32_t)(a.z & 0xffff) | ((uint32_t)a.w << 16);
@@ -903,7 +905,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int I = (int)c->I, H = (int)c->H;
     const int row_bytes = (int)(c->H * c->esz), chunks = row_bytes >> 4;
-    constexpr int TPB = 1024, RB = 6;
+    constexpr int TPB = 1024;
     int gs_log2 = 6;
     while ((1 << gs_log2) < chunks && (1 << gs_log2) < TPB) ++gs_log2;
     const int ngrp = TPB >> gs_log2;
@@ -953,13 +955,14 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
         // split roles need whole row groups for each half and the plan done by half the threads
         static const bool split_off = [] { const char *v = getenv("ST_FUSED_SPLIT"); return v && atoi(v) == 0; }();
         // (only the fp16 instantiation of the split kernel fits the register file without spilling)
-        const bool split = !split_off && c->dtype == ST_F16 && ngrp >= 2 && (ngrp & 1) == 0 && hint > 0 &&
+        // and it pays only when a block has enough rows to stream while the plan is worked out
+        const bool split = !split_off && c->dtype == ST_F16 && ngrp >= 2 && (ngrp & 1) == 0 && hint >= 6 * G &&
                            I <= 8 * (TPB / 2) * kPlanMaxWords;
 #define ST_FUSED_LAUNCH(TYPE)                                                                                       \
-    rc = split ? launch(cache_update_decode_kernel<TYPE, RB, true, TPB>, static_cast<const TYPE *>(x),              \
-                        static_cast<TYPE *>(combined))                                                              \
-               : launch(cache_update_decode_kernel<TYPE, RB, false, TPB>, static_cast<const TYPE *>(x),             \
-                        static_cast<TYPE *>(combined))
+    rc = split ? launch(cache_update_decode_kernel<TYPE, DecodeRows<TYPE>::value, true, TPB>,                      \
+                        static_cast<const TYPE *>(x), static_cast<TYPE *>(combined))                                \
+               : launch(cache_update_decode_kernel<TYPE, DecodeRows<TYPE>::value, false, TPB>,                     \
+                        static_cast<const TYPE *>(x), static_cast<TYPE *>(combined))
         if (c->dtype == ST_F32) ST_FUSED_LAUNCH(float);
         else if (c->dtype == ST_F16) ST_FUSED_LAUNCH(f16_t);
         else ST_FUSED_LAUNCH(bf16_t);

@@ -386,7 +386,7 @@ template <typename T, int NB> static int launch_one(const MlpLaunch &a, int b0, 
         }
         if (want_rb == 3) return launch_inst<T, 1, 3, 1, 1024, true>(a, b0, bcount);
         if (want_rb == 4) return launch_inst<T, 1, 4, 1, 1024, false>(a, b0, bcount);
-        return launch_inst<T, 1, 6, 1, 1024, false>(a, b0, bcount);
+        return launch_inst<T, 1, DecodeRows<T>::value, 1, 1024, false>(a, b0, bcount);
     } else if constexpr (NB == 2) {
         return launch_inst<T, 2, 2, 1, 1024, true>(a, b0, bcount);
     } else if constexpr (NB == 4) {

@@ -180,6 +180,11 @@ int hip_fail(hipError_t e, const char *what);
 
 int device_cu_count();
 
+// Rows a thread group of the single-row decode kernels keeps in flight (18 16-byte loads per thread).
+// The stand-alone and the fused kernel must agree on it: it decides which block sums which rows, and the
+// two are meant to give the same bits.
+template <typename T> struct DecodeRows { static constexpr int value = 6; };
+
 // Blocks of the streaming decode kernels (one per CU by default) and the fixed-order sum of their
 // fp32 partial rows [G][NB][H] into out[bcount][H].
 int mlp_grid();
