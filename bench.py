@@ -6,10 +6,11 @@ predictor + threshold mask, the differential weight-cache update (driven by a pr
 with the workload's active fraction and per-step churn) and the fused sparse MLP.  All inputs (weights,
 predictor inputs, mask trace) are resident in HBM before the timed region starts.
 
-Prints ONE JSON line (see README / DESIGN.md for the fields).  `roofline` is for the dominant kernel
-(the fused decode MLP): algorithmic bytes 3*n*H*s per launch over its mean duration, measured with HIP
-events recorded on the launch stream in a second pass over the same workload.  `cpu_baseline` times the
-same path on the host cores on a bounded sample.
+Prints ONE JSON line.  `roofline` is for the dominant kernel (the decode MLP with the cache update fused
+into it): algorithmic bytes per launch -- 3*n*H*s of active weights plus 2*3*k*H*s for the k changed rows
+of the update -- over its mean duration, measured with HIP events stamped at the kernel's begin and end
+in a second pass over the same workload.  `cpu_baseline` times the same path on the host cores on a
+bounded sample.
 """
 from __future__ import annotations
 
@@ -144,7 +145,7 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on ONE GPU (every box has one); --gpus {args.gpus} is not supported. "
-              "The path shards along the intermediate dimension (see DESIGN.md) but no multi-GPU code exists.",
+              "The path would shard along the intermediate dimension, but no multi-GPU code exists.",
               file=sys.stderr)
         sys.exit(2)
 
