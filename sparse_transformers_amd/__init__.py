@@ -6,7 +6,7 @@ Unlike the reference's ``sparse_transformers/__init__.py`` nothing global is cha
 fallback: without the built library, or without a GPU tensor, calls raise.
 """
 from .ops import predictor_mask, predictor_scores, sparse_mlp_forward
-from .skip_mlp import FastLoRAProjection, SkipMLP, SparseDecodeLayer, SparseMLPStack
+from .skip_mlp import FastLoRAProjection, SkipMLP, SparseDecodeLayer, SparseMLPStack, load_predictors
 from .weight_cache import WeightCache
 
 __all__ = [
@@ -18,4 +18,5 @@ __all__ = [
     "SkipMLP",
     "SparseDecodeLayer",
     "SparseMLPStack",
+    "load_predictors",
 ]

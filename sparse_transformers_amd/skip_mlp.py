@@ -34,6 +34,18 @@ class FastLoRAProjection:
         d, u = sd["down.weight"], sd["up.weight"]
         return cls(d.to(device=device, dtype=dtype), u.to(device=device, dtype=dtype))
 
+    @classmethod
+    def from_file(cls, path: str, device=None, dtype=None) -> "FastLoRAProjection":
+        """One trained predictor as the reference's trainer saves it (``torch.save(state_dict)``,
+        src/trainer.py:570-585).  Loaded with ``weights_only=True``: nothing in the file is executed."""
+        sd = torch.load(path, map_location="cpu", weights_only=True)
+        return cls.from_state_dict(sd, device=device, dtype=dtype)
+
+    @staticmethod
+    def checkpoint_name(layer_idx: int, lora_pct: float) -> str:
+        """File name the reference gives layer ``layer_idx``'s final predictor (src/trainer.py:573,904)."""
+        return f"final_predictor_layer_{layer_idx}_lora_{lora_pct:.1f}pct.pt"
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return predictor_scores(x, self.down_weight, self.up_weight)
 
@@ -70,6 +82,15 @@ class FastLoRAProjection:
         return m
 
 
+def load_predictors(directory: str, num_layers: int, lora_pct: float, device=None, dtype=None) -> List["FastLoRAProjection"]:
+    """The per-layer predictors of a trained model, from the directory the reference's trainer writes
+    (consumed by benchmark.py:460-468 in the reference)."""
+    import os
+
+    return [FastLoRAProjection.from_file(os.path.join(directory, FastLoRAProjection.checkpoint_name(l, lora_pct)),
+                                         device=device, dtype=dtype) for l in range(num_layers)]
+
+
 class SkipMLP:
     """Gated (or ungated) MLP whose decode path runs on the differential weight cache."""
 
@@ -91,6 +112,11 @@ class SkipMLP:
         if self.weight_cache is None:
             self.weight_cache = WeightCache(self.init_mask, self.hidden_size, self.gate_weight, self.up_weight,
                                             self.down_weight, self.has_gate)
+
+    def reset_cache(self) -> None:
+        """Back to the all-ones mask of a fresh cache (every row active, order 0..I-1)."""
+        self.weight_cache = None
+        self.initialize_weight_cache()
 
     def forward(self, x: torch.Tensor, use_sparse: bool = True) -> torch.Tensor:
         if not use_sparse:

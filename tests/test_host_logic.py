@@ -67,3 +67,23 @@ def test_workloads_match_reference_shapes():
     assert (w.layers, w.hidden, w.intermediate, w.rank, w.n_active) == (28, 3072, 8192, 128, 2867)
     assert syn.WORKLOADS["mistral7b_stack_bf16"].n_active == 3584
     assert syn.WORKLOADS["relullama7b_stack_fp16"].rank == int(0.04 * 11008)
+
+
+def test_predictor_checkpoints_round_trip(tmp_path):
+    """Predictor files as the reference's trainer writes them (state dict with down.weight [r,H] and up.weight
+    [I,r], src/trainer.py:570-585) load back, by the reference's file names, without executing anything."""
+    import torch
+    import sparse_transformers_amd as st
+
+    H, I, r = 32, 96, 8
+    want = []
+    for layer in range(3):
+        sd = {"down.weight": torch.randn(r, H), "up.weight": torch.randn(I, r)}
+        name = st.FastLoRAProjection.checkpoint_name(layer, 4.0)
+        assert name == f"final_predictor_layer_{layer}_lora_4.0pct.pt"
+        torch.save(sd, tmp_path / name)
+        want.append(sd)
+    preds = st.load_predictors(str(tmp_path), 3, 4.0, device="cpu", dtype=torch.float16)
+    for p, sd in zip(preds, want):
+        assert p.lora_size == r and p.hidden_size == H and p.intermediate_size == I
+        assert torch.equal(p.down_weight, sd["down.weight"].half()) and torch.equal(p.up_weight, sd["up.weight"].half())
