@@ -40,10 +40,12 @@ def _same_state(a, b, step):
     assert torch.equal(a.cur_mask[ea], b.cur_mask[eb]), step
 
 
-@pytest.mark.parametrize("dtype,H", [("float16", 3072), ("bfloat16", 1024), ("float32", 2048), ("float16", 4096)])
+# I = 4096 / 9216 with about half the rows active: enough rows per block for the kernel variants that split the
+# waves' roles
+@pytest.mark.parametrize("dtype,H,I", [("float16", 3072, 4096), ("bfloat16", 1024, 4096), ("float32", 2048, 4096),
+                                       ("float16", 4096, 4096), ("float16", 2048, 9216)])
 @pytest.mark.parametrize("has_gate", [True, False])
-def test_fused_equals_update_then_forward(dtype, H, has_gate):
-    I = 4096      # about half active: enough rows per block for the kernel variant that splits the waves' roles
+def test_fused_equals_update_then_forward(dtype, H, I, has_gate):
     rng = np.random.default_rng(5)
     trace = syn.ragged_mask_trace(11 + H, I, 40)      # growth, shrinkage (sequential removals), no-ops, tiny sets
     fused, plain, (gate, up, down), g = _pair(I, H, dtype, has_gate, 3, torch.from_numpy(trace[0]))
