@@ -135,6 +135,7 @@ enum st_state_word {
     ST_STATE_TICKET = 8,    /* internal: (epoch << 16) | blocks arrived in the running update */
     ST_STATE_N_BUF0 = 9,    /* internal: active count of bookkeeping buffer 0 */
     ST_STATE_N_BUF1 = 10,   /* internal: active count of bookkeeping buffer 1 */
+    ST_STATE_FAULT = 11,    /* sticky: a bounded in-kernel wait ran out (never expected); reported as ST_ERR_HIP */
     ST_STATE_WORDS = 16
 };
 

@@ -76,12 +76,17 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wave_t
 // Barrier among a subset of the block's waves (all of which are resident together), through a counter in
 // LDS that only grows: each wave adds one and waits until all `waves` have.  The wait is bounded, so a
 // wave can never hang the GPU; running out of spins would mean a broken launch, not a slow one.
-__device__ __forceinline__ void sub_barrier(uint32_t *counter, uint32_t &target, int waves, int tid)
+__device__ __forceinline__ void sub_barrier(uint32_t *counter, uint32_t &target, int waves, int tid,
+                                            int32_t *fault)
 {
     target += (uint32_t)waves;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     if ((tid & (kWave - 1)) == 0) atomicAdd(counter, 1u);
-    for (uint32_t spins = 0; spins < (1u << 22); ++spins) {
+    for (uint32_t spins = 0;; ++spins) {
+        if (spins == (1u << 22)) {   // leave a mark the host will see; the results of this launch are void
+            if ((tid & (kWave - 1)) == 0) *fault = 1;
+            break;
+        }
         // (an atomic load rather than a volatile one: the latter is emitted as a flat load, which queues
         // behind the block's global memory traffic)
         if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= target) break;
@@ -170,7 +175,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
     // SUB: the PT threads are only part of the block and synchronise among themselves
     uint32_t sub_target = 0;
     auto sync = [&]() __attribute__((always_inline)) {
-        if constexpr (SUB) sub_barrier(&ps->sub_count, sub_target, PT / kWave, tid);
+        if constexpr (SUB) sub_barrier(&ps->sub_count, sub_target, PT / kWave, tid, &state[ST_STATE_FAULT]);
         else lds_barrier();
     };
     pv.pos_l = pos_l; pv.idx_l = idx_l; pv.lists = lists; pv.dirty = dirty;
@@ -985,6 +990,10 @@ extern "C" int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream
     ST_HIP(hipStreamSynchronize(s));
     if (state_out)
         for (int i = 0; i < ST_STATE_WORDS; ++i) state_out[i] = c->host_state[i];
+    if (c->host_state[ST_STATE_FAULT] != 0) {
+        set_error("st_cache: an in-kernel wait ran out; the cache contents are undefined");
+        return ST_ERR_HIP;
+    }
     if (c->host_state[ST_STATE_STATUS] == ST_ERR_NO_ACTIVE) {
         set_error("No active weights");
         return ST_ERR_NO_ACTIVE;
