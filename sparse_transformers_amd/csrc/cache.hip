@@ -568,8 +568,9 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     unsigned char *const act_g = cp.active[0], *const act_u = has_gate ? cp.active[1] : cp.active[0];
     unsigned char *const act_d = has_gate ? cp.active[2] : cp.active[1];
 
-    uint4 xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff);
-    if (!valid) xr = zero4;
+    // x is requested behind the loads the plan hangs on (planning waves) or while waiting for them (the
+    // others), and looked at only in phase 1
+    uint4 xr = zero4;
 
     auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
 
@@ -587,6 +588,7 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     PlanView pv;
     if (SPLIT && tid == 0) plan_shared.sub_count = 0;
     if (streams_ahead) {
+        xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff);
         lds_barrier();   // (A) the plan's own loads have arrived (inside cache_plan, after the LDS fill)
         if (wave_live && n_spec > 0) {
 #pragma unroll
@@ -605,7 +607,8 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
         // waves synchronise among themselves, so the streaming waves are free to stall on their own
         // memory requests
         cache_plan<true, PT, true, SPLIT>(pv, smem, &plan_shared, new_mask, cur_mask2, indices2, state, I,
-                                          SPLIT ? tid - (TPB - PT) : tid, [] {});
+                                          SPLIT ? tid - (TPB - PT) : tid,
+                                          [&] { xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff); });
         if (SPLIT) {
             plan_publish(pv, &plan_shared);
             lds_barrier();   // (B)
@@ -650,7 +653,7 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
 
         // ---- phase 1: partial dot products on this thread's chunk
         float fx[VEC];
-        unpack<T>(xr, fx);
+        unpack<T>(valid ? xr : zero4, fx);
 #pragma unroll
         for (int k = 0; k < RB; ++k) {
             float fg[VEC], fu[VEC], pg = 0.f, pu = 0.f;
