@@ -355,8 +355,6 @@ static int launch_inst(const MlpLaunch &a, int b0, int bcount)
     return ST_OK;
 }
 
-// Tuning knobs (0 = automatic), read once from the environment: ST_MLP_TPB
-// (512 | 1024) and ST_MLP_RB (rows a thread group keeps in flight).
 static int env_int(const char *name)
 {
     const char *v = getenv(name);
@@ -369,23 +367,13 @@ static int env_int(const char *name)
 // the two register buffers.
 template <typename T, int NB> static int launch_one(const MlpLaunch &a, int b0, int bcount)
 {
-    static const int want_tpb = env_int("ST_MLP_TPB"), want_rb = env_int("ST_MLP_RB");
     const int chunks = a.H / Elem<T>::kVec;
     ST_REQUIRE(chunks <= 2048, "st_mlp_forward: hidden size %d too large for this dtype (max %d)", a.H,
                2048 * Elem<T>::kVec);
     if constexpr (NB == 1) {
         if (chunks > 1024) return launch_inst<T, 1, 3, 2, 1024, false>(a, b0, bcount);
-        if (want_tpb == 512) {
-            if (chunks > 512) return launch_inst<T, 1, 6, 2, 512, false>(a, b0, bcount);
-            switch (want_rb) {
-            case 3: return launch_inst<T, 1, 3, 1, 512, true>(a, b0, bcount);
-            case 4: return launch_inst<T, 1, 4, 1, 512, false>(a, b0, bcount);
-            case 12: return launch_inst<T, 1, 12, 1, 512, false>(a, b0, bcount);
-            default: return launch_inst<T, 1, 6, 1, 512, false>(a, b0, bcount);
-            }
-        }
-        if (want_rb == 3) return launch_inst<T, 1, 3, 1, 1024, true>(a, b0, bcount);
-        if (want_rb == 4) return launch_inst<T, 1, 4, 1, 1024, false>(a, b0, bcount);
+        // (512-thread blocks, 3 / 4 / 12 rows in flight and double-buffered row batches were all measured
+        // slower for one row of x)
         return launch_inst<T, 1, DecodeRows<T>::value, 1, 1024, false>(a, b0, bcount);
     } else if constexpr (NB == 2) {
         return launch_inst<T, 2, 2, 1, 1024, true>(a, b0, bcount);

@@ -85,25 +85,14 @@ __device__ __forceinline__ uint4 ld16(const void *p) { return *reinterpret_cast<
 // Streaming variant for data that is read once per launch (weight rows): non-temporal hint.
 __device__ __forceinline__ uint4 ld16_stream(const void *p)
 {
-#ifdef ST_NO_NT_LOADS
-    return *reinterpret_cast<const uint4 *>(p);
-#else
     typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
     const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p));
     return make_uint4(v.x, v.y, v.z, v.w);
-#endif
 }
 __device__ __forceinline__ void st16(void *p, const uint4 &v) { *reinterpret_cast<uint4 *>(p) = v; }
 
-// Sum over the 64 lanes of a wave; every lane receives the total.
-__device__ __forceinline__ float wave_sum(float v)
-{
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
-// Same sum with DPP row operations (no LDS traffic): four steps reduce each
-// row of 16 lanes, the four row totals are then read through scalar registers.
+// Sum over the 64 lanes of a wave with DPP row operations (no LDS traffic): four steps reduce each row of
+// 16 lanes, the four row totals are then read through scalar registers.  Every lane receives the total.
 template <int CTRL> __device__ __forceinline__ float dpp_add(float v)
 {
     const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
@@ -137,13 +126,6 @@ template <int WIDTH> __device__ __forceinline__ float group_sum_dpp(float v)
         if constexpr (WIDTH == 32) v += __shfl_xor(v, 16, kWave);
         return v;
     }
-}
-
-// Sum over aligned groups of `width` lanes (power of two <= 64).
-__device__ __forceinline__ float group_sum(float v, int width)
-{
-    for (int off = width >> 1; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
 }
 
 __device__ __forceinline__ float activate(float v, int act)
