@@ -102,6 +102,34 @@ int st_predictor_mask(const void *x, int64_t B, int64_t H, const void *A, int64_
                       int dtype, float thr, int cmp_ge, float *t_ws, float *scores, uint8_t *mask, void *stream);
 
 /* ------------------------------------------------------------------------
+ * Mask methods that need a statistic of the whole score row, then the union
+ * over rows.  Replaces the "topk" and "statistical_topk" branches and the
+ * any(dim=0) of SkipDecoderLayer._compute_binary_mask
+ * (src/modeling_skip.py:208-214, _gaussian_topk :197-202).
+ *   scores  float [B,I] (what st_predictor_mask leaves in `scores`)
+ *   method  ST_MASK_TOPK: per row the k largest scores (equal scores: lower
+ *           index first; k <= 0 selects nothing, k >= I everything)
+ *           ST_MASK_STATISTICAL: score > mean + std * z per row, population
+ *           std, strict >; z = Normal(0,1).icdf(sparsity) in the reference
+ *   mask    uint8 [I], union over the B rows
+ *   cutoff  optional float [B]: the k-th largest score / the statistical cut
+ *   workspace  only for B > 1: st_mask_select_workspace_bytes(B, I) bytes,
+ *           16-byte aligned; its first 16 bytes must be zero before the first
+ *           call and are left zero by every call.  Calls that share a
+ *           workspace must not overlap.
+ * ------------------------------------------------------------------------ */
+enum st_mask_method { ST_MASK_TOPK = 0, ST_MASK_STATISTICAL = 1 };
+int64_t st_mask_select_workspace_bytes(int64_t B, int64_t I);
+int st_mask_select(const float *scores, int64_t B, int64_t I, int method, int64_t k, float z, uint8_t *mask,
+                   float *cutoff, void *workspace, int64_t workspace_bytes, void *stream);
+
+/* Per-row approximate top-k threshold from four max-sketches.  Replaces
+ * approx_topk_threshold (sparse_transformers/csrc/approx_topk.h:10-88, registered
+ * in sparse_mlp_op.cpp:208) for float scores: threshold[b] = 0.9 * the
+ * max(1, k*cells/F)-th largest sketch cell of row b.  F >= 4, 0 < k <= F. */
+int st_approx_topk_threshold(const float *scores, int64_t B, int64_t F, int64_t k, float *threshold, void *stream);
+
+/* ------------------------------------------------------------------------
  * Differential weight cache, resident in HBM.
  * Replaces class WeightCache (sparse_transformers/csrc/weight_cache.h:13-381)
  * as registered in sparse_mlp_op.cpp:198-202.  The caller owns every device
@@ -204,7 +232,7 @@ typedef enum st_kernel_kind {
     ST_K_MLP_DECODE = 0,
     ST_K_MLP_REDUCE = 1,
     ST_K_CACHE_UPDATE = 2,
-    ST_K_RESERVED = 3,
+    ST_K_MASK_SELECT = 3,
     ST_K_PRED_DOWN = 4,
     ST_K_PRED_UP_MASK = 5,
     ST_K_MLP_PREFILL_GATEUP = 6,

@@ -59,6 +59,7 @@ def lib() -> C.CDLL:
         L.orc_mask_threshold.argtypes = [vp, i64, i64, C.c_float, ci, vp]
         L.orc_mask_topk.argtypes = [vp, i64, i64, i64, vp]
         L.orc_mask_statistical.argtypes = [vp, i64, i64, C.c_float, vp, vp]
+        L.orc_approx_topk_threshold.argtypes = [vp, i64, i64, i64, vp]
         _lib = L
     return _lib
 
@@ -182,6 +183,22 @@ def mask_statistical(scores, z):
     cut = np.empty(s.shape[0], dtype=np.float32)
     lib().orc_mask_statistical(_p(s), s.shape[0], s.shape[1], float(z), _p(m), _p(cut))
     return m.astype(bool), cut
+
+
+def approx_topk_threshold(scores, k) -> np.ndarray:
+    """Per-row sketch threshold [B] (sparse_transformers/csrc/approx_topk.h:10-88)."""
+    s = _f32(scores)
+    if s.ndim != 2:
+        raise ValueError("Input scores must be 2D tensor [batch_size, features]")
+    if k <= 0:
+        raise ValueError("k must be positive")
+    if k > s.shape[1]:
+        raise ValueError("k cannot be larger than feature size")
+    if s.shape[1] < 4:
+        raise ValueError("feature size below 4: the reference divides by a sketch width of zero")
+    thr = np.empty(s.shape[0], dtype=np.float32)
+    lib().orc_approx_topk_threshold(_p(s), s.shape[0], s.shape[1], int(k), _p(thr))
+    return thr
 
 
 # ---------------------------------------------------------------------------

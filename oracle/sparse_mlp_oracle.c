@@ -19,6 +19,7 @@
  *   orc_mask_threshold        src/modeling_skip.py:206-207,214 (naive, thr = 0, >=)
  *   orc_mask_topk             src/modeling_skip.py:208-211,214
  *   orc_mask_statistical      src/modeling_skip.py:197-202,212-214
+ *   orc_approx_topk_threshold sparse_transformers/csrc/approx_topk.h:10-88
  *
  * How the oracle itself is pinned (the reference ships no tests or vectors):
  *   - cache order / layout: against the reference's own C++ compiled from its
@@ -30,6 +31,9 @@
  *     activations: against float64 closed forms evaluated with numpy/torch.
  *   - predictor / masks: against float64 numpy closed forms, numpy
  *     partition/argsort for top-k, brute force on tiny inputs.
+ *   - approx top-k threshold: against the compiled reference operator
+ *     (bit-equal: only max, selection and one float multiply are involved) and
+ *     the golden vectors written from it.
  *   Floating-point summation order of the reference's BLAS is unspecified, so
  *   floating-point parity is tolerance-based; this oracle accumulates in
  *   double and rounds once.
@@ -356,4 +360,39 @@ void orc_mask_statistical(const float *scores, int64_t B, int64_t I, float z, ui
         if (cutoff) cutoff[b] = cut;
         for (int64_t i = 0; i < I; ++i) if (s[i] > cut) mask[i] = 1;
     }
+}
+
+/* Count-min-style sketch threshold per row.  libstdc++'s std::hash<int64_t> is the identity, so cell
+ * (s, p) of the four sketches holds the largest score of the features f with (s*F + f) % W == p,
+ * W = min(1024, F/4).  Cells still at -inf are dropped; the result is the sketch_k-th largest of the
+ * rest times 0.9f, sketch_k = clamp(k * cells / F, 1, cells); 0 when no cell is left.  F >= 4. */
+static int cmp_float_desc(const void *a, const void *b)
+{
+    const float x = *(const float *)a, y = *(const float *)b;
+    return x > y ? -1 : (x < y ? 1 : 0);
+}
+
+void orc_approx_topk_threshold(const float *scores, int64_t B, int64_t F, int64_t k, float *threshold)
+{
+    const int64_t W = F / 4 < 1024 ? F / 4 : 1024;
+    float *cell = (float *)malloc((size_t)(4 * W) * sizeof(float));
+    for (int64_t b = 0; b < B; ++b) {
+        const float *s = scores + b * F;
+        for (int64_t i = 0; i < 4 * W; ++i) cell[i] = -INFINITY;
+        for (int64_t t = 0; t < 4; ++t)
+            for (int64_t f = 0; f < F; ++f) {
+                float *c = cell + t * W + (t * F + f) % W;
+                if (s[f] > *c) *c = s[f];
+            }
+        int64_t cells = 0;
+        for (int64_t i = 0; i < 4 * W; ++i)
+            if (cell[i] != -INFINITY) cell[cells++] = cell[i];
+        if (cells == 0) { threshold[b] = 0.f; continue; }
+        int64_t sk = k * cells / F;
+        if (sk < 1) sk = 1;
+        if (sk > cells) sk = cells;
+        qsort(cell, (size_t)cells, sizeof(float), cmp_float_desc);
+        threshold[b] = cell[sk - 1] * 0.9f;
+    }
+    free(cell);
 }

@@ -5,7 +5,7 @@ Unlike the reference's ``sparse_transformers/__init__.py`` nothing global is cha
 (no thread-count or JIT settings).  The HIP library is loaded on first use and there is no CPU
 fallback: without the built library, or without a GPU tensor, calls raise.
 """
-from .ops import predictor_mask, predictor_scores, sparse_mlp_forward
+from .ops import approx_topk_threshold, mask_select, predictor_mask, predictor_scores, sparse_mlp_forward
 from .skip_mlp import FastLoRAProjection, SkipMLP, SparseDecodeLayer, SparseMLPStack, load_predictors
 from .weight_cache import WeightCache
 
@@ -14,6 +14,8 @@ __all__ = [
     "WeightCache",
     "predictor_mask",
     "predictor_scores",
+    "mask_select",
+    "approx_topk_threshold",
     "FastLoRAProjection",
     "SkipMLP",
     "SparseDecodeLayer",

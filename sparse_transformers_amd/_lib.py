@@ -41,6 +41,9 @@ SIGNATURES = {
     "st_mlp_forward": (_ci, [_vp, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _ci, _ci, _ci,
                              _vp]),
     "st_predictor_mask": (_ci, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _ci, _f, _ci, _vp, _vp, _vp, _vp]),
+    "st_mask_select_workspace_bytes": (_i64, [_i64, _i64]),
+    "st_mask_select": (_ci, [_vp, _i64, _i64, _ci, _i64, _f, _vp, _vp, _vp, _i64, _vp]),
+    "st_approx_topk_threshold": (_ci, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "st_cache_max_intermediate": (_i64, []),
     "st_cache_create": (_vp, [C.POINTER(CacheBuffers), _i64, _i64, _ci, _ci]),
     "st_cache_destroy": (None, [_vp]),
@@ -54,7 +57,7 @@ SIGNATURES = {
     "st_profile_collect": (_ci, [_vp, _vp, _ci]),
 }
 
-KERNEL_KINDS = ["mlp_decode", "mlp_reduce", "cache_update", "reserved", "pred_down", "pred_up_mask",
+KERNEL_KINDS = ["mlp_decode", "mlp_reduce", "cache_update", "mask_select", "pred_down", "pred_up_mask",
                 "mlp_prefill_gateup", "mlp_prefill_down", "mlp_batch_gateup", "mlp_batch_down",
                 "cache_update_decode"]
 

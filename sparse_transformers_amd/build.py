@@ -15,7 +15,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libsparse_mlp_amd.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["capi.hip", "mlp_decode.hip", "mlp_batch.hip", "mlp_prefill.hip", "predictor.hip", "cache.hip"]
+SOURCES = ["capi.hip", "mlp_decode.hip", "mlp_batch.hip", "mlp_prefill.hip", "predictor.hip", "mask_select.hip",
+           "cache.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -6,6 +6,10 @@ Mirrors the operator surface of NimbleEdge/sparse_transformers:
     README.md:108-116 (six-argument call).
   * ``predictor_mask`` / ``predictor_scores`` — FastLoRAProjection.forward and
     SkipDecoderLayer._compute_binary_mask, src/modeling_skip.py:52-53,204-214.
+  * ``mask_select`` — the "topk" and "statistical_topk" methods of the same function
+    (src/modeling_skip.py:197-202,208-214).
+  * ``approx_topk_threshold(scores, k)`` — sparse_transformers/csrc/approx_topk.h:10-88
+    (registered in sparse_mlp_op.cpp:208).
 
 torch is used for device memory and the current stream only; all arithmetic is
 done by the HIP kernels behind the C ABI.
@@ -178,3 +182,67 @@ def predictor_mask(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.
 def predictor_scores(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.Tensor) -> torch.Tensor:
     """fp32 scores [B, I] of the LoRA predictor (FastLoRAProjection.forward)."""
     return predictor_mask(x, down_weight, up_weight, 0.0, True, return_scores=True)[1]
+
+
+MASK_METHODS = {"topk": 0, "statistical_topk": 1}
+_select_workspaces: dict = {}
+
+
+def _select_workspace(device: torch.device, B: int, I: int) -> torch.Tensor:
+    """Zero-initialised once; every call leaves the ticket word at the front zero again."""
+    need = int(_lib.lib().st_mask_select_workspace_bytes(B, I))
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    ws = _select_workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(need, dtype=torch.uint8, device=device)
+        _select_workspaces[key] = ws
+    return ws
+
+
+def mask_select(scores: torch.Tensor, method: str, k: int = 0, std_multiplier: float = 0.0,
+                out: Optional[torch.Tensor] = None, return_cutoff: bool = False):
+    """Union over rows of the per-row selection on fp32 ``scores`` [B, I].
+
+    ``topk``: the k largest scores of every row (src/modeling_skip.py:208-211; equal scores are taken in
+    index order).  ``statistical_topk``: score > mean + std * std_multiplier with the population standard
+    deviation (src/modeling_skip.py:197-202).  Returns bool[I] (and the per-row cutoffs [B] on request).
+    """
+    dev = require_gpu(scores, out)
+    if method not in MASK_METHODS:
+        raise ValueError(f"unknown sparsity method {method!r}")
+    if scores.dim() != 2 or scores.dtype != torch.float32:
+        raise ValueError("scores must be a float32 [B, I] tensor")
+    scores = scores if scores.is_contiguous() else scores.contiguous()
+    B, I = scores.shape
+    mask = out if out is not None else torch.empty(I, dtype=torch.bool, device=dev)
+    if mask.dtype != torch.bool or mask.numel() != I or not mask.is_contiguous():
+        raise ValueError("out must be a contiguous bool[I] tensor")
+    cutoff = torch.empty(B, dtype=torch.float32, device=dev) if return_cutoff else None
+    ws = _select_workspace(dev, B, I) if B > 1 else None
+    rc = _lib.lib().st_mask_select(
+        scores.data_ptr(), B, I, MASK_METHODS[method], int(k), float(std_multiplier), mask.data_ptr(),
+        cutoff.data_ptr() if cutoff is not None else None, ws.data_ptr() if ws is not None else None,
+        ws.numel() if ws is not None else 0, current_stream_ptr(dev))
+    _lib.check(rc, "st_mask_select")
+    return (mask, cutoff) if return_cutoff else mask
+
+
+def approx_topk_threshold(scores: torch.Tensor, k: int) -> torch.Tensor:
+    """Per-row approximate top-k threshold [B, 1] from four max-sketches
+    (sparse_transformers/csrc/approx_topk.h:10-88).  ``scores`` is a float32 [B, F] GPU tensor."""
+    dev = require_gpu(scores)
+    if scores.dim() != 2:
+        raise RuntimeError("Input scores must be 2D tensor [batch_size, features]")
+    if scores.dtype != torch.float32:
+        raise TypeError("approx_topk_threshold: scores must be float32")
+    if k <= 0:
+        raise RuntimeError("k must be positive")
+    if k > scores.size(1):
+        raise RuntimeError("k cannot be larger than feature size")
+    scores = scores if scores.is_contiguous() else scores.contiguous()
+    B, F = scores.shape
+    thr = torch.empty(B, 1, dtype=torch.float32, device=dev)
+    rc = _lib.lib().st_approx_topk_threshold(scores.data_ptr(), B, F, int(k), thr.data_ptr(), current_stream_ptr(dev))
+    _lib.check(rc, "st_approx_topk_threshold")
+    return thr

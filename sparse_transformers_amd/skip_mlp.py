@@ -14,7 +14,7 @@ from typing import List, Optional, Sequence
 
 import torch
 
-from .ops import predictor_mask, predictor_scores, sparse_mlp_forward
+from .ops import mask_select, predictor_mask, predictor_scores, sparse_mlp_forward
 from .weight_cache import WeightCache
 
 
@@ -57,29 +57,17 @@ class FastLoRAProjection:
         """Union-over-rows boolean mask, src/modeling_skip.py:204-214.
 
         ``naive`` (score >= 0) and ``threshold`` (score >= thr, or > thr) are fused into the predictor
-        kernel.  ``topk`` and ``statistical_topk`` take the kernel's fp32 scores and finish with torch
-        reductions on the device.
+        kernel.  ``topk`` and ``statistical_topk`` need a statistic of the whole row: the predictor kernel
+        leaves its fp32 scores and a selection kernel (one block per row) finishes.
         """
         if method == "naive":
             return predictor_mask(x, self.down_weight, self.up_weight, 0.0, True, out=out, t_ws=t_ws)
         if method == "threshold":
             return predictor_mask(x, self.down_weight, self.up_weight, thr, ge, out=out, t_ws=t_ws)
-        scores = self.forward(x)
-        if method == "topk":
-            idx = scores.topk(k, sorted=False)[1]
-            m = torch.zeros_like(scores, dtype=torch.bool)
-            m.scatter_(-1, idx, True)
-        elif method == "statistical_topk":
-            mean = scores.mean(dim=-1, keepdim=True)
-            std = scores.std(dim=-1, keepdim=True, unbiased=False)
-            m = scores > (mean + std * std_multiplier)
-        else:
+        if method not in ("topk", "statistical_topk"):
             raise ValueError(f"unknown sparsity method {method!r}")
-        m = m.any(dim=0)
-        if out is not None:
-            out.copy_(m)
-            return out
-        return m
+        scores = self.forward(x)
+        return mask_select(scores, method, k=k, std_multiplier=std_multiplier, out=out)
 
 
 def load_predictors(directory: str, num_layers: int, lora_pct: float, device=None, dtype=None) -> List["FastLoRAProjection"]:

@@ -10,9 +10,13 @@ produced by compiling its sources (sparse_transformers/csrc/sparse_mlp_op.cpp + 
                       cache does afterwards, gated and ungated
   mlp_forward.json    tiny fp32 inputs and outputs of torch.ops.sparse_mlp.forward
                       (sparse_mlp_op.cpp:79-192, the ReLU operator), gated and ungated
+  approx_topk.json    fp32 score rows and the thresholds torch.ops.sparse_mlp.approx_topk_threshold
+                      returns for them (approx_topk.h:10-88), incl. feature sizes that are not
+                      multiples of the sketch width, repeated values and -inf scores
 
 Run from the repository root in a container that has /root/reference:  python tests/golden/make_golden.py
 """
+import base64
 import json
 import os
 import sys
@@ -118,6 +122,26 @@ def main():
     with open(os.path.join(HERE, "mlp_forward.json"), "w") as f:
         json.dump({"source": "torch.ops.sparse_mlp.forward compiled from sparse_transformers/csrc (ReLU operator)",
                    "cases": cases}, f, separators=(",", ":"))
+    approx = torch.ops.sparse_mlp.approx_topk_threshold
+    acases = []
+    g = torch.Generator().manual_seed(9)
+    for (B, F, k, kind) in [(1, 16, 4, "normal"), (3, 37, 5, "normal"), (2, 64, 64, "normal"), (2, 100, 1, "normal"),
+                            (1, 257, 30, "coarse"), (2, 96, 20, "neginf"), (1, 5000, 700, "normal"),
+                            (2, 4099, 1025, "coarse")]:
+        sc = torch.randn(B, F, generator=g)
+        if kind == "coarse":       # many equal values
+            sc = (sc * 4).round() / 4
+        elif kind == "neginf":     # whole residue classes at -inf: some sketch cells stay empty
+            sc[:, ::2] = float("-inf")
+            sc[1] = float("-inf")
+        thr = approx(sc, k)
+        # little-endian float32 bytes, base64 (keeps the fixture small and bit-exact)
+        acases.append({"B": B, "F": F, "k": k,
+                       "scores_f32_b64": base64.b64encode(sc.numpy().astype("<f4").tobytes()).decode("ascii"),
+                       "threshold_f32_b64": base64.b64encode(thr.numpy().astype("<f4").tobytes()).decode("ascii")})
+    with open(os.path.join(HERE, "approx_topk.json"), "w") as f:
+        json.dump({"source": "torch.ops.sparse_mlp.approx_topk_threshold compiled from sparse_transformers/csrc",
+                   "cases": acases}, f, separators=(",", ":"))
     print("wrote", os.listdir(HERE))
 
 

@@ -231,3 +231,58 @@ def test_mask_bruteforce_tiny():
     assert oracle.mask_threshold(s, 0.0, True).tolist() == [True, False, True]
     assert oracle.mask_threshold(s, 0.0, False).tolist() == [True, False, False]
     assert oracle.mask_topk(s, 1).tolist() == [True, True, False]
+
+
+# ------------------------------------------------------------------ sketch threshold (approx_topk.h)
+def _b64_f32(s):
+    import base64
+
+    return np.frombuffer(base64.b64decode(s), dtype="<f4").copy()
+
+
+def test_approx_topk_matches_reference_vectors():
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(__file__), "golden", "approx_topk.json")) as f:
+        cases = json.load(f)["cases"]
+    assert len(cases) >= 8
+    for c in cases:
+        sc = _b64_f32(c["scores_f32_b64"]).reshape(c["B"], c["F"])
+        want = _b64_f32(c["threshold_f32_b64"])
+        got = oracle.approx_topk_threshold(sc, c["k"])
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (c["B"], c["F"], c["k"])
+
+
+def test_approx_topk_against_compiled_reference_random():
+    if oracle.load_reference() is None:
+        pytest.skip("oracle/_ref not built (needs the reference checkout)")
+    import torch
+
+    op = torch.ops.sparse_mlp.approx_topk_threshold
+    rng = np.random.default_rng(21)
+    for F in (4, 7, 63, 64, 1000, 4096, 4097, 8192, 11008, 14336):
+        for B in (1, 3):
+            sc = rng.standard_normal((B, F)).astype(np.float32)
+            if F % 2:
+                sc = np.round(sc * 8) / 8          # ties
+            for k in sorted({1, max(1, F // 10), max(1, F // 2), F}):
+                want = op(torch.from_numpy(sc), k).numpy().reshape(-1)
+                got = oracle.approx_topk_threshold(sc, k)
+                assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (F, B, k)
+
+
+def test_approx_topk_special_cases():
+    # F a multiple of the sketch width: all four sketches equal the per-residue maxima, so with k = F the
+    # threshold is 0.9 * the smallest of those maxima
+    F, W = 64, 16
+    rng = np.random.default_rng(3)
+    sc = rng.standard_normal((1, F)).astype(np.float32)
+    maxima = sc[0].reshape(F // W, W).max(0)
+    assert oracle.approx_topk_threshold(sc, F)[0] == np.float32(maxima.min()) * np.float32(0.9)
+    # k = 1: sketch_k = 1, the largest cell, which is the global maximum
+    assert oracle.approx_topk_threshold(sc, 1)[0] == np.float32(sc.max()) * np.float32(0.9)
+    with pytest.raises(ValueError):
+        oracle.approx_topk_threshold(sc, 0)
+    with pytest.raises(ValueError):
+        oracle.approx_topk_threshold(sc, F + 1)
