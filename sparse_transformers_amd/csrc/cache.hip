@@ -102,6 +102,14 @@ struct CopyPlan {
     int row_bytes;
 };
 
+// The same matrices for the fused update + MLP kernel, by name (no arrays: nothing for the compiler to index).
+// Without a gate the gate members repeat the up members and are not used.
+struct FusedRows {
+    const unsigned char *pool_g, *pool_u, *pool_d;
+    unsigned char *act_g, *act_u, *act_d;
+    int row_bytes, has_gate;
+};
+
 constexpr int kCopyUnroll = 4;  // rows a thread group keeps in flight
 
 constexpr int kPlanMaxWords = 4;  // 8-element words per thread in the vector path: I <= 32 * threads
@@ -542,7 +550,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
 // ---------------------------------------------------------------------------
 template <typename T, int RB, int PLANW, int TPB>
 __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
-    CopyPlan cp, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
+    FusedRows fr, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
     int32_t *__restrict__ state, int I, const T *__restrict__ x, int H, T *__restrict__ combined, long ldc,
     float *__restrict__ partials, int act, int gs_log2, int plan_bytes, int n_hint)
 {
@@ -560,13 +568,10 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     const bool valid = cc < chunks;
     const size_t coff = valid ? (size_t)cc * 16 : 0;   // byte offset of this thread's chunk (clamped)
     const bool wave_live = __builtin_amdgcn_readfirstlane(cc & ~(kWave - 1)) < chunks;
-    const bool has_gate = cp.nmat == 3;
-    const int row_bytes = cp.row_bytes;
-    // matrix pointers picked with constant subscripts, so that they stay in scalar registers
-    const unsigned char *const pool_g = cp.pool[0], *const pool_u = has_gate ? cp.pool[1] : cp.pool[0];
-    const unsigned char *const pool_d = has_gate ? cp.pool[2] : cp.pool[1];
-    unsigned char *const act_g = cp.active[0], *const act_u = has_gate ? cp.active[1] : cp.active[0];
-    unsigned char *const act_d = has_gate ? cp.active[2] : cp.active[1];
+    const bool has_gate = fr.has_gate != 0;
+    const int row_bytes = fr.row_bytes;
+    const unsigned char *const pool_g = fr.pool_g, *const pool_u = fr.pool_u, *const pool_d = fr.pool_d;
+    unsigned char *const act_g = fr.act_g, *const act_u = fr.act_u, *const act_d = fr.act_d;
 
     // x is requested behind the loads the plan hangs on (planning waves) or while waiting for them (the
     // others), and looked at only in phase 1
@@ -623,19 +628,21 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     const int jcount = n > blk ? (n - blk + G - 1) / G : 0;      // rows of this block
     const int nbat = ((jcount + ngrp - 1) / ngrp + RB - 1) / RB;  // uniform over the block
     for (int bat = 0; bat < nbat; ++bat) {
-        bool fresh[RB];   // row comes from the pool and has to be written back
+        unsigned fresh = 0u;   // bit k: row of slot k comes from the pool and has to be written back
         // (rows, source) of slot k; issues the loads unless the speculative request already covers them
         auto request = [&](int k, bool speculated) __attribute__((always_inline)) {
             const int p = row_of(bat, k);
             const bool ok = p < n;
             const int pc = ok ? p : n - 1;   // clamped; rows past the count are neutralised below
             const bool moved = pc >= n_old || ((pv.dirty[pc >> 5] >> (pc & 31)) & 1u);
-            fresh[k] = ok && moved && pv.changed;
-            if (speculated && !fresh[k] && p < n_spec) return;
-            const size_t ro = (size_t)(fresh[k] ? (int)pv.idx_l[pc] : pc) * row_bytes + coff;
-            wu[k] = ld16_stream((fresh[k] ? pool_u : act_u) + ro);
-            wd[k] = ld16_stream((fresh[k] ? pool_d : act_d) + ro);
-            wg[k] = has_gate ? ld16_stream((fresh[k] ? pool_g : act_g) + ro) : zero4;
+            const bool pooled = ok && moved && pv.changed;
+            if (pooled) fresh |= 1u << k;
+            if (speculated && !pooled && p < n_spec) return;
+            const int pooled_row = (int)pv.idx_l[pc];   // read whether needed or not: no branch, plain selects below
+            const size_t ro = (size_t)(pooled ? pooled_row : pc) * row_bytes + coff;
+            wu[k] = ld16_stream((pooled ? pool_u : act_u) + ro);
+            wd[k] = ld16_stream((pooled ? pool_d : act_d) + ro);
+            wg[k] = has_gate ? ld16_stream((pooled ? pool_g : act_g) + ro) : zero4;
         };
         if (wave_live) {
             const bool spec = streams_ahead && bat == 0 && n_spec > 0;   // uniform over the wave
@@ -647,23 +654,16 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
             }
         } else {
 #pragma unroll
-            for (int k = 0; k < RB; ++k) { wg[k] = wu[k] = wd[k] = zero4; fresh[k] = false; }
+            for (int k = 0; k < RB; ++k) wg[k] = wu[k] = wd[k] = zero4;
         }
         ST_TL(6);
 
         // ---- phase 1: partial dot products on this thread's chunk
-        float fx[VEC];
-        unpack<T>(valid ? xr : zero4, fx);
+        const uint4 xq = valid ? xr : zero4;
 #pragma unroll
         for (int k = 0; k < RB; ++k) {
-            float fg[VEC], fu[VEC], pg = 0.f, pu = 0.f;
-            unpack<T>(wg[k], fg);
-            unpack<T>(wu[k], fu);
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                pg = fmaf(fg[e], fx[e], pg);
-                pu = fmaf(fu[e], fx[e], pu);
-            }
+            float pg = 0.f, pu = 0.f;
+            dot_chunk<T>(wg[k], wu[k], xq, pg, pu);
             const float sg = wave_sum_dpp(pg), su = wave_sum_dpp(pu);
             if (lane == 0) {
                 red[wave][k][0] = sg;
@@ -673,7 +673,7 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
         // write the fresh rows back while the reductions settle
 #pragma unroll
         for (int k = 0; k < RB; ++k) {
-            if (fresh[k] && valid) {
+            if (((fresh >> k) & 1u) && valid) {
                 const size_t ro = (size_t)row_of(bat, k) * row_bytes + coff;
                 st16(act_u + ro, wu[k]);
                 st16(act_d + ro, wd[k]);
@@ -702,11 +702,7 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
 #pragma unroll
         for (int k = 0; k < RB; ++k) {
             const bool row_ok = row_of(bat, k) < n;
-            float fw[VEC];
-            unpack<T>(row_ok ? wd[k] : zero4, fw);
-            const float hv = hs[grp][k];
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) acc[e] = fmaf(hv, fw[e], acc[e]);
+            axpy_chunk<T>(hs[grp][k], row_ok ? wd[k] : zero4, acc);
         }
     }
 
@@ -933,18 +929,15 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
                               c->b.state + ST_STATE_N_ACTIVE, 0, out, combined, ldc, workspace, workspace_bytes, act,
                               c->dtype, c->has_gate, stream);
     }
-    CopyPlan cp;
-    cp.nmat = 0;
-    if (c->has_gate) {
-        cp.pool[cp.nmat] = static_cast<const unsigned char *>(c->b.gate_pool);
-        cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.gate_active);
-    }
-    cp.pool[cp.nmat] = static_cast<const unsigned char *>(c->b.up_pool);
-    cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.up_active);
-    cp.pool[cp.nmat] = static_cast<const unsigned char *>(c->b.downT_pool);
-    cp.active[cp.nmat++] = static_cast<unsigned char *>(c->b.down_active);
-    for (int k = cp.nmat; k < 3; ++k) { cp.pool[k] = cp.pool[0]; cp.active[k] = cp.active[0]; }
-    cp.row_bytes = row_bytes;
+    FusedRows fr;
+    fr.pool_u = static_cast<const unsigned char *>(c->b.up_pool);
+    fr.act_u = static_cast<unsigned char *>(c->b.up_active);
+    fr.pool_d = static_cast<const unsigned char *>(c->b.downT_pool);
+    fr.act_d = static_cast<unsigned char *>(c->b.down_active);
+    fr.pool_g = c->has_gate ? static_cast<const unsigned char *>(c->b.gate_pool) : fr.pool_u;
+    fr.act_g = c->has_gate ? static_cast<unsigned char *>(c->b.gate_active) : fr.act_u;
+    fr.row_bytes = row_bytes;
+    fr.has_gate = c->has_gate ? 1 : 0;
     const int G = mlp_grid();
     float *partials = static_cast<float *>(workspace);
     const int hint = (int)(n_hint < 0 ? 0 : (n_hint > c->I ? c->I : n_hint));
@@ -957,7 +950,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
                 attr_set = true;
             }
-            ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state, I,
+            ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, fr, mask, c->b.cur_mask, c->b.indices, c->b.state, I,
                                xt, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint);
             return ST_OK;
         };
@@ -966,7 +959,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
         static const bool split_off = [] { const char *v = getenv("ST_FUSED_SPLIT"); return v && atoi(v) == 0; }();
         // (only the fp16 instantiation of the split kernel fits the register file without spilling)
         // and it pays only when a block has enough rows to stream while the plan is worked out
-        const bool split = !split_off && c->dtype == ST_F16 && ngrp >= 2 && (ngrp & 1) == 0 && hint >= 6 * G &&
+        const bool split = !split_off && c->dtype != ST_F32 && ngrp >= 2 && (ngrp & 1) == 0 && hint >= 6 * G &&
                            I <= 8 * (TPB / 2) * kPlanMaxWords;
         // (four planning waves instead of eight leave less to arrive late, but take so much longer over the
         // plan that the kernel measures 21.1 us instead of 18.9 us)
@@ -974,6 +967,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
     rc = launch(cache_update_decode_kernel<TYPE, DecodeRows<TYPE>::value, PLANW, TPB>, static_cast<const TYPE *>(x), \
                 static_cast<TYPE *>(combined))
         if (c->dtype == ST_F32) ST_FUSED_LAUNCH(float, 0);
+        else if (c->dtype == ST_BF16 && split) ST_FUSED_LAUNCH(bf16_t, 8);
         else if (c->dtype == ST_BF16) ST_FUSED_LAUNCH(bf16_t, 0);
         else if (split) ST_FUSED_LAUNCH(f16_t, 8);
         else ST_FUSED_LAUNCH(f16_t, 0);

@@ -136,21 +136,9 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
 #pragma unroll
             for (int b = 0; b < NB; ++b) pg[k][b] = pu[k][b] = 0.f;
 #pragma unroll
-            for (int q = 0; q < CPT; ++q) {
-                float fg[VEC], fu[VEC];
-                unpack<T>(w.g[k][q], fg);
-                unpack<T>(w.u[k][q], fu);
+            for (int q = 0; q < CPT; ++q)
 #pragma unroll
-                for (int b = 0; b < NB; ++b) {
-                    float fx[VEC];
-                    unpack<T>(xr[b][q], fx);
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
-                        pg[k][b] = fmaf(fg[e], fx[e], pg[k][b]);
-                        pu[k][b] = fmaf(fu[e], fx[e], pu[k][b]);
-                    }
-                }
-            }
+                for (int b = 0; b < NB; ++b) dot_chunk<T>(w.g[k][q], w.u[k][q], xr[b][q], pg[k][b], pu[k][b]);
         }
 #pragma unroll
         for (int k = 0; k < RB; ++k)
@@ -191,14 +179,9 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
             const bool row_ok = row_of(bat, k) < n;
 #pragma unroll
             for (int q = 0; q < CPT; ++q) {
-                float fw[VEC];
-                unpack<T>(row_ok ? w.d[k][q] : zero4, fw);   // rows past the count may hold anything
+                const uint4 wsel = row_ok ? w.d[k][q] : zero4;   // rows past the count may hold anything
 #pragma unroll
-                for (int b = 0; b < NB; ++b) {
-                    const float hv = hs[grp][k][b];
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) acc[b][q][e] = fmaf(hv, fw[e], acc[b][q][e]);
-                }
+                for (int b = 0; b < NB; ++b) axpy_chunk<T>(hs[grp][k][b], wsel, acc[b][q]);
             }
         }
     };

@@ -57,6 +57,20 @@ template <> __device__ __forceinline__ void unpack<bf16_t>(const uint4 &v, float
     }
 }
 
+// One 32-bit word of a 2-byte type -> its two floats.
+template <typename T> __device__ __forceinline__ void unpack_word(uint32_t w, float *f);
+template <> __device__ __forceinline__ void unpack_word<f16_t>(uint32_t w, float *f)
+{
+    const half2_t h = __builtin_bit_cast(half2_t, w);
+    f[0] = (float)h.x;
+    f[1] = (float)h.y;
+}
+template <> __device__ __forceinline__ void unpack_word<bf16_t>(uint32_t w, float *f)
+{
+    f[0] = __uint_as_float(w << 16);
+    f[1] = __uint_as_float(w & 0xffff0000u);
+}
+
 // float -> storage element (round to nearest even).
 template <typename T> __device__ __forceinline__ T from_float(float f);
 template <> __device__ __forceinline__ float from_float<float>(float f) { return f; }
@@ -74,6 +88,58 @@ template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float f)
     u += 0x7fffu + ((u >> 16) & 1u);
     r.bits = (uint16_t)(u >> 16);
     return r;
+}
+
+// pg += <g, x>, pu += <u, x> over one 16-byte chunk, elements in order.  Every kernel whose results are
+// meant to agree bit for bit goes through this one function.  The 2-byte types use the two-element dot
+// product instructions (fp32 accumulate) named explicitly: left to itself the compiler forms them from
+// multiply-add chains in some places and not in others, and they round differently from the chain.
+template <typename T>
+__device__ __forceinline__ void dot_chunk(const uint4 &g, const uint4 &u, const uint4 &x, float &pg, float &pu)
+{
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w}, xw[4] = {x.x, x.y, x.z, x.w};
+    if constexpr (__is_same(T, float)) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            pg = fmaf(__uint_as_float(gw[e]), __uint_as_float(xw[e]), pg);
+            pu = fmaf(__uint_as_float(uw[e]), __uint_as_float(xw[e]), pu);
+        }
+    } else if constexpr (__is_same(T, bf16_t)) {
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bf16x2_t xv = __builtin_bit_cast(bf16x2_t, xw[j]);
+            pg = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, gw[j]), xv, pg, false);
+            pu = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, uw[j]), xv, pu, false);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const half2_t xv = __builtin_bit_cast(half2_t, xw[j]);
+            pg = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, gw[j]), xv, pg, false);
+            pu = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, uw[j]), xv, pu, false);
+        }
+    }
+}
+
+// acc[e] += h * w[e] over one 16-byte chunk (same word-at-a-time scheme).
+template <typename T> __device__ __forceinline__ void axpy_chunk(float h, const uint4 &w, float *acc)
+{
+    if constexpr (Elem<T>::kBytes == 4) {
+        float fw[4];
+        unpack<T>(w, fw);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = fmaf(h, fw[e], acc[e]);
+    } else {
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float fw[2];
+            unpack_word<T>(ww[j], fw);
+            acc[2 * j] = fmaf(h, fw[0], acc[2 * j]);
+            acc[2 * j + 1] = fmaf(h, fw[1], acc[2 * j + 1]);
+        }
+    }
 }
 
 template <typename T> __device__ __forceinline__ float to_float(T v);
