@@ -143,11 +143,12 @@ def sparse_mlp_forward(x: torch.Tensor, concat_weight: torch.Tensor, active_down
 
 def predictor_mask(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.Tensor, thr: float = 0.0,
                    ge: bool = True, return_scores: bool = False, out: Optional[torch.Tensor] = None,
-                   t_ws: Optional[torch.Tensor] = None):
+                   t_ws: Optional[torch.Tensor] = None, scores_out: Optional[torch.Tensor] = None):
     """mask[i] = any over rows b of ((x @ down^T) @ up^T)[b, i] >= thr  (``>`` when ``ge`` is False).
 
     x: [..., H]; down_weight: [r, H] (FastLoRAProjection.down.weight); up_weight: [I, r].
-    Returns a bool[I] tensor (and the fp32 scores [B, I] when ``return_scores``).
+    Returns a bool[I] tensor (and the fp32 scores [B, I] when ``return_scores`` or ``scores_out`` is given;
+    ``scores_out`` is a caller-owned buffer, for loops that must not allocate).
     thr = 0, ge = True is the reference's "naive" method (src/modeling_skip.py:206-207).
     """
     dev = require_gpu(x, down_weight, up_weight, out)
@@ -168,7 +169,14 @@ def predictor_mask(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.
         t_ws = torch.empty(B, r, dtype=torch.float32, device=dev)
     elif t_ws.dtype != torch.float32 or t_ws.numel() < B * r or not t_ws.is_cuda:
         raise ValueError("t_ws must be a float32 GPU tensor with at least B*r elements")
-    scores = torch.empty(B, I, dtype=torch.float32, device=dev) if return_scores else None
+    scores = None
+    if scores_out is not None:
+        if scores_out.dtype != torch.float32 or scores_out.numel() < B * I or not scores_out.is_cuda or \
+                not scores_out.is_contiguous():
+            raise ValueError("scores_out must be a contiguous float32 GPU tensor with at least B*I elements")
+        scores = scores_out.view(-1)[:B * I].view(B, I)
+    elif return_scores:
+        scores = torch.empty(B, I, dtype=torch.float32, device=dev)
     mask = out if out is not None else torch.empty(I, dtype=torch.bool, device=dev)
     if mask.dtype != torch.bool or mask.numel() != I or not mask.is_contiguous():
         raise ValueError("out must be a contiguous bool[I] tensor")
@@ -176,7 +184,7 @@ def predictor_mask(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.
         x2.data_ptr(), B, H, down_weight.data_ptr(), r, up_weight.data_ptr(), I, dtype_code(x2), float(thr), int(ge),
         t_ws.data_ptr(), scores.data_ptr() if scores is not None else None, mask.data_ptr(), current_stream_ptr(dev))
     _lib.check(rc, "st_predictor_mask")
-    return (mask, scores) if return_scores else mask
+    return (mask, scores) if (return_scores or scores_out is not None) else mask
 
 
 def predictor_scores(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.Tensor) -> torch.Tensor:
@@ -200,8 +208,17 @@ def _select_workspace(device: torch.device, B: int, I: int) -> torch.Tensor:
     return ws
 
 
+def select_workspace(device: torch.device, B: int, I: int) -> Optional[torch.Tensor]:
+    """A workspace for ``mask_select`` with B rows (None for B = 1), zeroed as the first call needs it.  For
+    callers that keep their own (one per stream of overlapping calls; allocate it outside graph capture)."""
+    if B <= 1:
+        return None
+    return torch.zeros(int(_lib.lib().st_mask_select_workspace_bytes(B, I)), dtype=torch.uint8, device=device)
+
+
 def mask_select(scores: torch.Tensor, method: str, k: int = 0, std_multiplier: float = 0.0,
-                out: Optional[torch.Tensor] = None, return_cutoff: bool = False):
+                out: Optional[torch.Tensor] = None, return_cutoff: bool = False,
+                workspace: Optional[torch.Tensor] = None):
     """Union over rows of the per-row selection on fp32 ``scores`` [B, I].
 
     ``topk``: the k largest scores of every row (src/modeling_skip.py:208-211; equal scores are taken in
@@ -219,7 +236,11 @@ def mask_select(scores: torch.Tensor, method: str, k: int = 0, std_multiplier: f
     if mask.dtype != torch.bool or mask.numel() != I or not mask.is_contiguous():
         raise ValueError("out must be a contiguous bool[I] tensor")
     cutoff = torch.empty(B, dtype=torch.float32, device=dev) if return_cutoff else None
-    ws = _select_workspace(dev, B, I) if B > 1 else None
+    ws = None
+    if B > 1:
+        ws = workspace if workspace is not None else _select_workspace(dev, B, I)
+        if ws.dtype != torch.uint8 or not ws.is_cuda:
+            raise ValueError("workspace must be a uint8 GPU tensor (see select_workspace)")
     rc = _lib.lib().st_mask_select(
         scores.data_ptr(), B, I, MASK_METHODS[method], int(k), float(std_multiplier), mask.data_ptr(),
         cutoff.data_ptr() if cutoff is not None else None, ws.data_ptr() if ws is not None else None,

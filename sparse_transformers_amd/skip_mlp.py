@@ -14,7 +14,7 @@ from typing import List, Optional, Sequence
 
 import torch
 
-from .ops import mask_select, predictor_mask, predictor_scores, sparse_mlp_forward
+from .ops import mask_select, predictor_mask, predictor_scores, select_workspace, sparse_mlp_forward
 from .weight_cache import WeightCache
 
 
@@ -53,12 +53,15 @@ class FastLoRAProjection:
 
     def mask(self, x: torch.Tensor, method: str = "naive", thr: float = 0.0, ge: bool = True, k: int = 0,
              std_multiplier: float = 0.0, out: Optional[torch.Tensor] = None,
-             t_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+             t_ws: Optional[torch.Tensor] = None, scores_ws: Optional[torch.Tensor] = None,
+             select_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Union-over-rows boolean mask, src/modeling_skip.py:204-214.
 
         ``naive`` (score >= 0) and ``threshold`` (score >= thr, or > thr) are fused into the predictor
         kernel.  ``topk`` and ``statistical_topk`` need a statistic of the whole row: the predictor kernel
-        leaves its fp32 scores and a selection kernel (one block per row) finishes.
+        leaves its fp32 scores and a selection kernel (one block per row) finishes.  ``scores_ws`` (float32,
+        B*I elements) and, for several rows, ``select_ws`` (``ops.select_workspace``) make the call
+        allocation-free.
         """
         if method == "naive":
             return predictor_mask(x, self.down_weight, self.up_weight, 0.0, True, out=out, t_ws=t_ws)
@@ -66,8 +69,12 @@ class FastLoRAProjection:
             return predictor_mask(x, self.down_weight, self.up_weight, thr, ge, out=out, t_ws=t_ws)
         if method not in ("topk", "statistical_topk"):
             raise ValueError(f"unknown sparsity method {method!r}")
-        scores = self.forward(x)
-        return mask_select(scores, method, k=k, std_multiplier=std_multiplier, out=out)
+        if scores_ws is None:
+            scores = self.forward(x)
+        else:   # caller-owned buffers: nothing is allocated (what a captured decode loop needs)
+            scores = predictor_mask(x, self.down_weight, self.up_weight, 0.0, True, out=out, t_ws=t_ws,
+                                    scores_out=scores_ws)[1]
+        return mask_select(scores, method, k=k, std_multiplier=std_multiplier, out=out, workspace=select_ws)
 
 
 def load_predictors(directory: str, num_layers: int, lora_pct: float, device=None, dtype=None) -> List["FastLoRAProjection"]:
@@ -122,13 +129,33 @@ class SparseDecodeLayer:
     """predictor -> mask -> cache update -> sparse MLP for one layer, all stream-ordered."""
 
     def __init__(self, predictor: FastLoRAProjection, cache: WeightCache, act: str = "silu", thr: float = 0.0,
-                 ge: bool = True):
+                 ge: bool = True, method: str = "threshold", k: int = 0, std_multiplier: float = 0.0):
+        """``method`` is one of SkipDecoderLayer's sparsity methods (src/modeling_skip.py:204-213): "naive",
+        "topk" (``k`` per row), "statistical_topk" (``std_multiplier`` = Normal(0,1).icdf(sparsity)), or
+        "threshold" (score >= ``thr``; ``ge=False`` for a strict comparison)."""
+        if method not in ("naive", "threshold", "topk", "statistical_topk"):
+            raise ValueError(f"unknown sparsity method {method!r}")
         self.predictor, self.cache, self.act, self.thr, self.ge = predictor, cache, act, thr, ge
+        self.method, self.k, self.std_multiplier = method, k, std_multiplier
         self.mask = torch.zeros(cache.intermediate_size, dtype=torch.bool, device=cache.device)
+        self._scores_ws: Optional[torch.Tensor] = None
+        self._select_ws: Optional[torch.Tensor] = None
+
+    def predict_mask(self, x_pred: torch.Tensor, t_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The layer's mask for ``x_pred`` into ``self.mask``.  The buffers the row-statistic methods need are
+        created on the first call with a given batch size (so: before a graph capture, not inside one)."""
+        if self.method in ("topk", "statistical_topk"):
+            B, I = x_pred.reshape(-1, x_pred.shape[-1]).size(0), self.cache.intermediate_size
+            if self._scores_ws is None or self._scores_ws.numel() < B * I:
+                self._scores_ws = torch.empty(B * I, dtype=torch.float32, device=self.cache.device)
+                self._select_ws = select_workspace(self.cache.device, B, I)
+        return self.predictor.mask(x_pred, self.method, self.thr, self.ge, k=self.k,
+                                   std_multiplier=self.std_multiplier, out=self.mask, t_ws=t_ws,
+                                   scores_ws=self._scores_ws, select_ws=self._select_ws)
 
     def compute_mask_and_update(self, x_pred: torch.Tensor, mask_override: Optional[torch.Tensor] = None,
                                 t_ws: Optional[torch.Tensor] = None) -> None:
-        self.predictor.mask(x_pred, "threshold", self.thr, self.ge, out=self.mask, t_ws=t_ws)
+        self.predict_mask(x_pred, t_ws)
         self.cache.update_active_weights_async(self.mask if mask_override is None else mask_override)
 
     def mlp(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -137,7 +164,7 @@ class SparseDecodeLayer:
     def step(self, x_pred: torch.Tensor, x: torch.Tensor, mask_override: Optional[torch.Tensor] = None,
              out: Optional[torch.Tensor] = None, t_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Predictor mask, then cache update and MLP in one call (``WeightCache.update_and_forward``)."""
-        self.predictor.mask(x_pred, "threshold", self.thr, self.ge, out=self.mask, t_ws=t_ws)
+        self.predict_mask(x_pred, t_ws)
         return self.cache.update_and_forward(self.mask if mask_override is None else mask_override, x, self.act,
                                              out=out)
 

@@ -118,3 +118,58 @@ def test_skip_mlp_module_surface():
     want, _ = oracle.mlp_forward(x.numpy(), oc.get_concat_weight(), oc.get_active_down_weight(), "silu", True)
     assert_close(out.cpu().numpy(), want, "float32", "SkipMLP")
     assert sorted(mlp.weight_cache.get_active_indices().cpu().tolist()) == idx.tolist()
+
+
+@pytest.mark.parametrize("method,B", [("topk", 1), ("topk", 3), ("statistical_topk", 1), ("statistical_topk", 2)])
+def test_row_statistic_methods_drive_the_stack(method, B):
+    """The stack stepped with the top-k / statistical masks of SkipDecoderLayer._compute_binary_mask:
+    masks (selected by the oracle from the same scores) and index order, outputs within tolerance, and a HIP-graph replay equal to
+    the eager step (the layer's score and selection buffers are created before the capture)."""
+    L, H, I, r = 3, 256, 640, 16
+    dtype, act = "float16", "silu"
+    k, z = 160, 0.5244
+    stack, oracles = _build(dtype, L, H, I, r, B, True, act, seed=9)
+    stack_g, _ = _build(dtype, L, H, I, r, B, True, act, seed=9)
+    for s in (stack, stack_g):
+        for layer in s.layers:
+            layer.method, layer.k, layer.std_multiplier = method, k, z
+    rng = np.random.default_rng(4)
+    xs = round_to(rng.standard_normal((8, B, H)).astype(np.float32), dtype)
+    xps = round_to(rng.standard_normal((8, L, B, H)).astype(np.float32), dtype)
+    tx = torch.from_numpy(xs).to(DEV, torch.float16)
+    txp = torch.from_numpy(xps).to(DEV, torch.float16)
+    stack_g.prepare(B)
+    stack_g.use_trace_masks = False
+    for t in range(8):
+        x = xs[t]
+        want_masks = []
+        for l, (oc, w) in enumerate(oracles):
+            # the selection is checked on the kernel's own fp32 scores (which are checked against the oracle's
+            # here and in test_gpu_predictor), so that a k-th score in a narrow gap cannot make the two diverge
+            s = stack.layers[l].predictor(txp[t, l]).cpu().numpy()
+            s_ref = oracle.predictor_scores(xps[t, l], w["A"], w["Bm"])
+            assert np.abs(s - s_ref).max() <= 4e-6 * np.abs(s_ref).max()
+            if method == "topk":
+                m = oracle.mask_topk(s, k)
+            else:
+                m, cut = oracle.mask_statistical(s, z)
+                assert (np.abs(s - cut[:, None]) > 1e-6 * np.abs(s).max()).all(), "score inside the guard band"
+            want_masks.append(m)
+            oc.update_active_weights(m)
+            y, _ = oracle.mlp_forward(x, oc.get_concat_weight(), oc.get_active_down_weight(), act, True)
+            x = round_to(y, dtype)
+        got = stack.decode_step(tx[t], [txp[t, l] for l in range(L)])
+        for l, (oc, _) in enumerate(oracles):
+            assert np.array_equal(stack.layers[l].mask.cpu().numpy(), want_masks[l]), (t, l)
+            assert stack.layers[l].cache.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist()
+        assert_close(got.float().cpu().numpy(), x, dtype, f"step {t}")
+        # the same step through the staged / captured path
+        if t == 1:
+            torch.cuda.synchronize()
+            stack_g.capture()
+        out_g = stack_g.step_staged(tx[t], txp[t], None, replay=t >= 1).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, got), t
+        for lg, le in zip(stack_g.layers, stack.layers):
+            assert torch.equal(lg.mask, le.mask)
+            assert torch.equal(lg.cache.get_active_indices(), le.cache.get_active_indices())
