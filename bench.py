@@ -259,6 +259,54 @@ def main():
         unfused = summarise()
         stack.fused = True
     L.st_profile_disable()
+
+    # ---- wall time of the two halves of a layer's chain, each replayed from a graph of its own (a kernel's
+    # ---- begin/end events cannot show what it costs inside the chain: an empty kernel already reads 4 us
+    # ---- between its two events, while a dependent empty kernel adds only 1.6 us to a replayed chain)
+    wall_parts = None
+    if use_graph and not args.overlap:
+        def part_predictor():
+            for l, layer in enumerate(stack.layers):
+                layer.predict_mask(stack.xp_stage[l], stack._t_ws)
+
+        def part_update_mlp():
+            x = stack.x_stage
+            for l, layer in enumerate(stack.layers):
+                out = stack._pingpong[l & 1]
+                if stack.fused:
+                    layer.cache.update_and_forward(stack.mask_stage[l], x, layer.act, out=out)
+                else:
+                    layer.cache.update_active_weights_async(stack.mask_stage[l])
+                    layer.cache.forward(x, layer.act, out=out)
+                x = out
+
+        wall_parts = {}
+        t_cur = min(t_lo + 2 + max(4, P // 4), W + K) - 1 if unfused is not None else t_lo + 1
+        steps_w = max(4, min(32, K // 2))
+        for name, fn in (("predictor", part_predictor), ("update_mlp", part_update_mlp)):
+            # walk the trace one step at a time (up, then down again) so every update has the configured churn
+            seq = list(range(t_cur + 1, min(t_cur + 1 + steps_w + 2, T)))
+            if len(seq) < steps_w + 2:
+                seq = list(range(t_cur - 1, t_cur - 3 - steps_w, -1))
+            stack.x_stage.copy_(x_in[seq[0]]); stack.xp_stage.copy_(x_pred[seq[0]]); stack.mask_stage.copy_(trace[seq[0]])
+            fn()
+            torch.cuda.synchronize()
+            gpart = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gpart):
+                fn()
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            for i, t in enumerate(seq[1:]):
+                if i == 1:
+                    ev0.record()
+                stack.x_stage.copy_(x_in[t]); stack.xp_stage.copy_(x_pred[t]); stack.mask_stage.copy_(trace[t])
+                gpart.replay()
+            ev1.record()
+            torch.cuda.synchronize()
+            wall_parts[name] = round(ev0.elapsed_time(ev1) * 1e3 / (len(seq) - 2) / layers, 2)
+            t_cur = seq[-1]
+            for layer in stack.layers:
+                layer.cache._dirty = True
+        wall_parts["whole_layer"] = round(ms_per_step * 1e3 / layers, 2)
     mats = 3 if wl.has_gate else 2
     alg_bytes = mats * n * H * esz                      # active-weight bytes one launch streams
     dom = "cache_update_decode" if "cache_update_decode" in per_kernel else \
@@ -296,6 +344,8 @@ def main():
                               "runs it fused into the decode kernel") if unfused else "standalone kernel",
         "stack_hbm_gbps": round(layers * alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
         "host_wall_ms_per_step": round(host_s * 1e3 / K, 5),
+        "wall_us_per_layer": wall_parts,
+        "wall_note": "graph replays of the predictor kernels alone, of update + MLP (+ reduce) alone, and of the whole step",
         "kernels_us": per_kernel,
         "kernels_us_unfused": unfused,
         "churn_mean": churn_mean,
