@@ -52,6 +52,20 @@ def build(verbose: bool = True) -> str:
     return LIB_PATH
 
 
+def build_capi_client(verbose: bool = True) -> str:
+    """tests/capi/capi_client: a C++ client of the C ABI that links nothing but the library and the HIP
+    runtime (run by tests/test_gpu_capi_client.py on the GPU box)."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "capi", "capi_client.cpp")
+    exe = os.path.join(root, "tests", "capi", "capi_client")
+    subprocess.run([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-o", exe, src, "-L" + HERE,
+                    "-lsparse_mlp_amd", "-Wl,-rpath,$ORIGIN/../../sparse_transformers_amd"], check=True)
+    if verbose:
+        print(f"[build] wrote {exe}", flush=True)
+    return exe
+
+
 if __name__ == "__main__":
     build()
+    build_capi_client()
     sys.exit(0)
