@@ -157,16 +157,16 @@ struct PlanShared {
 // 8-byte aligned, so masks are read as 8-byte words and indices as 16-byte vectors; both bookkeeping
 // buffers are requested together with the ticket, so the front costs one memory round trip.  MARK: the
 // dirty bitmap is kept on the fast path too.  `after_issue()` runs right after the front loads have
-// been issued.
+// been issued, `after_fill()` right after the first barrier (the front loads have arrived and been consumed).
 //
 // Barrier sequence: 1 after the LDS fill; 2 in the diff scan;
 // [unchanged mask: done]; 1 after the lists; 1 after phases 1 and 2; [surplus removals: 1 after phase 3,
 // 2 in the compaction scan, 1 after the compaction].
-template <bool VEC, int PT, bool MARK, bool SUB, typename F>
+template <bool VEC, int PT, bool MARK, bool SUB, typename F, typename F2>
 __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, PlanShared *ps,
                                            const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2,
                                            int32_t *__restrict__ indices2, int32_t *__restrict__ state, int I,
-                                           const int tid, F after_issue)
+                                           const int tid, F after_issue, F2 after_fill)
 {
     constexpr int TPB = PT;
     uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);  // index -> position
@@ -267,6 +267,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
     // times longer, and the whole plan hangs on them)
     if constexpr (SUB) lds_barrier();
     else sync();
+    after_fill();
     ST_TL(2);
     for (int p = tid; p < n; p += TPB) pos_l[idx_l[p]] = (uint16_t)p;
 
@@ -485,7 +486,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     __shared__ PlanShared ps;
     const int tid = threadIdx.x;
     PlanView pv;
-    cache_plan<VEC, TPB, false, false>(pv, smem, &ps, new_mask, cur_mask2, indices2, state, I, tid, [] {});
+    cache_plan<VEC, TPB, false, false>(pv, smem, &ps, new_mask, cur_mask2, indices2, state, I, tid, [] {}, [] {});
     if (!pv.changed) {
         plan_finish(pv, state);
         return;
@@ -548,7 +549,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
 // update followed by forward.
 // Rows are dealt to blocks round-robin: row(bat, k) = blk + G * (grp + ngrp * (bat * RB + k)).
 // ---------------------------------------------------------------------------
-template <typename T, int RB, int PLANW, int TPB>
+template <typename T, int RB, int PLANW, int TPB, bool AHEAD = false>
 __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     FusedRows fr, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
     int32_t *__restrict__ state, int I, const T *__restrict__ x, int H, T *__restrict__ combined, long ldc,
@@ -588,13 +589,16 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     constexpr bool SPLIT = PLANW > 0;
     constexpr int PT = SPLIT ? PLANW * kWave : TPB;
     const bool streams_ahead = SPLIT && tid < TPB - PT;
-    const int n_spec = SPLIT ? (n_hint < I ? n_hint : I) : 0;
+    // AHEAD (all waves plan): every wave requests its first batch on the host's guess as soon as the plan's
+    // own loads are in, and goes on planning with those requests in flight.  Wherever the plan code makes
+    // a wave wait for its outstanding loads it waits for the rows too, so this pays when a block's rows
+    // arrive in less time than the plan takes (few active rows per block).
+    static_assert(!(AHEAD && SPLIT), "the two ways of streaming ahead exclude each other");
+    const int n_spec = (SPLIT || AHEAD) ? (n_hint < I ? n_hint : I) : 0;
     __shared__ PlanShared plan_shared;
     PlanView pv;
     if (SPLIT && tid == 0) plan_shared.sub_count = 0;
-    if (streams_ahead) {
-        xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff);
-        lds_barrier();   // (A) the plan's own loads have arrived (inside cache_plan, after the LDS fill)
+    auto speculate = [&]() __attribute__((always_inline)) {
         if (wave_live && n_spec > 0) {
 #pragma unroll
             for (int k = 0; k < RB; ++k) {
@@ -605,6 +609,11 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
                 if (has_gate) wg[k] = ld16_stream(act_g + ro);
             }
         }
+    };
+    if (streams_ahead) {
+        xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff);
+        lds_barrier();   // (A) the plan's own loads have arrived (inside cache_plan, after the LDS fill)
+        speculate();
         lds_barrier();   // (B) the plan is finished
         plan_adopt(pv, smem, &plan_shared, I);
     } else {
@@ -613,7 +622,8 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
         // memory requests
         cache_plan<true, PT, true, SPLIT>(pv, smem, &plan_shared, new_mask, cur_mask2, indices2, state, I,
                                           SPLIT ? tid - (TPB - PT) : tid,
-                                          [&] { xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff); });
+                                          [&] { xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff); },
+                                          [&] { if constexpr (AHEAD) speculate(); });
         if (SPLIT) {
             plan_publish(pv, &plan_shared);
             lds_barrier();   // (B)
@@ -645,7 +655,7 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
             wg[k] = has_gate ? ld16_stream((pooled ? pool_g : act_g) + ro) : zero4;
         };
         if (wave_live) {
-            const bool spec = streams_ahead && bat == 0 && n_spec > 0;   // uniform over the wave
+            const bool spec = (streams_ahead || AHEAD) && bat == 0 && n_spec > 0;   // uniform over the wave
 #pragma unroll
             for (int k = 0; k < RB; ++k) request(k, spec);   // static slot numbers keep the rows in registers
             if (spec && !has_gate) {
@@ -963,14 +973,23 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
                            I <= 8 * (TPB / 2) * kPlanMaxWords;
         // (four planning waves instead of eight leave less to arrive late, but take so much longer over the
         // plan that the kernel measures 21.1 us instead of 18.9 us)
-#define ST_FUSED_LAUNCH(TYPE, PLANW)                                                                   \
-    rc = launch(cache_update_decode_kernel<TYPE, DecodeRows<TYPE>::value, PLANW, TPB>, static_cast<const TYPE *>(x), \
-                static_cast<TYPE *>(combined))
-        if (c->dtype == ST_F32) ST_FUSED_LAUNCH(float, 0);
-        else if (c->dtype == ST_BF16 && split) ST_FUSED_LAUNCH(bf16_t, 8);
-        else if (c->dtype == ST_BF16) ST_FUSED_LAUNCH(bf16_t, 0);
-        else if (split) ST_FUSED_LAUNCH(f16_t, 8);
-        else ST_FUSED_LAUNCH(f16_t, 0);
+        // few rows per block: all waves plan, with their rows requested ahead
+        static const int ahead_env = [] { const char *v = getenv("ST_FUSED_AHEAD"); return v ? atoi(v) : -1; }();
+        const bool ahead = !split && hint > 0 && (ahead_env < 0 ? hint < 6 * G : ahead_env != 0);
+        // (the rows in flight per group do not change which rows a group sums or in which order, so the
+        // ahead variant is free to keep three: enough for fewer than 6 rows per block, and it leaves the
+        // registers the plan needs beside them)
+#define ST_FUSED_LAUNCH(TYPE, PLANW, AHEAD)                                                            \
+    rc = launch(cache_update_decode_kernel<TYPE, (AHEAD) ? 3 : DecodeRows<TYPE>::value, PLANW, TPB, AHEAD>, \
+                static_cast<const TYPE *>(x), static_cast<TYPE *>(combined))
+        if (c->dtype == ST_F32 && ahead) ST_FUSED_LAUNCH(float, 0, true);
+        else if (c->dtype == ST_F32) ST_FUSED_LAUNCH(float, 0, false);
+        else if (c->dtype == ST_BF16 && split) ST_FUSED_LAUNCH(bf16_t, 8, false);
+        else if (c->dtype == ST_BF16 && ahead) ST_FUSED_LAUNCH(bf16_t, 0, true);
+        else if (c->dtype == ST_BF16) ST_FUSED_LAUNCH(bf16_t, 0, false);
+        else if (split) ST_FUSED_LAUNCH(f16_t, 8, false);
+        else if (ahead) ST_FUSED_LAUNCH(f16_t, 0, true);
+        else ST_FUSED_LAUNCH(f16_t, 0, false);
 #undef ST_FUSED_LAUNCH
         if (rc != ST_OK) return rc;
     }
