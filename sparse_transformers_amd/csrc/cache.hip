@@ -158,6 +158,8 @@ struct PlanShared {
 // buffers are requested together with the ticket, so the front costs one memory round trip.  MARK: the
 // dirty bitmap is kept on the fast path too.  `after_issue()` runs right after the front loads have
 // been issued, `after_fill()` right after the first barrier (the front loads have arrived and been consumed).
+// idx_cap: only that many positions of the index lists are fetched up front (the rest follows if the count
+// turns out larger).
 //
 // Barrier sequence: 1 after the LDS fill; 2 in the diff scan;
 // [unchanged mask: done]; 1 after the lists; 1 after phases 1 and 2; [surplus removals: 1 after phase 3,
@@ -166,7 +168,7 @@ template <bool VEC, int PT, bool MARK, bool SUB, typename F, typename F2>
 __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, PlanShared *ps,
                                            const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2,
                                            int32_t *__restrict__ indices2, int32_t *__restrict__ state, int I,
-                                           const int tid, F after_issue, F2 after_fill)
+                                           const int idx_cap, const int tid, F after_issue, F2 after_fill)
 {
     constexpr int TPB = PT;
     uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);  // index -> position
@@ -214,10 +216,12 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
                 v_new[w] = *reinterpret_cast<const uint64_t *>(new_mask + e);
                 v_cur0[w] = *reinterpret_cast<const uint64_t *>(cur_mask2 + e);
                 v_cur1[w] = *reinterpret_cast<const uint64_t *>(cur_mask2 + (size_t)I + e);
-                v_i0a[w] = *reinterpret_cast<const int4 *>(indices2 + e);
-                v_i0b[w] = *reinterpret_cast<const int4 *>(indices2 + e + 4);
-                v_i1a[w] = *reinterpret_cast<const int4 *>(indices2 + (size_t)I + e);
-                v_i1b[w] = *reinterpret_cast<const int4 *>(indices2 + (size_t)I + e + 4);
+                if (e < idx_cap) {   // positions the caller expects to be in use (a multiple of 8, or all)
+                    v_i0a[w] = *reinterpret_cast<const int4 *>(indices2 + e);
+                    v_i0b[w] = *reinterpret_cast<const int4 *>(indices2 + e + 4);
+                    v_i1a[w] = *reinterpret_cast<const int4 *>(indices2 + (size_t)I + e);
+                    v_i1b[w] = *reinterpret_cast<const int4 *>(indices2 + (size_t)I + e + 4);
+                }
             }
         }
         n_both[0] = state[ST_STATE_N_BUF0];
@@ -241,13 +245,15 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
             if (e < e1) {
                 w_new[w] = nonzero_bytes(v_new[w]);
                 w_cur[w] = nonzero_bytes(ep ? v_cur1[w] : v_cur0[w]);
-                const int4 a = ep ? v_i1a[w] : v_i0a[w], b4 = ep ? v_i1b[w] : v_i0b[w];
-                uint4 packed;
-                packed.x = (uint32_t)(a.x & 0xffff) | ((uint32_t)a.y << 16);
-                packed.y = (uint32_t)(a.z & 0xffff) | ((uint32_t)a.w << 16);
-                packed.z = (uint32_t)(b4.x & 0xffff) | ((uint32_t)b4.y << 16);
-                packed.w = (uint32_t)(b4.z & 0xffff) | ((uint32_t)b4.w << 16);
-                *reinterpret_cast<uint4 *>(idx_l + e) = packed;
+                if (e < idx_cap) {
+                    const int4 a = ep ? v_i1a[w] : v_i0a[w], b4 = ep ? v_i1b[w] : v_i0b[w];
+                    uint4 packed;
+                    packed.x = (uint32_t)(a.x & 0xffff) | ((uint32_t)a.y << 16);
+                    packed.y = (uint32_t)(a.z & 0xffff) | ((uint32_t)a.w << 16);
+                    packed.z = (uint32_t)(b4.x & 0xffff) | ((uint32_t)b4.y << 16);
+                    packed.w = (uint32_t)(b4.z & 0xffff) | ((uint32_t)b4.w << 16);
+                    *reinterpret_cast<uint4 *>(idx_l + e) = packed;
+                }
                 *reinterpret_cast<uint4 *>(pos_l + e) = make_uint4(0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu);
             }
         }
@@ -269,6 +275,11 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
     else sync();
     after_fill();
     ST_TL(2);
+    if (VEC && n > idx_cap) {   // more positions in use than the caller expected: fetch the rest (one more round trip)
+        const int32_t *indices = indices2 + (size_t)ep * I;
+        for (int p = idx_cap + tid; p < n; p += TPB) idx_l[p] = (uint16_t)indices[p];
+        sync();
+    }
     for (int p = tid; p < n; p += TPB) pos_l[idx_l[p]] = (uint16_t)p;
 
     // ---- diff: contiguous element range per thread keeps the lists ascending
@@ -486,7 +497,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     __shared__ PlanShared ps;
     const int tid = threadIdx.x;
     PlanView pv;
-    cache_plan<VEC, TPB, false, false>(pv, smem, &ps, new_mask, cur_mask2, indices2, state, I, tid, [] {}, [] {});
+    cache_plan<VEC, TPB, false, false>(pv, smem, &ps, new_mask, cur_mask2, indices2, state, I, I, tid, [] {}, [] {});
     if (!pv.changed) {
         plan_finish(pv, state);
         return;
@@ -553,7 +564,7 @@ template <typename T, int RB, int PLANW, int TPB, bool AHEAD = false>
 __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     FusedRows fr, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
     int32_t *__restrict__ state, int I, const T *__restrict__ x, int H, T *__restrict__ combined, long ldc,
-    float *__restrict__ partials, int act, int gs_log2, int plan_bytes, int n_hint)
+    float *__restrict__ partials, int act, int gs_log2, int plan_bytes, int n_hint, int idx_cap)
 {
     constexpr int VEC = Elem<T>::kVec;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -621,7 +632,7 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
         // waves synchronise among themselves, so the streaming waves are free to stall on their own
         // memory requests
         cache_plan<true, PT, true, SPLIT>(pv, smem, &plan_shared, new_mask, cur_mask2, indices2, state, I,
-                                          SPLIT ? tid - (TPB - PT) : tid,
+                                          idx_cap, SPLIT ? tid - (TPB - PT) : tid,
                                           [&] { xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff); },
                                           [&] { if constexpr (AHEAD) speculate(); });
         if (SPLIT) {
@@ -951,6 +962,10 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
     const int G = mlp_grid();
     float *partials = static_cast<float *>(workspace);
     const int hint = (int)(n_hint < 0 ? 0 : (n_hint > c->I ? c->I : n_hint));
+    // The plan needs the index list only up to the count in use, which lives on the device: blocks fetch the
+    // first `idx_cap` positions with their other bookkeeping loads (a quarter more than the caller's guess)
+    // and the rest, if the guess was too low, in a second round trip.
+    const int idx_cap = hint > 0 && hint + hint / 4 + 64 < I ? (hint + hint / 4 + 64 + 7) & ~7 : I;
     {
         ProfScope ps(ST_K_CACHE_UPDATE_DECODE, s);
         auto launch = [&](auto kern, auto *xt, auto *ct) -> int {
@@ -961,7 +976,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
                 attr_set = true;
             }
             ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, fr, mask, c->b.cur_mask, c->b.indices, c->b.state, I,
-                               xt, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint);
+                               xt, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint, idx_cap);
             return ST_OK;
         };
         int rc;

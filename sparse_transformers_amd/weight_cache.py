@@ -159,11 +159,13 @@ class WeightCache:
 
     # ---------------------------------------------------------------- fast path
     def update_and_forward(self, mask: torch.Tensor, x: torch.Tensor, act: str = "silu",
-                           out: Optional[torch.Tensor] = None, combined: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           out: Optional[torch.Tensor] = None, combined: Optional[torch.Tensor] = None,
+                           n_hint: Optional[int] = None) -> torch.Tensor:
         """``update_active_weights(mask)`` followed by the sparse MLP on x, enqueued as one call and never
         touching the host.  For one row of x this is a single kernel that takes the rows whose index
         changed straight from the pool (and writes them back to the active buffers on the way); the
-        cache state and the result equal those of the two separate calls bit for bit."""
+        cache state and the result equal those of the two separate calls bit for bit.  ``n_hint`` (default:
+        the last count the host saw) only steers what the kernel requests before it knows the true count."""
         m = self._mask_arg(mask)
         H = self.hidden_size
         x2 = x.reshape(-1, H)
@@ -178,7 +180,8 @@ class WeightCache:
         if act not in _lib.ACT_CODES:
             raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
         rc = _lib.lib().st_cache_update_forward(
-            self._h, m.data_ptr(), x2.data_ptr(), B, int(self._host_state[_lib.STATE_N_ACTIVE]), out.data_ptr(),
+            self._h, m.data_ptr(), x2.data_ptr(), B,
+            int(self._host_state[_lib.STATE_N_ACTIVE]) if n_hint is None else int(n_hint), out.data_ptr(),
             combined.data_ptr() if combined is not None else None, combined.stride(0) if combined is not None else 0,
             ws.data_ptr(), ws.numel(), _lib.ACT_CODES[act], current_stream_ptr(self.device))
         _lib.check(rc, "st_cache_update_forward")

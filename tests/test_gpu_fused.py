@@ -131,3 +131,28 @@ def test_fused_call_with_several_rows_takes_the_two_kernel_path():
         yp = plain.forward(x, "relu")
         assert torch.equal(yf, yp), t
     _same_state(fused, plain, "end")
+
+
+@pytest.mark.parametrize("dtype,H,I,n0", [("float16", 3072, 8192, 2867), ("bfloat16", 4096, 4096, 400),
+                                          ("float32", 2048, 4096, 1500)])
+def test_fused_result_does_not_depend_on_the_hint(dtype, H, I, n0):
+    """The caller's guess of the active count decides which kernel variant runs, what is requested before
+    the plan is known and how much of the index list is fetched up front; a wrong guess (far too low: the
+    rest of the list is fetched in a second round trip; far too high; zero = unknown) must change nothing."""
+    rng = np.random.default_rng(17)
+    m = np.zeros(I, bool)
+    m[rng.permutation(I)[:n0]] = True
+    fused, plain, _, g = _pair(I, H, dtype, True, 5, torch.from_numpy(m))
+    tdt = getattr(torch, dtype)
+    for step, hint in enumerate((0, 1, 8, n0 // 3, n0 - 1, n0, n0 + 1000, I, 2 * I, 40, n0)):
+        flip = rng.permutation(I)[: max(2, n0 // 8)]
+        m = m.copy()
+        m[flip] = ~m[flip]
+        md = torch.from_numpy(m).to(DEV)
+        x = torch.randn(1, H, generator=g).to(tdt).to(DEV)
+        yf = fused.update_and_forward(md, x, "silu", n_hint=hint)
+        plain.update_active_weights_async(md)
+        yp = plain.forward(x, "silu")
+        torch.cuda.synchronize()
+        assert torch.equal(yf, yp), (step, hint)
+        _same_state(fused, plain, step)
