@@ -491,13 +491,14 @@ template <bool VEC, int TPB>
 __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const uint8_t *__restrict__ new_mask,
                                                                     uint8_t *__restrict__ cur_mask2,
                                                                     int32_t *__restrict__ indices2,
-                                                                    int32_t *__restrict__ state, int I, int gs_log2)
+                                                                    int32_t *__restrict__ state, int I, int gs_log2,
+                                                                    int idx_cap)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ PlanShared ps;
     const int tid = threadIdx.x;
     PlanView pv;
-    cache_plan<VEC, TPB, false, false>(pv, smem, &ps, new_mask, cur_mask2, indices2, state, I, I, tid, [] {}, [] {});
+    cache_plan<VEC, TPB, false, false>(pv, smem, &ps, new_mask, cur_mask2, indices2, state, I, idx_cap, tid, [] {}, [] {});
     if (!pv.changed) {
         plan_finish(pv, state);
         return;
@@ -822,6 +823,7 @@ extern "C" st_cache *st_cache_create(const st_cache_buffers *bufs, int64_t I, in
         delete c;
         return fail("hipHostMalloc failed");
     }
+    for (int i = 0; i < ST_STATE_WORDS; ++i) c->host_state[i] = 0;
     return c;
 }
 
@@ -894,6 +896,10 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     const bool vec = aligned && I <= 8 * tpb * kPlanMaxWords;
     int gs_log2 = 6;
     while ((1 << gs_log2) < chunks && (1 << gs_log2) < tpb) ++gs_log2;
+    // how much of the index list the blocks fetch up front: a quarter more than the count the host saw
+    // last (st_cache_sync_state), everything when it has seen none
+    const int seen = c->host_state[ST_STATE_N_ACTIVE];
+    const int idx_cap = seen > 0 && seen + seen / 4 + 64 < I ? (seen + seen / 4 + 64 + 7) & ~7 : I;
     {
         ProfScope ps(ST_K_CACHE_UPDATE, s);
         auto launch = [&](auto kern) -> int {
@@ -904,7 +910,7 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
                 attr_set = true;
             }
             ST_LAUNCH(ps, kern, dim3(grid), dim3(tpb), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state,
-                               I, gs_log2);
+                               I, gs_log2, idx_cap);
             return ST_OK;
         };
         int rc;
