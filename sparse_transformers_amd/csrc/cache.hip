@@ -990,7 +990,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
         static const bool split_off = [] { const char *v = getenv("ST_FUSED_SPLIT"); return v && atoi(v) == 0; }();
         // (only the fp16 instantiation of the split kernel fits the register file without spilling)
         // and it pays only when a block has enough rows to stream while the plan is worked out
-        const bool split = !split_off && c->dtype != ST_F32 && ngrp >= 2 && (ngrp & 1) == 0 && hint >= 6 * G &&
+        const bool split = !split_off && ngrp >= 2 && (ngrp & 1) == 0 && hint >= 6 * G &&
                            I <= 8 * (TPB / 2) * kPlanMaxWords;
         // (four planning waves instead of eight leave less to arrive late, but take so much longer over the
         // plan that the kernel measures 21.1 us instead of 18.9 us)
@@ -1003,7 +1003,8 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
 #define ST_FUSED_LAUNCH(TYPE, PLANW, AHEAD)                                                            \
     rc = launch(cache_update_decode_kernel<TYPE, (AHEAD) ? 3 : DecodeRows<TYPE>::value, PLANW, TPB, AHEAD>, \
                 static_cast<const TYPE *>(x), static_cast<TYPE *>(combined))
-        if (c->dtype == ST_F32 && ahead) ST_FUSED_LAUNCH(float, 0, true);
+        if (c->dtype == ST_F32 && split) ST_FUSED_LAUNCH(float, 8, false);
+        else if (c->dtype == ST_F32 && ahead) ST_FUSED_LAUNCH(float, 0, true);
         else if (c->dtype == ST_F32) ST_FUSED_LAUNCH(float, 0, false);
         else if (c->dtype == ST_BF16 && split) ST_FUSED_LAUNCH(bf16_t, 8, false);
         else if (c->dtype == ST_BF16 && ahead) ST_FUSED_LAUNCH(bf16_t, 0, true);
