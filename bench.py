@@ -29,8 +29,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by
 # what the same counter reads for a 256 MiB copy; see profiles/decode_traffic_llama3b_stack_fp16.md
-MEASURED_TRAFFIC_BYTES = {("llama3b_stack_fp16", "mlp_decode"): 53_040_000 + 3_145_728,
-                          ("llama3b_stack_fp16", "cache_update_decode"): 56_909_824 + 8_297_779}
+MEASURED_TRAFFIC_BYTES = {("llama3b_stack_fp16", "mlp_decode"): 53_169_357 + 3_145_728,
+                          ("llama3b_stack_fp16", "cache_update_decode"): 56_787_558 + 8_574_259}
 
 
 def parse_args():
