@@ -47,8 +47,8 @@ def parse_args():
     ap.add_argument("--no-fused", action="store_true",
                     help="cache update and MLP as two kernels per layer instead of the fused update+decode kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-layers", type=int, default=2)
-    ap.add_argument("--cpu-steps", type=int, default=24)
+    ap.add_argument("--cpu-layers", type=int, default=4)
+    ap.add_argument("--cpu-steps", type=int, default=300)
     ap.add_argument("--profile-steps", type=int, default=32)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a known-size reference for rocprofv3 --pmc)")
