@@ -248,34 +248,36 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
     ST_TL(6);
 }
 
-// out[b, c] = sum over blocks of partials[blk][b][c], fixed order.
-template <typename T>
+// out[b, c] = sum over blocks of partials[blk][b][c], fixed order.  CW threads share a row of 4 * CW columns,
+// 256 / CW groups of threads take the partial rows round-robin, U rows per thread requested together (one
+// memory round trip for G <= 256).
+template <typename T, int CW>
 __global__ __launch_bounds__(256) void mlp_reduce_kernel(const float *__restrict__ partials, int G, int NB, int B,
                                                          int H, T *__restrict__ out)
 {
-    __shared__ float4 red[16][16];
-    const int tid = threadIdx.x, q = tid & 15, rg = tid >> 4;
+    constexpr int RG = 256 / CW, U = 256 / RG;
+    __shared__ float4 red[RG][CW];
+    const int tid = threadIdx.x, q = tid % CW, rg = tid / CW;
     const int b = blockIdx.y;
-    const int col = blockIdx.x * 64 + q * 4;
+    const int col = blockIdx.x * (4 * CW) + q * 4;
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     if (col < H) {
-        // 16 partial rows per thread are requested together (one memory round trip for G <= 256)
-        for (int blk0 = rg; blk0 < G; blk0 += 16 * 16) {
-            float4 v[16];
+        for (int blk0 = rg; blk0 < G; blk0 += RG * U) {
+            float4 v[U];
 #pragma unroll
-            for (int k = 0; k < 16; ++k) {
-                const int blk = blk0 + 16 * k;
+            for (int k = 0; k < U; ++k) {
+                const int blk = blk0 + RG * k;
                 v[k] = blk < G ? *reinterpret_cast<const float4 *>(partials + ((size_t)blk * NB + b) * H + col)
                                : make_float4(0.f, 0.f, 0.f, 0.f);
             }
 #pragma unroll
-            for (int k = 0; k < 16; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
+            for (int k = 0; k < U; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
         }
     }
     red[rg][q] = s;
     __syncthreads();
     if (rg == 0 && col < H) {
-        for (int k = 1; k < 16; ++k) {
+        for (int k = 1; k < RG; ++k) {
             const float4 v = red[k][q];
             s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
         }
@@ -289,6 +291,10 @@ __global__ __launch_bounds__(256) void mlp_reduce_kernel(const float *__restrict
 // host side
 // ---------------------------------------------------------------------------
 constexpr int kMaxLds = 160 * 1024;
+#ifndef ST_REDUCE_CW
+#define ST_REDUCE_CW 8
+#endif
+constexpr int kReduceCW = ST_REDUCE_CW;   // threads per row of the reduce kernel: 4 * CW columns per block
 
 struct MlpLaunch {
     const void *x; int B; int H;
@@ -331,8 +337,8 @@ static int launch_inst(const MlpLaunch &a, int b0, int bcount)
     T *out = static_cast<T *>(a.out) + (size_t)b0 * a.H;
     {
         ProfScope ps(ST_K_MLP_REDUCE, a.stream);
-        ST_LAUNCH(ps, mlp_reduce_kernel<T>, dim3((a.H + 63) / 64, bcount), dim3(256), 0, a.stream, a.partials,
-                           a.G, NB, bcount, a.H, out);
+        ST_LAUNCH(ps, (mlp_reduce_kernel<T, kReduceCW>), dim3((a.H + 4 * kReduceCW - 1) / (4 * kReduceCW), bcount),
+                  dim3(256), 0, a.stream, a.partials, a.G, NB, bcount, a.H, out);
     }
     ST_HIP(hipGetLastError());
     return ST_OK;
@@ -417,15 +423,16 @@ int launch_mlp_reduce(int dtype, const float *partials, int G, int NB, int bcoun
                       hipStream_t stream)
 {
     ProfScope ps(ST_K_MLP_REDUCE, stream);
-    const dim3 grid((H + 63) / 64, bcount);
+    constexpr int CW = kReduceCW;
+    const dim3 grid((H + 4 * CW - 1) / (4 * CW), bcount);
     if (dtype == ST_F32)
-        ST_LAUNCH(ps, mlp_reduce_kernel<float>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+        ST_LAUNCH(ps, (mlp_reduce_kernel<float, CW>), grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
                            static_cast<float *>(out));
     else if (dtype == ST_F16)
-        ST_LAUNCH(ps, mlp_reduce_kernel<f16_t>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+        ST_LAUNCH(ps, (mlp_reduce_kernel<f16_t, CW>), grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
                            static_cast<f16_t *>(out));
     else
-        ST_LAUNCH(ps, mlp_reduce_kernel<bf16_t>, grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+        ST_LAUNCH(ps, (mlp_reduce_kernel<bf16_t, CW>), grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
                            static_cast<bf16_t *>(out));
     ST_HIP(hipGetLastError());
     return ST_OK;
