@@ -251,11 +251,12 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
 // out[b, c] = sum over blocks of partials[blk][b][c], fixed order.  CW threads share a row of 4 * CW columns,
 // 256 / CW groups of threads take the partial rows round-robin, U rows per thread requested together (one
 // memory round trip for G <= 256).
+constexpr int kReduceThreads = 128;   // measured against 64 / 256 / 512 threads per block
 template <typename T, int CW>
-__global__ __launch_bounds__(256) void mlp_reduce_kernel(const float *__restrict__ partials, int G, int NB, int B,
+__global__ __launch_bounds__(kReduceThreads) void mlp_reduce_kernel(const float *__restrict__ partials, int G, int NB, int B,
                                                          int H, T *__restrict__ out)
 {
-    constexpr int RG = 256 / CW, U = 256 / RG;
+    constexpr int RG = kReduceThreads / CW, U = 256 / RG;
     __shared__ float4 red[RG][CW];
     const int tid = threadIdx.x, q = tid % CW, rg = tid / CW;
     const int b = blockIdx.y;
@@ -338,7 +339,7 @@ static int launch_inst(const MlpLaunch &a, int b0, int bcount)
     {
         ProfScope ps(ST_K_MLP_REDUCE, a.stream);
         ST_LAUNCH(ps, (mlp_reduce_kernel<T, kReduceCW>), dim3((a.H + 4 * kReduceCW - 1) / (4 * kReduceCW), bcount),
-                  dim3(256), 0, a.stream, a.partials, a.G, NB, bcount, a.H, out);
+                  dim3(kReduceThreads), 0, a.stream, a.partials, a.G, NB, bcount, a.H, out);
     }
     ST_HIP(hipGetLastError());
     return ST_OK;
@@ -426,13 +427,13 @@ int launch_mlp_reduce(int dtype, const float *partials, int G, int NB, int bcoun
     constexpr int CW = kReduceCW;
     const dim3 grid((H + 4 * CW - 1) / (4 * CW), bcount);
     if (dtype == ST_F32)
-        ST_LAUNCH(ps, (mlp_reduce_kernel<float, CW>), grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+        ST_LAUNCH(ps, (mlp_reduce_kernel<float, CW>), grid, dim3(kReduceThreads), 0, stream, partials, G, NB, bcount, H,
                            static_cast<float *>(out));
     else if (dtype == ST_F16)
-        ST_LAUNCH(ps, (mlp_reduce_kernel<f16_t, CW>), grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+        ST_LAUNCH(ps, (mlp_reduce_kernel<f16_t, CW>), grid, dim3(kReduceThreads), 0, stream, partials, G, NB, bcount, H,
                            static_cast<f16_t *>(out));
     else
-        ST_LAUNCH(ps, (mlp_reduce_kernel<bf16_t, CW>), grid, dim3(256), 0, stream, partials, G, NB, bcount, H,
+        ST_LAUNCH(ps, (mlp_reduce_kernel<bf16_t, CW>), grid, dim3(kReduceThreads), 0, stream, partials, G, NB, bcount, H,
                            static_cast<bf16_t *>(out));
     ST_HIP(hipGetLastError());
     return ST_OK;

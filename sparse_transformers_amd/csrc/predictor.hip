@@ -80,13 +80,14 @@ __global__ __launch_bounds__(kPredDownThreads) void predictor_down_kernel(const 
     }
 }
 
-constexpr int kPredUpThreads = 256;
-// rows of Bm a wave owns: fewer when a whole wave is needed per row, to keep the accumulators in registers
-constexpr int pred_rows_per_wave(int lpr) { return lpr >= 64 ? 4 : (lpr >= 32 ? 8 : 16); }
+constexpr int kPredUpThreads = 256;   // (128-thread blocks measure the same)
+// rows of Bm a wave owns per pass: four for every row length.  (More rows per wave mean fewer blocks; with 16
+// the 8192-row matrix made 128 blocks and a decode layer measured 1 us slower than with the 512 blocks of 4.)
+constexpr int pred_rows_per_wave(int) { return 4; }
 constexpr int kPredUpBTile = 8;
 
 // LPR lanes share one row of Bm (LPR >= r/VEC unless the row needs several
-// passes); a wave owns 16 consecutive rows and issues the loads of all of them
+// passes); a wave owns RPW consecutive rows and issues the loads of all of them
 // before the rank-r intermediate is staged in LDS.
 template <typename T, int LPR, int RPW>
 __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_kernel(const float *__restrict__ t, int B, int r,
@@ -188,21 +189,18 @@ template <typename T, int LPR, int RPW>
 static void launch_up_rpw(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
                           float *scores, uint8_t *mask, hipStream_t stream)
 {
-    // padded to whole staging batches of 256 threads x 2 x 16 bytes
-    const size_t lds = ((size_t)B * r * sizeof(float) + 8191) / 8192 * 8192;
+    constexpr size_t batch = (size_t)kPredUpThreads * 2 * 16;   // the staging buffer is padded to whole batches
+    const size_t lds = ((size_t)B * r * sizeof(float) + batch - 1) / batch * batch;
     constexpr int rows = RPW * (kPredUpThreads / kWave);
     ST_LAUNCH(ps, (predictor_up_mask_kernel<T, LPR, RPW>), dim3((I + rows - 1) / rows), dim3(kPredUpThreads), lds,
               stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask);
 }
 
-// One row of x: 16 rows per wave (8 when a whole wave shares a row).  Several rows of x: 4 rows per wave,
-// so that four times as many waves hide each other's latencies.
 template <typename T, int LPR>
 static void launch_up(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
                       float *scores, uint8_t *mask, hipStream_t stream)
 {
-    if (B == 1) launch_up_rpw<T, LPR, pred_rows_per_wave(LPR)>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
-    else launch_up_rpw<T, LPR, 4>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+    launch_up_rpw<T, LPR, pred_rows_per_wave(LPR)>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
 }
 
 template <typename T>
