@@ -886,7 +886,7 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
         const char *v = getenv("ST_CACHE_TPB");
         return v ? atoi(v) : 0;
     }();
-    const int grid = blocks ? blocks : device_cu_count() / 2;
+    const int grid = blocks ? blocks : device_cu_count() * 3 / 4;   // (measured against 1/4, 3/8, 1/2 and all of the CUs)
     const bool aligned = (I % 8 == 0) && ((uintptr_t)mask % 8 == 0) && ((uintptr_t)c->b.cur_mask % 8 == 0) &&
                          ((uintptr_t)c->b.indices % 16 == 0);
     // 512-thread blocks (ST_CACHE_TPB=512) leave room on the CU for a kernel of another stream, but

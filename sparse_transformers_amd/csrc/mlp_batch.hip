@@ -17,7 +17,7 @@
 //             has to be transposed: blocks own (column group, row split), each
 //             wave stages 32 rows x 64 columns in LDS and reads the fragment
 //             column-wise.  Split-K partial rows are summed in a fixed order
-//             by kernel 3.
+//             by kernel 3 (mlp_reduce_kernel).
 // Unlike a per-CU fused kernel this writes no per-CU partial [B,H] rows (which
 // would cost B * 3 MB of extra traffic); h (B * n elements) is the only
 // intermediate.
@@ -292,28 +292,6 @@ __global__ __launch_bounds__(kBtThreads) void batch_down_kernel(
     }
 }
 
-// kernel 3: out[b][c] = sum over the row splits, fixed order.
-template <typename T>
-__global__ __launch_bounds__(256) void batch_reduce_kernel(const float *__restrict__ partial, int RS, int B, int H,
-                                                           T *__restrict__ out)
-{
-    const int col = (blockIdx.x * 256 + threadIdx.x) * 4;
-    const int b = blockIdx.y;
-    if (col >= H) return;
-    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int r0 = 0; r0 < RS; r0 += 8) {
-        float4 v[8];
-#pragma unroll
-        for (int k = 0; k < 8; ++k)
-            v[k] = r0 + k < RS ? *reinterpret_cast<const float4 *>(partial + ((size_t)(r0 + k) * kBtRows + b) * H + col)
-                               : make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-        for (int k = 0; k < 8; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
-    }
-    T *o = out + (size_t)b * H + col;
-    o[0] = from_float<T>(s.x); o[1] = from_float<T>(s.y); o[2] = from_float<T>(s.z); o[3] = from_float<T>(s.w);
-}
-
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -416,12 +394,11 @@ static int launch_batch_t(const void *x_, int B, int H, const void *gate_, const
                        : launch_down<T, 2>(hbuf, ldh, bc, down, H, n, n_dev, partial, s, stream);
         if (rc != ST_OK) return rc;
         ST_HIP(hipGetLastError());
-        {
-            ProfScope ps(ST_K_MLP_REDUCE, stream);
-            ST_LAUNCH(ps, batch_reduce_kernel<T>, dim3((H / 4 + 255) / 256, bc), dim3(256), 0, stream, partial,
-                               s.rs, bc, H, out);
-        }
-        ST_HIP(hipGetLastError());
+        // kernel 3: the row splits' partial rows [rs][16][H] summed in a fixed order (the streaming kernels'
+        // reduce kernel: one memory round trip, 32-column blocks)
+        rc = launch_mlp_reduce(sizeof(T) == 2 && __is_same(T, f16_t) ? ST_F16 : ST_BF16, partial, s.rs, kBtRows, bc, H,
+                               out, stream);
+        if (rc != ST_OK) return rc;
     }
     return ST_OK;
 }

@@ -185,6 +185,88 @@ __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_kernel(const
     }
 }
 
+// Several rows of x (B > 1), rank rows of at most LPR chunks: a lane keeps its chunk of t for eight rows of x
+// in registers and reuses it for the NITER rows of Bm it visits, so the LDS is read once per lane instead of
+// once per (row of Bm, row of x) -- the first form of the kernel was bound by exactly those reads (32-byte
+// strides, half the banks idle) and took 1.3 us per additional row of x at r = 256.  All NITER row loads of a
+// wave are issued before anything else.
+template <typename T, int LPR, int NITER>
+__global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_rows_kernel(const float *__restrict__ t, int B, int r,
+                                                                       const T *__restrict__ Bm, int I, float thr,
+                                                                       int cmp_ge, float *__restrict__ scores,
+                                                                       uint8_t *__restrict__ mask)
+{
+    constexpr int VEC = Elem<T>::kVec;
+    constexpr int RPI = kWave / LPR;   // rows per iteration
+    extern __shared__ __align__(16) unsigned char smem[];
+    float *ts = reinterpret_cast<float *>(smem);  // [B][r]
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int chunks = r / VEC;
+    const int cl = lane & (LPR - 1), gidx = lane / LPR;
+    const int tile = (blockIdx.x * (kPredUpThreads / kWave) + wave) * (RPI * NITER);
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+    const bool has_chunk = cl < chunks;
+
+    uint4 w[NITER];
+#pragma unroll
+    for (int it = 0; it < NITER; ++it) {
+        const int row = tile + it * RPI + gidx;
+        w[it] = ld16(Bm + (size_t)(row < I ? row : I - 1) * r + (size_t)(has_chunk ? cl : 0) * VEC);
+        if (!has_chunk) w[it] = zero4;
+    }
+    {   // stage t: 16-byte pieces, two per thread requested together (the buffer is padded to whole batches)
+        const float4 *t4 = reinterpret_cast<const float4 *>(t);
+        float4 *ts4 = reinterpret_cast<float4 *>(ts);
+        const int n4 = (B * r) >> 2;
+        for (int i0 = 0; i0 < n4; i0 += kPredUpThreads * 2) {
+            float4 v[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int i = i0 + u * kPredUpThreads + tid;
+                v[u] = t4[i < n4 ? i : n4 - 1];
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) ts4[i0 + u * kPredUpThreads + tid] = v[u];
+        }
+        __syncthreads();
+    }
+    unsigned any = 0u;   // bit per iteration
+    for (int b0 = 0; b0 < B; b0 += kPredUpBTile) {
+        float tr[kPredUpBTile][VEC];
+#pragma unroll
+        for (int b = 0; b < kPredUpBTile; ++b) {
+            const float *tp = ts + (size_t)(b0 + b < B ? b0 + b : B - 1) * r + (has_chunk ? cl : 0) * VEC;
+#pragma unroll
+            for (int e = 0; e < VEC; e += 4) {
+                const float4 q = *reinterpret_cast<const float4 *>(tp + e);
+                tr[b][e] = q.x; tr[b][e + 1] = q.y; tr[b][e + 2] = q.z; tr[b][e + 3] = q.w;
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < NITER; ++it) {
+            const int row = tile + it * RPI + gidx;
+            float fw[VEC];
+            unpack<T>(w[it], fw);   // zeros in lanes without a chunk
+#pragma unroll
+            for (int b = 0; b < kPredUpBTile; ++b) {
+                if (b0 + b < B) {   // uniform
+                    float acc = 0.f;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc = fmaf(fw[e], tr[b][e], acc);
+                    const float v = group_sum_dpp<LPR>(acc);
+                    if (cmp_ge ? (v >= thr) : (v > thr)) any |= 1u << it;
+                    if (scores && cl == 0 && row < I) scores[(size_t)(b0 + b) * I + row] = v;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < NITER; ++it) {
+        const int row = tile + it * RPI + gidx;
+        if (cl == 0 && row < I) mask[row] = (any >> it) & 1u;
+    }
+}
+
 template <typename T, int LPR, int RPW>
 static void launch_up_rpw(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
                           float *scores, uint8_t *mask, hipStream_t stream)
@@ -200,6 +282,15 @@ template <typename T, int LPR>
 static void launch_up(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
                       float *scores, uint8_t *mask, hipStream_t stream)
 {
+    constexpr int NITER = LPR >= 16 ? LPR / 16 : 1;   // about four rows of Bm per wave (measured against 1, 2 and 8 per lane)
+    if (B > 1 && r / Elem<T>::kVec <= LPR) {
+        constexpr size_t batch = (size_t)kPredUpThreads * 2 * 16;
+        const size_t lds = ((size_t)B * r * sizeof(float) + batch - 1) / batch * batch;
+        constexpr int rows = (kWave / LPR) * NITER * (kPredUpThreads / kWave);
+        ST_LAUNCH(ps, (predictor_up_mask_rows_kernel<T, LPR, NITER>), dim3((I + rows - 1) / rows), dim3(kPredUpThreads),
+                  lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask);
+        return;
+    }
     launch_up_rpw<T, LPR, pred_rows_per_wave(LPR)>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
 }
 
