@@ -81,9 +81,10 @@ __global__ __launch_bounds__(kPredDownThreads) void predictor_down_kernel(const 
 }
 
 constexpr int kPredUpThreads = 256;   // (128-thread blocks measure the same)
-// rows of Bm a wave owns per pass: four for every row length.  (More rows per wave mean fewer blocks; with 16
-// the 8192-row matrix made 128 blocks and a decode layer measured 1 us slower than with the 512 blocks of 4.)
-constexpr int pred_rows_per_wave(int) { return 4; }
+// Rows of Bm a wave owns: as few as keep every lane busy for one pass (four rows of 16 chunks, two of 32 or
+// 64).  More rows per wave mean fewer blocks, and the layer measures slower: 16 rows per wave (128 blocks at
+// I = 8192) cost 1 us per layer against 4, and 4 against 2 cost 1.2 us at r = 256 and 0.7 us at r = 440.
+constexpr int pred_rows_per_wave(int lpr) { return lpr >= 32 ? 2 : 4; }
 constexpr int kPredUpBTile = 8;
 
 // LPR lanes share one row of Bm (LPR >= r/VEC unless the row needs several
