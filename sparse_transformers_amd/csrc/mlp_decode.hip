@@ -364,6 +364,16 @@ template <typename T, int NB> static int launch_one(const MlpLaunch &a, int b0, 
         if (chunks > 1024) return launch_inst<T, 1, 3, 2, 1024, false>(a, b0, bcount);
         // (512-thread blocks, 3 / 4 / 12 rows in flight and double-buffered row batches were all measured
         // slower for one row of x)
+        // (the rows in flight do not change which rows a group sums or in which order: when the expected count
+        // gives a group seven rows, one batch of seven beats a batch of six followed by a batch of one; likewise
+        // wherever sevens need fewer batches than sixes)
+        if constexpr (Elem<T>::kBytes == 2) {
+            int gs_log2 = 6;
+            while ((1 << gs_log2) < chunks && (1 << gs_log2) < 1024) ++gs_log2;
+            const int ngrp = 1024 >> gs_log2, expect = a.n_dev ? (a.n_hint < a.n ? a.n_hint : a.n) : a.n;
+            const int rpg = ((expect + a.G - 1) / a.G + ngrp - 1) / ngrp;
+            if ((rpg + 6) / 7 < (rpg + 5) / 6) return launch_inst<T, 1, 7, 1, 1024, false>(a, b0, bcount);   // 7, 13, 14, ...
+        }
         return launch_inst<T, 1, DecodeRows<T>::value, 1, 1024, false>(a, b0, bcount);
     } else if constexpr (NB == 2) {
         return launch_inst<T, 2, 2, 1, 1024, true>(a, b0, bcount);

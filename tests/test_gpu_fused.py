@@ -134,7 +134,9 @@ def test_fused_call_with_several_rows_takes_the_two_kernel_path():
 
 
 @pytest.mark.parametrize("dtype,H,I,n0", [("float16", 3072, 8192, 2867), ("bfloat16", 4096, 4096, 400),
-                                          ("float32", 2048, 4096, 1500)])
+                                          ("float32", 2048, 4096, 1500),
+                                          # seven rows per thread group: the variants with seven rows in flight
+                                          ("bfloat16", 4096, 14336, 3584), ("float16", 3072, 8192, 3500)])
 def test_fused_result_does_not_depend_on_the_hint(dtype, H, I, n0):
     """The caller's guess of the active count decides which kernel variant runs, what is requested before
     the plan is known and how much of the index list is fetched up front; a wrong guess (far too low: the
