@@ -64,7 +64,8 @@ const char *st_last_error(void);
  *                      the buffers must really hold n rows)
  *   n_hint             only with n_dev: the count the host expects (0 = no
  *                      idea).  Rows below it are requested before *n_dev has
- *                      arrived; a wrong hint costs time, never correctness
+ *                      arrived and it picks how many rows stay in flight; a
+ *                      wrong hint costs time, never correctness
  *   out        [B,H]   dtype `dtype`   (the reference's down_proj_buffer)
  *   combined   [B,ldc] dtype `dtype`, optional (NULL = skip): receives
  *                      act(gate)*up in columns [0,n) and, when gated, the raw
@@ -205,8 +206,9 @@ int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream);
  * ends in the same state and `out` holds the same bits as the two separate
  * calls.  x, out: [B,H] in the cache's dtype; combined: [B,ldc] or NULL;
  * workspace: st_mlp_workspace_bytes(B, H, I) bytes.  n_hint: the active count
- * the host last saw (0 = unknown); it only decides which rows are requested
- * before the plan is known and never affects results.  An update that empties
+ * the host last saw (0 = unknown); it picks the kernel variant, which rows are
+ * requested before the plan is known and how much of the index list is
+ * fetched up front, and never affects results.  An update that empties
  * the cache leaves status ST_ERR_NO_ACTIVE in the state words (reported by
  * st_cache_sync_state) and zeros in `out`. */
 int st_cache_update_forward(st_cache *c, const uint8_t *mask, const void *x, int64_t B, int64_t n_hint, void *out,
