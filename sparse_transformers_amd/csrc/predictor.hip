@@ -305,8 +305,11 @@ static int launch_predictor(const void *x, int B, int H, const void *A, int r, c
         if (B == 1)
             ST_LAUNCH(ps, (predictor_down_kernel<T, 1>), dim3(r), dim3(kPredDownThreads), 0, stream,
                       static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
-        else
+        else if (B <= kPredBTile)
             ST_LAUNCH(ps, (predictor_down_kernel<T, kPredBTile>), dim3(r), dim3(kPredDownThreads), 0, stream,
+                      static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
+        else   // 9 to 16 rows of x in one pass (one memory round trip instead of two)
+            ST_LAUNCH(ps, (predictor_down_kernel<T, 2 * kPredBTile>), dim3(r), dim3(kPredDownThreads), 0, stream,
                       static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
     }
     ST_HIP(hipGetLastError());
