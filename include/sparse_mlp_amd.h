@@ -73,8 +73,8 @@ const char *st_last_error(void);
  *                      leaves in combined_proj_buffer
  *   workspace          scratch of st_mlp_workspace_bytes(B,H,n) bytes
  * All rows must be 16-byte aligned (H*sizeof(dtype) % 16 == 0). B <= 4096.
- * B == 1 (and any B < 32 in fp32 or with a hidden size the MFMA kernels do not
- * cover) runs the streaming decode kernel; 2 <= B < 32 in fp16 / bf16 with H in
+ * B <= 2 (and any B < 32 in fp32 or with a hidden size the MFMA kernels do not
+ * cover) runs the streaming decode kernel; 3 <= B < 32 in fp16 / bf16 with H in
  * {2048, 3072, 4096} runs the MFMA batch kernels (still HBM-bound, one pass over
  * the weights per 16 rows); B >= 32 in fp16 / bf16 with H % 128 == 0 runs the
  * MFMA GEMM kernels (then only columns [0,n) of `combined` are written).
@@ -198,7 +198,7 @@ int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream);
 /* update_active_weights(mask) immediately followed by the sparse MLP on the
  * updated cache -- weight_cache.h:229-359 then sparse_mlp_op.cpp:53-192 /
  * src/modeling_skip.py:114-117, i.e. what SkipDecoderLayer.forward does per
- * layer (src/modeling_skip.py:234-261) -- enqueued as one call.  For B == 1
+ * layer (src/modeling_skip.py:234-261) -- enqueued as one call.  For B <= 2
  * (16-byte aligned rows, 8-byte aligned mask, I % 8 == 0) this is ONE kernel
  * that replays the bookkeeping and streams the active rows, taking rows whose
  * index changed from the pool and writing them back on the way; otherwise it

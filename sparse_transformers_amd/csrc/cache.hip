@@ -561,16 +561,17 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
 // update followed by forward.
 // Rows are dealt to blocks round-robin: row(bat, k) = blk + G * (grp + ngrp * (bat * RB + k)).
 // ---------------------------------------------------------------------------
-template <typename T, int RB, int PLANW, int TPB, bool AHEAD = false>
+template <typename T, int RB, int PLANW, int TPB, bool AHEAD = false, int NB = 1>
 __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     FusedRows fr, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
-    int32_t *__restrict__ state, int I, const T *__restrict__ x, int H, T *__restrict__ combined, long ldc,
+    int32_t *__restrict__ state, int I, const T *__restrict__ x, int B, int H, T *__restrict__ combined, long ldc,
     float *__restrict__ partials, int act, int gs_log2, int plan_bytes, int n_hint, int idx_cap)
 {
+    // NB rows of x per pass (B <= NB; rows past B are zeros): [G][NB][H] partial rows
     constexpr int VEC = Elem<T>::kVec;
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ float red[TPB / kWave][RB][2];  // per-wave partial (g,u)
-    __shared__ float hs[TPB / kWave][RB];      // h of the rows being computed
+    __shared__ float red[TPB / kWave][RB][NB][2];  // per-wave partial (g,u)
+    __shared__ float hs[TPB / kWave][RB][NB];      // h of the rows being computed
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int G = gridDim.x, blk = blockIdx.x;
@@ -588,7 +589,12 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
 
     // x is requested behind the loads the plan hangs on (planning waves) or while waiting for them (the
     // others), and looked at only in phase 1
-    uint4 xr = zero4;
+    uint4 xr[NB];
+    auto load_x = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            xr[b] = ld16(reinterpret_cast<const unsigned char *>(x) + (size_t)(b < B ? b : 0) * row_bytes + coff);
+    };
 
     auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
 
@@ -623,7 +629,7 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
         }
     };
     if (streams_ahead) {
-        xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff);
+        load_x();
         lds_barrier();   // (A) the plan's own loads have arrived (inside cache_plan, after the LDS fill)
         speculate();
         lds_barrier();   // (B) the plan is finished
@@ -634,7 +640,7 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
         // memory requests
         cache_plan<true, PT, true, SPLIT>(pv, smem, &plan_shared, new_mask, cur_mask2, indices2, state, I,
                                           idx_cap, SPLIT ? tid - (TPB - PT) : tid,
-                                          [&] { xr = ld16(reinterpret_cast<const unsigned char *>(x) + coff); },
+                                          [&] { load_x(); },
                                           [&] { if constexpr (AHEAD) speculate(); });
         if (SPLIT) {
             plan_publish(pv, &plan_shared);
@@ -643,9 +649,11 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     }
     const int n = pv.n_new, n_old = pv.n_old;
 
-    float acc[VEC];
+    float acc[NB][VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[b][e] = 0.f;
 
     const int jcount = n > blk ? (n - blk + G - 1) / G : 0;      // rows of this block
     const int nbat = ((jcount + ngrp - 1) / ngrp + RB - 1) / RB;  // uniform over the block
@@ -681,15 +689,20 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
         ST_TL(6);
 
         // ---- phase 1: partial dot products on this thread's chunk
-        const uint4 xq = valid ? xr : zero4;
+        uint4 xq[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) xq[b] = (valid && b < B) ? xr[b] : zero4;
 #pragma unroll
         for (int k = 0; k < RB; ++k) {
-            float pg = 0.f, pu = 0.f;
-            dot_chunk<T>(wg[k], wu[k], xq, pg, pu);
-            const float sg = wave_sum_dpp(pg), su = wave_sum_dpp(pu);
-            if (lane == 0) {
-                red[wave][k][0] = sg;
-                red[wave][k][1] = su;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                float pg = 0.f, pu = 0.f;
+                dot_chunk<T>(wg[k], wu[k], xq[b], pg, pu);
+                const float sg = wave_sum_dpp(pg), su = wave_sum_dpp(pu);
+                if (lane == 0) {
+                    red[wave][k][b][0] = sg;
+                    red[wave][k][b][1] = su;
+                }
             }
         }
         // write the fresh rows back while the reductions settle
@@ -703,20 +716,21 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
             }
         }
         __syncthreads();
-        if (tid < ngrp * RB) {
-            const int g_ = tid / RB, k_ = tid - g_ * RB;
+        if (tid < ngrp * RB * NB) {
+            const int g_ = tid / (RB * NB), rem = tid - g_ * (RB * NB);
+            const int k_ = rem / NB, b_ = rem - k_ * NB;
             const int row = blk + G * (g_ + ngrp * (bat * RB + k_));
             float sg = 0.f, su = 0.f;
             for (int wv = g_ * wpg; wv < (g_ + 1) * wpg; ++wv) {
-                sg += red[wv][k_][0];
-                su += red[wv][k_][1];
+                sg += red[wv][k_][b_][0];
+                su += red[wv][k_][b_][1];
             }
             const float hv = has_gate ? activate(sg, act) * su : activate(su, act);
             const bool ok = row < n;
-            hs[g_][k_] = ok ? hv : 0.f;
-            if (ok && combined) {
-                combined[row] = from_float<T>(hv);
-                if (has_gate) combined[n + row] = from_float<T>(su);
+            hs[g_][k_][b_] = ok ? hv : 0.f;
+            if (ok && combined && b_ < B) {
+                combined[(size_t)b_ * ldc + row] = from_float<T>(hv);
+                if (has_gate) combined[(size_t)b_ * ldc + n + row] = from_float<T>(su);
             }
         }
         __syncthreads();
@@ -724,34 +738,43 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
 #pragma unroll
         for (int k = 0; k < RB; ++k) {
             const bool row_ok = row_of(bat, k) < n;
-            axpy_chunk<T>(hs[grp][k], row_ok ? wd[k] : zero4, acc);
+            const uint4 rd = row_ok ? wd[k] : zero4;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) axpy_chunk<T>(hs[grp][k][b], rd, acc[b]);
         }
     }
 
     // ---- combine the thread groups through LDS (behind the plan arrays), one fp32 partial row per block
     if (ngrp > 1) {
-        float *redc = reinterpret_cast<float *>(smem + plan_bytes);  // [ngrp-1][H]
+        float *redc = reinterpret_cast<float *>(smem + plan_bytes);  // [ngrp-1][NB][H]
         if (grp > 0 && valid) {
 #pragma unroll
-            for (int e = 0; e < VEC; e += 4)
-                *reinterpret_cast<float4 *>(redc + (size_t)(grp - 1) * H + (size_t)cc * VEC + e) =
-                    make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int e = 0; e < VEC; e += 4)
+                    *reinterpret_cast<float4 *>(redc + ((size_t)(grp - 1) * NB + b) * H + (size_t)cc * VEC + e) =
+                        make_float4(acc[b][e], acc[b][e + 1], acc[b][e + 2], acc[b][e + 3]);
         }
         __syncthreads();
         if (grp == 0 && valid) {
             for (int gq = 1; gq < ngrp; ++gq)
 #pragma unroll
-                for (int e = 0; e < VEC; e += 4) {
-                    const float4 v = *reinterpret_cast<const float4 *>(redc + (size_t)(gq - 1) * H + (size_t)cc * VEC + e);
-                    acc[e] += v.x; acc[e + 1] += v.y; acc[e + 2] += v.z; acc[e + 3] += v.w;
-                }
+                for (int b = 0; b < NB; ++b)
+#pragma unroll
+                    for (int e = 0; e < VEC; e += 4) {
+                        const float4 v = *reinterpret_cast<const float4 *>(redc + ((size_t)(gq - 1) * NB + b) * H +
+                                                                            (size_t)cc * VEC + e);
+                        acc[b][e] += v.x; acc[b][e + 1] += v.y; acc[b][e + 2] += v.z; acc[b][e + 3] += v.w;
+                    }
         }
     }
     if (grp == 0 && valid) {
 #pragma unroll
-        for (int e = 0; e < VEC; e += 4)
-            *reinterpret_cast<float4 *>(partials + (size_t)blk * H + (size_t)cc * VEC + e) =
-                make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int e = 0; e < VEC; e += 4)
+                *reinterpret_cast<float4 *>(partials + ((size_t)blk * NB + b) * H + (size_t)cc * VEC + e) =
+                    make_float4(acc[b][e], acc[b][e + 1], acc[b][e + 2], acc[b][e + 3]);
     }
     plan_finish(pv, state);
     ST_TL(7);
@@ -943,11 +966,12 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
     while ((1 << gs_log2) < chunks && (1 << gs_log2) < TPB) ++gs_log2;
     const int ngrp = TPB >> gs_log2;
     const size_t plan_bytes = (plan_lds_bytes(I) + 15) & ~(size_t)15;
-    const size_t lds = plan_bytes + (size_t)(ngrp - 1) * H * 4;
+    const int NBF = B == 2 ? 2 : 1;   // rows of x the fused kernel takes in one pass
+    const size_t lds = plan_bytes + (size_t)(ngrp - 1) * NBF * H * 4;
     const bool aligned = (I % 8 == 0) && ((uintptr_t)mask % 8 == 0) && ((uintptr_t)c->b.cur_mask % 8 == 0) &&
                          ((uintptr_t)c->b.indices % 16 == 0);
     static const bool fused_off = [] { const char *v = getenv("ST_CACHE_FUSED"); return v && atoi(v) == 0; }();
-    const bool fused = !fused_off && B == 1 && aligned && I <= 8 * TPB * kPlanMaxWords && chunks <= TPB &&
+    const bool fused = !fused_off && B <= 2 && aligned && I <= 8 * TPB * kPlanMaxWords && chunks <= TPB &&
                        row_bytes % 16 == 0 && lds <= (size_t)(156 * 1024);
     if (!fused) {   // two launches: update, then the forward that reads the count on the device
         const int rc = st_cache_update_async(c, mask, stream);
@@ -982,7 +1006,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
                 attr_set = true;
             }
             ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, fr, mask, c->b.cur_mask, c->b.indices, c->b.state, I,
-                               xt, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint, idx_cap);
+                               xt, (int)B, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint, idx_cap);
             return ST_OK;
         };
         int rc;
@@ -1007,7 +1031,18 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
 #define ST_FUSED_LAUNCH(TYPE, PLANW, AHEAD)                                                            \
     rc = launch(cache_update_decode_kernel<TYPE, (AHEAD) ? 3 : DecodeRows<TYPE>::value, PLANW, TPB, AHEAD>, \
                 static_cast<const TYPE *>(x), static_cast<TYPE *>(combined))
-        if (c->dtype == ST_F32 && split) ST_FUSED_LAUNCH(float, 8, false);
+        // two rows of x: all waves plan (the second row of x costs the registers the split form would need); six
+        // rows per group in flight when that is one batch, else five (measured faster than six at seven rows)
+        if (B == 2) {
+#define ST_FUSED_LAUNCH2(TYPE, ROWS)                                                                             \
+    rc = launch(cache_update_decode_kernel<TYPE, ROWS, 0, TPB, false, 2>, static_cast<const TYPE *>(x),          \
+                static_cast<TYPE *>(combined))
+            const bool one_batch = ((hint + G - 1) / G + ngrp - 1) / ngrp <= 6;
+            if (c->dtype == ST_F32) { if (one_batch) ST_FUSED_LAUNCH2(float, 6); else ST_FUSED_LAUNCH2(float, 5); }
+            else if (c->dtype == ST_BF16) { if (one_batch) ST_FUSED_LAUNCH2(bf16_t, 6); else ST_FUSED_LAUNCH2(bf16_t, 5); }
+            else { if (one_batch) ST_FUSED_LAUNCH2(f16_t, 6); else ST_FUSED_LAUNCH2(f16_t, 5); }
+#undef ST_FUSED_LAUNCH2
+        } else if (c->dtype == ST_F32 && split) ST_FUSED_LAUNCH(float, 8, false);
         else if (c->dtype == ST_F32 && ahead) ST_FUSED_LAUNCH(float, 0, true);
         else if (c->dtype == ST_F32) ST_FUSED_LAUNCH(float, 0, false);
         else if (c->dtype == ST_BF16 && rows7)
@@ -1026,7 +1061,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
         if (rc != ST_OK) return rc;
     }
     ST_HIP(hipGetLastError());
-    return launch_mlp_reduce(c->dtype, partials, G, 1, 1, H, out, s);
+    return launch_mlp_reduce(c->dtype, partials, G, NBF, (int)B, H, out, s);
 }
 
 extern "C" int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream)

@@ -1,4 +1,4 @@
-// Sparse MLP over the active set for a small batch of rows of x (2 <= B < 32):
+// Sparse MLP over the active set for a small batch of rows of x (3 <= B < 32):
 // still bound by the HBM stream of the active rows, but with B rows of x the
 // multiply-adds no longer fit beside it on the vector ALUs, so they go to the
 // matrix cores (fp16 / bf16 MFMA 16x16x32, fp32 accumulate).  Up to 16 rows of

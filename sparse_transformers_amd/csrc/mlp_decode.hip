@@ -415,11 +415,13 @@ template <typename T> static int launch_nb(const MlpLaunch &a)
 
 constexpr int kMlpMaxBatchPerLaunch = 8;
 
-// Rows of x from which the MFMA batch kernels take over from the streaming kernel
-// (ST_MLP_BATCH_MIN overrides; 32 or more switches them off).
+// Rows of x from which the MFMA batch kernels take over from the streaming kernel: three (with two the
+// streaming kernel measures the same as they do, and it is the arithmetic of the fused update + decode kernel
+// for two rows, whose result has to equal update followed by forward).  ST_MLP_BATCH_MIN overrides; 32 or more
+// switches the batch kernels off.
 int batch_min_rows()
 {
-    static const int v = [] { const int m = env_int("ST_MLP_BATCH_MIN"); return m >= 2 ? m : 2; }();
+    static const int v = [] { const int m = env_int("ST_MLP_BATCH_MIN"); return m >= 2 ? m : 3; }();
     return v;
 }
 

@@ -247,7 +247,7 @@ int launch_prefill(int dtype, const void *x, int M, int H, const void *gate, con
                    const int *n_dev, void *out, void *comb, long ldc, void *workspace, int act, int has_gate,
                    hipStream_t stream);
 
-// MFMA kernels for a small batch of rows (2 <= B < 32, fp16 / bf16, supported hidden sizes only).
+// MFMA kernels for a small batch of rows (batch_min_rows() <= B < 32, fp16 / bf16, supported hidden sizes only).
 int batch_min_rows();
 bool batch_supported(int dtype, int H);
 int64_t batch_workspace_bytes(int64_t H, int64_t n);

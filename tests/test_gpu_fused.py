@@ -158,3 +158,35 @@ def test_fused_result_does_not_depend_on_the_hint(dtype, H, I, n0):
         torch.cuda.synchronize()
         assert torch.equal(yf, yp), (step, hint)
         _same_state(fused, plain, step)
+
+
+@pytest.mark.parametrize("dtype,H,I", [("float16", 3072, 4096), ("bfloat16", 4096, 4096), ("float32", 2048, 4096),
+                                       ("float16", 1024, 4096)])
+@pytest.mark.parametrize("has_gate", [True, False])
+def test_fused_two_rows_of_x(dtype, H, I, has_gate):
+    """Two rows of x go through the fused kernel too (one pass over the rows for both): result, the
+    combined buffer and the cache state equal update followed by forward, bit for bit, over a ragged trace;
+    and each row equals what the same row gives on its own."""
+    trace = syn.ragged_mask_trace(23 + H, I, 24)
+    fused, plain, _, g = _pair(I, H, dtype, has_gate, 7, torch.from_numpy(trace[0]))
+    single, _, _, _ = _pair(I, H, dtype, has_gate, 7, torch.from_numpy(trace[0]))
+    tdt = getattr(torch, dtype)
+    for t in range(1, len(trace)):
+        if not trace[t].any():
+            continue
+        m = torch.from_numpy(trace[t]).to(DEV)
+        x = torch.randn(2, H, generator=g).to(tdt).to(DEV)
+        comb_f = torch.zeros(2, 2 * I, dtype=tdt, device=DEV)
+        comb_p = torch.zeros_like(comb_f)
+        yf = fused.update_and_forward(m, x, "silu", combined=comb_f)
+        plain.update_active_weights_async(m)
+        yp = plain.forward(x, "silu", combined=comb_p)
+        single.update_active_weights_async(m)
+        y0, y1 = single.forward(x[0:1], "silu").clone(), single.forward(x[1:2], "silu").clone()
+        torch.cuda.synchronize()
+        assert torch.equal(yf, yp), (t, (yf.float() - yp.float()).abs().max().item())
+        assert torch.equal(comb_f, comb_p), t
+        assert torch.equal(yf[0:1], y0) and torch.equal(yf[1:2], y1), t
+        if t % 6 == 0:
+            _same_state(fused, plain, t)
+    _same_state(fused, plain, "end")
