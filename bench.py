@@ -52,6 +52,9 @@ def parse_args():
     ap.add_argument("--profile-steps", type=int, default=32)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a known-size reference for rocprofv3 --pmc)")
+    ap.add_argument("--active-frac", type=float, default=0.0,
+                    help="override the active fraction (e.g. the union of several rows' masks)")
+    ap.add_argument("--churn", type=float, default=-1.0, help="override the fraction of the active set swapped per step")
     ap.add_argument("--seed", type=int, default=1236)
     return ap.parse_args()
 
@@ -157,6 +160,11 @@ def main():
     from sparse_transformers_amd import _lib, synthetic as syn
 
     wl = syn.WORKLOADS[args.workload]
+    if args.active_frac > 0.0 or args.churn >= 0.0:
+        import dataclasses
+        wl = dataclasses.replace(wl, active_frac=args.active_frac if args.active_frac > 0.0 else wl.active_frac,
+                                 churn_lo=args.churn if args.churn >= 0.0 else wl.churn_lo,
+                                 churn_hi=args.churn if args.churn >= 0.0 else wl.churn_hi)
     layers = args.layers or wl.layers
     B = args.batch or wl.batch
     dev = torch.device("cuda:0")

@@ -38,6 +38,10 @@ WORKLOADS = {
     "llama1b_layer_fp32": Workload("llama1b_layer_fp32", 1, 2048, 8192, 64, "float32", "silu", True, 0.30, 0.10, 0.10, 128),
     # Llama-3.2-3B-shaped stack, fp16, 35 % active, 5-15 % churn  (the headline workload)
     "llama3b_stack_fp16": Workload("llama3b_stack_fp16", 28, 3072, 8192, 128, "float16", "silu", True, 0.35, 0.05, 0.15, 512),
+    # Llama-3.2-3B-shaped layer in bf16 with per-token masks of 30 % that overlap by 0.6 from one token to the next
+    # (40 % of the active set swapped per step), stacked 28 deep so that the weights cannot sit in the Infinity Cache
+    "llama3b_stack_bf16_overlap06": Workload("llama3b_stack_bf16_overlap06", 28, 3072, 8192, 128, "bfloat16", "silu", True,
+                                             0.30, 0.40, 0.40, 64),
     # Mistral-7B-shaped stack, bf16, 25 % active, 10 % churn
     "mistral7b_stack_bf16": Workload("mistral7b_stack_bf16", 32, 4096, 14336, 256, "bfloat16", "silu", True, 0.25, 0.10, 0.10, 256),
     # ReLU-Llama-7B-shaped stack, fp16, 10 % active, 20 % churn, gated and ungated
