@@ -141,6 +141,20 @@ class SparseDecodeLayer:
         self._scores_ws: Optional[torch.Tensor] = None
         self._select_ws: Optional[torch.Tensor] = None
 
+    @classmethod
+    def from_sparsity(cls, predictor: FastLoRAProjection, cache: WeightCache, sparsity: float,
+                      sparsity_method: str = "naive", act: str = "silu") -> "SparseDecodeLayer":
+        """The layer as SkipDecoderLayer.__init__ configures it from ``config.sparsities[layer_idx]``
+        (src/modeling_skip.py:138-143): "statistical_topk" takes its multiplier from the inverse normal CDF
+        at ``sparsity``; "topk" keeps ``int(hidden_size * (1 - sparsity))`` scores per row -- the reference
+        sets ``self.intermediate_size = config.hidden_size`` (:134), so the count follows the hidden size."""
+        k, z = 0, 0.0
+        if sparsity_method == "statistical_topk":
+            z = float(torch.distributions.normal.Normal(0, 1).icdf(torch.tensor(float(sparsity))))
+        elif sparsity_method == "topk":
+            k = int(cache.hidden_size * (1 - sparsity))
+        return cls(predictor, cache, act=act, method=sparsity_method, k=k, std_multiplier=z)
+
     def predict_mask(self, x_pred: torch.Tensor, t_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
         """The layer's mask for ``x_pred`` into ``self.mask``.  The buffers the row-statistic methods need are
         created on the first call with a given batch size (so: before a graph capture, not inside one)."""

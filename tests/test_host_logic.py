@@ -87,3 +87,22 @@ def test_predictor_checkpoints_round_trip(tmp_path):
     for p, sd in zip(preds, want):
         assert p.lora_size == r and p.hidden_size == H and p.intermediate_size == I
         assert torch.equal(p.down_weight, sd["down.weight"].half()) and torch.equal(p.up_weight, sd["up.weight"].half())
+
+
+def test_layer_constants_from_sparsity():
+    """SkipDecoderLayer.__init__ (src/modeling_skip.py:134-143): the top-k count follows the *hidden* size and the
+    statistical multiplier is the standard normal quantile at the sparsity (checked against scipy's ppf)."""
+    from types import SimpleNamespace
+    from scipy.stats import norm
+
+    cache = SimpleNamespace(hidden_size=3072, intermediate_size=8192, device=torch.device("cpu"))
+    pred = SimpleNamespace()
+    layer = st.SparseDecodeLayer.from_sparsity(pred, cache, 0.65, "topk")
+    assert (layer.method, layer.k) == ("topk", int(3072 * (1 - 0.65))) and layer.k == 1075
+    layer = st.SparseDecodeLayer.from_sparsity(pred, cache, 0.9, "statistical_topk")
+    assert layer.method == "statistical_topk" and abs(layer.std_multiplier - norm.ppf(0.9)) < 1e-6
+    assert st.SparseDecodeLayer.from_sparsity(pred, cache, 0.5, "statistical_topk").std_multiplier == 0.0
+    layer = st.SparseDecodeLayer.from_sparsity(pred, cache, 0.7)
+    assert (layer.method, layer.k, layer.std_multiplier) == ("naive", 0, 0.0)
+    with pytest.raises(ValueError):
+        st.SparseDecodeLayer.from_sparsity(pred, cache, 0.7, "magnitude")
