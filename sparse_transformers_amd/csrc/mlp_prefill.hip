@@ -10,9 +10,10 @@
 //             down columns, i.e. K runs down the rows: pairs of rows are
 //             interleaved in registers so that LDS holds Wd^T tiles
 //             ([column][k]) and the fragment reads stay 16-byte
-// Block tile 128 x 128 (kernel 1: 128 rows of x by 64 active rows of gate and
-// of up), 4 waves of 64 x 64, K stage 128 (four MFMA steps), one LDS stage with
-// the next stage's global loads held in registers during the MFMAs.
+// Kernel 1: 128 or 256 rows of x by 64 active rows of gate and of up per block, waves of 64 x 64, K
+// stages of 64 through two LDS buffers with the following stages' global loads held in registers.
+// Kernel 2: block tile 128 x 128, 4 waves of 64 x 64, K stage 128 (four MFMA steps), one LDS stage
+// with the next stage's global loads held in registers during the MFMAs.
 //
 // The reference only runs the sparse path for decode (src/modeling_skip.py:236);
 // this is the same contraction as sparse_mlp_forward_cpu
@@ -42,41 +43,46 @@ __device__ __forceinline__ int xcd_tile_id(int bid, int ntiles)
     return (bid / kXcds < per && t < ntiles) ? t : -1;
 }
 
-// Each stage moves 256 contiguous bytes of every row from HBM/L2 into LDS (a short K step would pay a
-// full memory latency for 64 bytes per row); the next stage's loads are in flight during the MFMAs.
-
 // ---------------------------------------------------------------------------
 // kernel 1: gate / up projections + activation
 // ---------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(kPfThreads) void prefill_gateup_kernel(const T *__restrict__ X, int M, int H,
-                                                                    const T *__restrict__ gate,
-                                                                    const T *__restrict__ up, int n_host,
-                                                                    const int *__restrict__ n_dev,
-                                                                    T *__restrict__ Hh, long ldh,
-                                                                    T *__restrict__ comb, long ldc, int act,
-                                                                    int has_gate, int jt, int mt)
+// K stages of 64 (one 128-byte line of every row), two LDS buffers and NS register sets: stage s is
+// requested from memory NS stages ahead, goes from registers into the LDS buffer of its parity while the
+// MFMAs of stage s - 1 run, and costs one barrier.  BM rows of x by 64 gate + 64 up rows per block,
+// 2 BM threads, every wave a 64 x (32 + 32) tile.  HG: gated.
+constexpr int kPfBK1 = 64;
+constexpr int kPfCh1 = kPfBK1 / 8;   // 16-byte chunks per row and stage
+constexpr int kPfLd1 = kPfCh1 + 1;   // LDS row stride in 16-byte units
+
+template <typename T, bool HG, int BM, int NS>
+__global__ __launch_bounds__(2 * BM) void prefill_gateup_kernel(const T *__restrict__ X, int M, int H,
+                                                                const T *__restrict__ gate,
+                                                                const T *__restrict__ up, int n_host,
+                                                                const int *__restrict__ n_dev,
+                                                                T *__restrict__ Hh, long ldh,
+                                                                T *__restrict__ comb, long ldc, int act, int jt,
+                                                                int mt)
 {
-    __shared__ uint4 sX[kPfBM][kPfLd];
-    __shared__ uint4 sG[64][kPfLd];
-    __shared__ uint4 sU[64][kPfLd];
+    constexpr int kThreads = 2 * BM;
+    __shared__ uint4 sX[2][BM][kPfLd1];
+    __shared__ uint4 sG[2][HG ? 64 : 1][kPfLd1];
+    __shared__ uint4 sU[2][64][kPfLd1];
 
     const int n = device_count(n_host, n_dev);
     const int n_pad = (n + kPfBK - 1) / kPfBK * kPfBK;  // kernel 2 runs whole K stages over Hh
     const int tile = xcd_tile_id(blockIdx.x, jt * mt);   // row tiles of x fastest: they share the weight rows
     if (tile < 0) return;
-    const int j0 = (tile / mt) * 64, m0 = (tile % mt) * kPfBM;
+    const int j0 = (tile / mt) * 64, m0 = (tile % mt) * BM;
     if (j0 >= n_pad) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l16 = lane & 15, q = lane >> 4;
-    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
 
-    // global -> register staging: thread owns chunk `ch` of rows r0 + 16 i
-    const int ch = tid & (kPfCh - 1), r0 = tid / kPfCh;
-    constexpr int kRowStep = kPfThreads / kPfCh;   // 16
-    constexpr int kXL = kPfBM / kRowStep;          // 8 loads for x
-    constexpr int kWL = 64 / kRowStep;             // 4 loads for gate, 4 for up
+    // global -> register staging: thread owns chunk `ch` of rows r0 + kRowStep i
+    const int ch = tid & (kPfCh1 - 1), r0 = tid / kPfCh1;
+    constexpr int kRowStep = kThreads / kPfCh1;
+    constexpr int kXL = BM / kRowStep;             // loads for x
+    constexpr int kWL = 64 / kRowStep;             // loads for gate and for up
 
     f32x4_t ag[4][2], au[4][2];
 #pragma unroll
@@ -100,51 +106,66 @@ __global__ __launch_bounds__(kPfThreads) void prefill_gateup_kernel(const T *__r
         const int r = j0 + r0 + kRowStep * i;
         woff[i] = (r < n ? r : (n > 0 ? n - 1 : 0)) * H + ch * 8;
     }
-    uint4 rx[kXL], rg[kWL], ru[kWL];
-    auto gload = [&](int k0) __attribute__((always_inline)) {
+    struct Stage { uint4 x[kXL], g[kWL], u[kWL]; };
+    Stage R[NS];
+    const int nk = H / kPfBK1;   // even: H is a multiple of 128
+    const int klast = (nk - 1) * kPfBK1;
+    auto gload = [&](Stage &st, int stage) __attribute__((always_inline)) {
+        const int k0 = stage * kPfBK1 <= klast ? stage * kPfBK1 : klast;   // past the end: a harmless repeat
 #pragma unroll
-        for (int i = 0; i < kXL; ++i) rx[i] = ld16(X + xoff[i] + k0);
-#pragma unroll
-        for (int i = 0; i < kWL; ++i) {
-            ru[i] = ld16(up + woff[i] + k0);
-            rg[i] = has_gate ? ld16(gate + woff[i] + k0) : zero4;
-        }
-    };
-    auto sstore = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < kXL; ++i) sX[r0 + kRowStep * i][ch] = rx[i];
+        for (int i = 0; i < kXL; ++i) st.x[i] = ld16(X + xoff[i] + k0);
 #pragma unroll
         for (int i = 0; i < kWL; ++i) {
-            sG[r0 + kRowStep * i][ch] = rg[i];
-            sU[r0 + kRowStep * i][ch] = ru[i];
+            st.u[i] = ld16(up + woff[i] + k0);
+            if (HG) st.g[i] = ld16(gate + woff[i] + k0);
         }
     };
-
-    const int nk = (H + kPfBK - 1) / kPfBK;
-    gload(0);
-    for (int ks = 0; ks < nk; ++ks) {
-        sstore();
-        __syncthreads();
-        if (ks + 1 < nk) gload((ks + 1) * kPfBK);
+    auto sstore = [&](const Stage &st, int b) __attribute__((always_inline)) {
 #pragma unroll
-        for (int kb = 0; kb < kPfKB; ++kb) {
+        for (int i = 0; i < kXL; ++i) sX[b][r0 + kRowStep * i][ch] = st.x[i];
+#pragma unroll
+        for (int i = 0; i < kWL; ++i) {
+            if (HG) sG[b][r0 + kRowStep * i][ch] = st.g[i];
+            sU[b][r0 + kRowStep * i][ch] = st.u[i];
+        }
+    };
+    auto mfmas = [&](int b) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < kPfBK1 / 32; ++kb) {
             uint4 fa[4], fg[2], fu[2];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fa[i] = sX[64 * wm + 16 * i + l16][4 * kb + q];
+            for (int i = 0; i < 4; ++i) fa[i] = sX[b][64 * wm + 16 * i + l16][4 * kb + q];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                fg[j] = sG[32 * wn + 16 * j + l16][4 * kb + q];
-                fu[j] = sU[32 * wn + 16 * j + l16][4 * kb + q];
+                if (HG) fg[j] = sG[b][32 * wn + 16 * j + l16][4 * kb + q];
+                fu[j] = sU[b][32 * wn + 16 * j + l16][4 * kb + q];
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     au[i][j] = Mfma<T>::run(fa[i], fu[j], au[i][j]);
-                    if (has_gate) ag[i][j] = Mfma<T>::run(fa[i], fg[j], ag[i][j]);
+                    if (HG) ag[i][j] = Mfma<T>::run(fa[i], fg[j], ag[i][j]);
                 }
         }
-        __syncthreads();
+    };
+
+#pragma unroll
+    for (int s = 0; s < NS; ++s) gload(R[s], s);
+    sstore(R[0], 0);
+    __syncthreads();
+    gload(R[0], NS);
+    // stage s = base + u lives in LDS buffer u & 1 and came through register set u % NS (2 NS divides base)
+    for (int base = 0; base < nk; base += 2 * NS) {
+#pragma unroll
+        for (int u = 0; u < 2 * NS; ++u) {
+            const int s = base + u;
+            if (s >= nk) break;
+            mfmas(u & 1);
+            if (s + 1 < nk) sstore(R[(u + 1) % NS], (u + 1) & 1);
+            __syncthreads();
+            gload(R[(u + 1) % NS], s + 1 + NS);
+        }
     }
 
     // D[m][j]: lane holds rows 4*q + e (e = 0..3) of column l16 in every 16 x 16 block.
@@ -159,7 +180,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_gateup_kernel(const T *__r
                 const int m = m0 + 64 * wm + 16 * i + 4 * q + e;
                 if (m < M && col < n_pad) {
                     float hv = 0.f;
-                    if (col < n) hv = has_gate ? activate(ag[i][j][e], act) * au[i][j][e] : activate(au[i][j][e], act);
+                    if (col < n) hv = HG ? activate(ag[i][j][e], act) * au[i][j][e] : activate(au[i][j][e], act);
                     Hh[(size_t)m * ldh + col] = from_float<T>(hv);
                     if (comb && col < n) comb[(size_t)m * ldc + col] = from_float<T>(hv);
                 }
@@ -218,19 +239,34 @@ __global__ __launch_bounds__(kPfThreads) void prefill_down_kernel(const T *__res
     }
     const int ccol = cok ? c0 + 8 * cg : 0;
     const int nlast = n > 0 ? n - 1 : 0;
+    const T *wrow = Wd + (size_t)(2 * kp) * H + ccol;   // this thread's first row pair, stage 0
     uint4 ra[kAL], rb[kBP][2];
+    // stages that end at or before row n (all but possibly the last one) need no row checks
     auto gload = [&](int ks) __attribute__((always_inline)) {
         const int k0 = ks * kPfBK;
 #pragma unroll
         for (int i = 0; i < kAL; ++i) ra[i] = ld16(Hh + aoff[i] + k0);
+        if (k0 + kPfBK <= n) {
+            const T *w = wrow + (size_t)k0 * H;
 #pragma unroll
-        for (int i = 0; i < kBP; ++i) {
-            const int r = k0 + 2 * (kp + 16 * i);
-            const int ra0 = r < n ? r : nlast, ra1 = r + 1 < n ? r + 1 : nlast;
-            rb[i][0] = ld16(Wd + (size_t)ra0 * H + ccol);
-            rb[i][1] = ld16(Wd + (size_t)ra1 * H + ccol);
-            if (!(cok && r < n)) rb[i][0] = zero4;
-            if (!(cok && r + 1 < n)) rb[i][1] = zero4;
+            for (int i = 0; i < kBP; ++i) {
+                rb[i][0] = ld16(w + (size_t)(32 * i) * H);
+                rb[i][1] = ld16(w + (size_t)(32 * i + 1) * H);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kBP; ++i) {
+                const int r = k0 + 2 * (kp + 16 * i);
+                const int ra0 = r < n ? r : nlast, ra1 = r + 1 < n ? r + 1 : nlast;
+                rb[i][0] = ld16(Wd + (size_t)ra0 * H + ccol);
+                rb[i][1] = ld16(Wd + (size_t)ra1 * H + ccol);
+                if (r >= n) rb[i][0] = zero4;
+                if (r + 1 >= n) rb[i][1] = zero4;
+            }
+        }
+        if (!cok) {
+#pragma unroll
+            for (int i = 0; i < kBP; ++i) rb[i][0] = rb[i][1] = zero4;
         }
     };
     auto sstore = [&]() __attribute__((always_inline)) {
@@ -303,13 +339,20 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__rest
 
 int prefill_split_k(int M, int H, int n)
 {
+    // Two blocks fit a CU, so the blocks run in rounds of 2 x CUs; a split costs its K stages plus about two
+    // stages of prologue and epilogue per round.  Take the split with the least rounds x stages.
     const int tiles = ((M + kPfBM - 1) / kPfBM) * ((H + kPfBN - 1) / kPfBN);
-    int s = (2 * device_cu_count() + tiles - 1) / tiles;  // aim at two blocks per CU
+    const int slots = 2 * device_cu_count();
     const int nk = (n + kPfBK - 1) / kPfBK;
-    if (s > nk / 4) s = nk / 4;  // keep at least 4 K stages per split
-    if (s < 1) s = 1;
-    if (s > 16) s = 16;
-    return s;
+    int best = 1;
+    long best_cost = -1;
+    for (int s = 1; s <= 16; ++s) {
+        if (s > 1 && s > nk / 4) break;   // keep at least 4 K stages per split
+        const long rounds = ((long)tiles * s + slots - 1) / slots;
+        const long cost = rounds * ((nk + s - 1) / s + 2);
+        if (best_cost < 0 || cost < best_cost) { best = s; best_cost = cost; }
+    }
+    return best;
 }
 
 int64_t prefill_ldh(int64_t n) { return (n + kPfBK - 1) / kPfBK * kPfBK; }
@@ -333,11 +376,22 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
     const int split_k = prefill_split_k(M, H, n);
     {
         ProfScope ps(ST_K_MLP_PREFILL_GATEUP, stream);
-        const int jt = (int)(ldh / 64), mt = (M + kPfBM - 1) / kPfBM;
+        const int jt = (int)(ldh / 64);
+        // 256-row blocks (one per CU, 25 % less operand traffic) once 128-row tiles outnumber the CUs;
+        // below that a CU holds one block at most and the deeper register pipeline of the small form pays
+        const bool big = M > 128 && jt * ((M + 127) / 128) > device_cu_count();
+        const int mt = big ? (M + 255) / 256 : (M + 127) / 128;
         const int grid = (jt * mt + kXcds - 1) / kXcds * kXcds;
-        ST_LAUNCH(ps, prefill_gateup_kernel<T>, dim3(grid), dim3(kPfThreads), 0, stream,
-                           static_cast<const T *>(x), M, H, static_cast<const T *>(gate), static_cast<const T *>(up), n,
-                           n_dev, Hh, ldh, static_cast<T *>(comb), ldc, act, has_gate, jt, mt);
+        auto go = [&](auto kern, int threads) -> int {
+            ST_LAUNCH(ps, kern, dim3(grid), dim3(threads), 0, stream, static_cast<const T *>(x), M, H,
+                      static_cast<const T *>(gate), static_cast<const T *>(up), n, n_dev, Hh, ldh,
+                      static_cast<T *>(comb), ldc, act, jt, mt);
+            return ST_OK;
+        };
+        int rc;
+        if (big) rc = has_gate ? go(prefill_gateup_kernel<T, true, 256, 2>, 512) : go(prefill_gateup_kernel<T, false, 256, 2>, 512);
+        else rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 4>, 256) : go(prefill_gateup_kernel<T, false, 128, 4>, 256);
+        if (rc != ST_OK) return rc;
     }
     ST_HIP(hipGetLastError());
     {
