@@ -7,13 +7,12 @@
 //             gate and up share the X fragments, the activation is applied
 //             to the accumulators before Hh is written
 //   kernel 2  Out[M,H] = Hh[M,n] Wd[n,H]              Wd rows are the packed
-//             down columns, i.e. K runs down the rows: pairs of rows are
-//             interleaved in registers so that LDS holds Wd^T tiles
-//             ([column][k]) and the fragment reads stay 16-byte
-// Kernel 1: 128 or 256 rows of x by 64 active rows of gate and of up per block, waves of 64 x 64, K
-// stages of 64 through two LDS buffers with the following stages' global loads held in registers.
-// Kernel 2: block tile 128 x 128, 4 waves of 64 x 64, K stage 128 (four MFMA steps), one LDS stage
-// with the next stage's global loads held in registers during the MFMAs.
+//             down columns, i.e. K runs down the rows: the tile sits in LDS
+//             as [k][column] and the fragments are read with the
+//             transposing LDS load (ds_read_b64_tr_b16)
+// Kernel 1: 128 or 256 rows of x by 64 active rows of gate and of up per block; kernel 2: block tile
+// 128 x 128 with split-K.  Both: waves of 64 x 64, K stages of 64 through two LDS buffers with the
+// following stages' global loads held in registers, one barrier per stage.
 //
 // The reference only runs the sparse path for decode (src/modeling_skip.py:236);
 // this is the same contraction as sparse_mlp_forward_cpu
@@ -25,10 +24,7 @@ namespace st {
 constexpr int kPfThreads = 256;
 constexpr int kPfBM = 128;   // rows of x per block
 constexpr int kPfBN = 128;   // output columns per block (kernel 1: 64 gate + 64 up rows)
-constexpr int kPfBK = 128;   // K per stage = 4 MFMA steps; 256 contiguous bytes per row and stage
-constexpr int kPfKB = kPfBK / 32;
-constexpr int kPfCh = kPfBK / 8;   // 16-byte chunks per row and stage
-constexpr int kPfLd = kPfCh + 1;   // LDS row stride in 16-byte units (one pad chunk spreads the banks)
+constexpr int kPfBK = 128;   // columns of Hh are padded to a multiple of this
 
 constexpr int kXcds = 8;
 
@@ -191,15 +187,27 @@ __global__ __launch_bounds__(2 * BM) void prefill_gateup_kernel(const T *__restr
 // ---------------------------------------------------------------------------
 // kernel 2: down projection
 // ---------------------------------------------------------------------------
+// Out[M,H] = Hh[M,n] Wd[n,H].  Wd's rows run along K, so its tile goes to LDS as it is ([k][column], whole
+// 16-byte chunks, the two halves of a row swapped on every second group of eight k so that the four
+// lane groups of a fragment read meet different banks) and the B fragments come out through the
+// transposing LDS read: in a group of 16 lanes, lane j hands in the address of four consecutive columns
+// of row j / 4 and lane i receives column i of the four rows.  K stages of 64, two LDS buffers, two
+// register sets, block tile 128 x 128, 4 waves of 64 x 64, split-K with a fixed-order reduction.
+// H is a multiple of 128 here (the caller routes other widths elsewhere).
+constexpr int kPfBK2 = 64;
+constexpr int kPfLdB = 18;   // Wd rows in LDS: 16 chunks + 2 of padding (288 bytes)
+typedef short pf_v4i16_t __attribute__((ext_vector_type(4)));
+
 template <typename T>
-__global__ __launch_bounds__(kPfThreads) void prefill_down_kernel(const T *__restrict__ Hh, long ldh, int M,
-                                                                  const T *__restrict__ Wd, int H, int n_host,
-                                                                  const int *__restrict__ n_dev,
-                                                                  T *__restrict__ Out, float *__restrict__ partial,
-                                                                  int split_k, int ct, int mt)
+__global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__restrict__ Hh, long ldh, int M,
+                                                                     const T *__restrict__ Wd, int H, int n_host,
+                                                                     const int *__restrict__ n_dev,
+                                                                     T *__restrict__ Out, float *__restrict__ partial,
+                                                                     int split_k, int ct, int mt)
 {
-    __shared__ uint4 sA[kPfBM][kPfLd];
-    __shared__ uint32_t sB[kPfBN][kPfLd * 4];  // [column][k pairs]: Wd^T tile
+    constexpr int NS = 2;
+    __shared__ uint4 sA[2][kPfBM][kPfLd1];
+    __shared__ uint4 sB[2][kPfBK2][kPfLdB];
 
     const int n = device_count(n_host, n_dev);
     const int tile = xcd_tile_id(blockIdx.x, ct * mt * split_k);  // row tiles fastest, then column tiles, then splits
@@ -210,18 +218,15 @@ __global__ __launch_bounds__(kPfThreads) void prefill_down_kernel(const T *__res
     const int l16 = lane & 15, q = lane >> 4;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
 
-    // K range of this split, in whole K stages
-    const int nk_all = (n + kPfBK - 1) / kPfBK;
-    const int per = (nk_all + split_k - 1) / split_k;
-    const int ks0 = z * per, ks1 = (ks0 + per < nk_all) ? ks0 + per : nk_all;
+    // K range of this split, in stages of 64 (Hh is zero-padded to a multiple of 128 columns)
+    const int nst_all = (n + kPfBK - 1) / kPfBK * (kPfBK / kPfBK2);
+    const int per = (nst_all + split_k - 1) / split_k;
+    const int ks0 = z * per, ks1 = (ks0 + per < nst_all) ? ks0 + per : nst_all;
+    const int nst = ks1 - ks0;
 
-    const int ch = tid & (kPfCh - 1), r0 = tid / kPfCh;
-    constexpr int kRowStep = kPfThreads / kPfCh;   // 16
-    constexpr int kAL = kPfBM / kRowStep;          // 8 loads for Hh
-    // Wd tile: this thread owns the row pairs kp + 16 i (rows 2 kp', 2 kp' + 1) and 8 columns
-    const int kp = tid & 15, cg = tid >> 4;
-    constexpr int kBP = kPfBK / 2 / 16;            // 4 row pairs per thread
-    const bool cok = c0 + 8 * cg < H;
+    // staging: chunk ach of the Hh rows ar0 + 32 i; chunk bch (8 columns) of the Wd rows br0 + 16 i
+    const int ach = tid & 7, ar0 = tid >> 3;
+    const int bch = tid & 15, br0 = tid >> 4;
 
     f32x4_t acc[4][4];
 #pragma unroll
@@ -229,80 +234,91 @@ __global__ __launch_bounds__(kPfThreads) void prefill_down_kernel(const T *__res
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    // Unconditional loads from clamped rows; rows of Wd at or beyond n are replaced by zeros (they meet
-    // the zero padding of Hh, but stale rows may hold anything, and 0 * inf is not 0).
-    int aoff[kAL];
+    int aoff[4];
 #pragma unroll
-    for (int i = 0; i < kAL; ++i) {
-        const int r = m0 + r0 + kRowStep * i;
-        aoff[i] = (int)((r < M ? r : M - 1) * ldh) + ch * 8;
+    for (int i = 0; i < 4; ++i) {
+        const int r = m0 + ar0 + 32 * i;
+        aoff[i] = (int)((r < M ? r : M - 1) * ldh) + ach * 8;
     }
-    const int ccol = cok ? c0 + 8 * cg : 0;
+    const T *wcol = Wd + c0 + 8 * bch;
     const int nlast = n > 0 ? n - 1 : 0;
-    const T *wrow = Wd + (size_t)(2 * kp) * H + ccol;   // this thread's first row pair, stage 0
-    uint4 ra[kAL], rb[kBP][2];
-    // stages that end at or before row n (all but possibly the last one) need no row checks
-    auto gload = [&](int ks) __attribute__((always_inline)) {
-        const int k0 = ks * kPfBK;
+    struct Stage { uint4 a[4], b[4]; };
+    Stage R[NS];
+    // Rows of Wd at or beyond n are replaced by zeros (they meet the zero padding of Hh, but stale rows may
+    // hold anything, and 0 * inf is not 0); only a split's last stages can reach them.
+    auto gload = [&](Stage &st, int s) __attribute__((always_inline)) {
+        const int k0 = (s < ks1 ? s : ks1 - 1) * kPfBK2;   // past the end: a harmless repeat
 #pragma unroll
-        for (int i = 0; i < kAL; ++i) ra[i] = ld16(Hh + aoff[i] + k0);
-        if (k0 + kPfBK <= n) {
-            const T *w = wrow + (size_t)k0 * H;
+        for (int i = 0; i < 4; ++i) st.a[i] = ld16(Hh + aoff[i] + k0);
+        if (k0 + kPfBK2 <= n) {
 #pragma unroll
-            for (int i = 0; i < kBP; ++i) {
-                rb[i][0] = ld16(w + (size_t)(32 * i) * H);
-                rb[i][1] = ld16(w + (size_t)(32 * i + 1) * H);
-            }
+            for (int i = 0; i < 4; ++i) st.b[i] = ld16(wcol + (size_t)(k0 + br0 + 16 * i) * H);
         } else {
 #pragma unroll
-            for (int i = 0; i < kBP; ++i) {
-                const int r = k0 + 2 * (kp + 16 * i);
-                const int ra0 = r < n ? r : nlast, ra1 = r + 1 < n ? r + 1 : nlast;
-                rb[i][0] = ld16(Wd + (size_t)ra0 * H + ccol);
-                rb[i][1] = ld16(Wd + (size_t)ra1 * H + ccol);
-                if (r >= n) rb[i][0] = zero4;
-                if (r + 1 >= n) rb[i][1] = zero4;
-            }
-        }
-        if (!cok) {
-#pragma unroll
-            for (int i = 0; i < kBP; ++i) rb[i][0] = rb[i][1] = zero4;
-        }
-    };
-    auto sstore = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < kAL; ++i) sA[r0 + kRowStep * i][ch] = ra[i];
-#pragma unroll
-        for (int i = 0; i < kBP; ++i) {
-            const uint32_t lo[4] = {rb[i][0].x, rb[i][0].y, rb[i][0].z, rb[i][0].w};
-            const uint32_t hi[4] = {rb[i][1].x, rb[i][1].y, rb[i][1].z, rb[i][1].w};
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {  // word v holds columns 2v, 2v+1 of one row
-                sB[8 * cg + 2 * v][kp + 16 * i] = (lo[v] & 0xffffu) | (hi[v] << 16);
-                sB[8 * cg + 2 * v + 1][kp + 16 * i] = (lo[v] >> 16) | (hi[v] & 0xffff0000u);
+            for (int i = 0; i < 4; ++i) {
+                const int r = k0 + br0 + 16 * i;
+                st.b[i] = ld16(wcol + (size_t)(r < n ? r : nlast) * H);
+                if (r >= n) st.b[i] = zero4;
             }
         }
     };
-
-    if (ks0 < ks1) gload(ks0);
-    for (int ks = ks0; ks < ks1; ++ks) {
-        sstore();
-        __syncthreads();
-        if (ks + 1 < ks1) gload(ks + 1);
+    auto sstore = [&](const Stage &st, int b) __attribute__((always_inline)) {
 #pragma unroll
-        for (int kb = 0; kb < kPfKB; ++kb) {
+        for (int i = 0; i < 4; ++i) sA[b][ar0 + 32 * i][ach] = st.a[i];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int k = br0 + 16 * i;
+            sB[b][k][bch ^ (8 * ((k >> 3) & 1))] = st.b[i];
+        }
+    };
+    auto mfmas = [&](int b) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < kPfBK2 / 32; ++kb) {
             uint4 fa[4], fb[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fa[i] = sA[64 * wm + 16 * i + l16][4 * kb + q];
+            for (int i = 0; i < 4; ++i) fa[i] = sA[b][64 * wm + 16 * i + l16][4 * kb + q];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                fb[j] = *reinterpret_cast<const uint4 *>(&sB[64 * wn + 16 * j + l16][16 * kb + 4 * q]);
+            for (int j = 0; j < 4; ++j) {
+                pf_v4i16_t h[2];
+#pragma unroll
+                for (int hh = 0; hh < 2; ++hh) {
+                    const int k = 32 * kb + 8 * q + 4 * hh + (l16 >> 2);   // the row this lane hands in
+                    const int col = 64 * wn + 16 * j + 4 * (l16 & 3);      // first of its four columns
+                    const int chunk = (col >> 3) ^ (8 * ((k >> 3) & 1));
+                    const unsigned short *p = reinterpret_cast<const unsigned short *>(&sB[b][k][chunk]) + (col & 7);
+                    h[hh] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) pf_v4i16_t *)p);
+                }
+                fb[j].x = (unsigned short)h[0][0] | ((unsigned)(unsigned short)h[0][1] << 16);
+                fb[j].y = (unsigned short)h[0][2] | ((unsigned)(unsigned short)h[0][3] << 16);
+                fb[j].z = (unsigned short)h[1][0] | ((unsigned)(unsigned short)h[1][1] << 16);
+                fb[j].w = (unsigned short)h[1][2] | ((unsigned)(unsigned short)h[1][3] << 16);
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
         }
+    };
+
+    if (nst > 0) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) gload(R[s], ks0 + s);
+        sstore(R[0], 0);
         __syncthreads();
+        gload(R[0], ks0 + NS);
+        // stage ks0 + base + u sits in LDS buffer u & 1 and came through register set u % NS
+        for (int base = 0; base < nst; base += 2 * NS) {
+#pragma unroll
+            for (int u = 0; u < 2 * NS; ++u) {
+                const int s = base + u;
+                if (s >= nst) break;
+                mfmas(u & 1);
+                if (s + 1 < nst) sstore(R[(u + 1) % NS], (u + 1) & 1);
+                __syncthreads();
+                gload(R[(u + 1) % NS], ks0 + s + 1 + NS);
+            }
+        }
     }
 
 #pragma unroll
@@ -339,17 +355,17 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__rest
 
 int prefill_split_k(int M, int H, int n)
 {
-    // Two blocks fit a CU, so the blocks run in rounds of 2 x CUs; a split costs its K stages plus about two
+    // Two blocks fit a CU, so the blocks run in rounds of 2 x CUs; a split costs its K stages plus about four
     // stages of prologue and epilogue per round.  Take the split with the least rounds x stages.
     const int tiles = ((M + kPfBM - 1) / kPfBM) * ((H + kPfBN - 1) / kPfBN);
     const int slots = 2 * device_cu_count();
-    const int nk = (n + kPfBK - 1) / kPfBK;
+    const int nk = (n + kPfBK - 1) / kPfBK * (kPfBK / kPfBK2);   // K stages of 64
     int best = 1;
     long best_cost = -1;
     for (int s = 1; s <= 16; ++s) {
-        if (s > 1 && s > nk / 4) break;   // keep at least 4 K stages per split
+        if (s > 1 && s > nk / 8) break;   // keep at least 8 K stages per split
         const long rounds = ((long)tiles * s + slots - 1) / slots;
-        const long cost = rounds * ((nk + s - 1) / s + 2);
+        const long cost = rounds * ((nk + s - 1) / s + 4);
         if (best_cost < 0 || cost < best_cost) { best = s; best_cost = cost; }
     }
     return best;
