@@ -55,8 +55,87 @@ def parse_args():
     ap.add_argument("--active-frac", type=float, default=0.0,
                     help="override the active fraction (e.g. the union of several rows' masks)")
     ap.add_argument("--churn", type=float, default=-1.0, help="override the fraction of the active set swapped per step")
+    ap.add_argument("--prefill", type=int, default=0,
+                    help="time the MFMA path instead: this many rows of x per step through the stack's sparse MLPs, "
+                         "each cache at the union of the rows' masks (roofline against the dense MFMA peak)")
     ap.add_argument("--seed", type=int, default=1236)
     return ap.parse_args()
+
+
+MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 / bf16
+
+
+def prefill_bench(args, wl, torch, st, _lib, syn):
+    """One step = `--prefill` rows of x through the sparse MLP of every layer, the caches holding the union of the
+    rows' masks (per-row masks of the workload's active fraction that share 60 % of their indices)."""
+    import ctypes as C
+    dev = torch.device("cuda:0")
+    dt = getattr(torch, wl.dtype)
+    if wl.dtype == "float32":
+        print("bench.py: --prefill needs an fp16 / bf16 workload (the MFMA kernels)", file=sys.stderr)
+        sys.exit(2)
+    T, H, I = args.prefill, wl.hidden, wl.intermediate
+    layers = args.layers or min(wl.layers, 8)
+    K, W = args.steps, args.warmup
+    stack, g = build_stack(wl, layers, 1, args.seed, torch, st)
+    ns = []
+    for l, layer in enumerate(stack.layers):
+        union = syn.overlapping_token_masks(args.seed + 11 + l, I, T, wl.n_active, 0.6).any(axis=0)
+        layer.cache.update_active_weights(torch.from_numpy(union).to(dev))
+        ns.append(int(union.sum()))
+    x0 = torch.randn(T, H, generator=g, device=dev, dtype=torch.float32).to(dt)
+    bufs = [torch.empty(T, H, device=dev, dtype=dt) for _ in range(2)]
+
+    def step():
+        x = x0
+        for l, layer in enumerate(stack.layers):
+            x = layer.cache.forward(x, wl.act, out=bufs[l & 1])
+        return x
+
+    for _ in range(W):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(K):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms_per_step = e0.elapsed_time(e1) / K
+    L = _lib.lib()
+    cap = 8 * layers
+    kinds, ms = (C.c_int * cap)(), (C.c_float * cap)()
+    per = {}
+    for _ in range(max(4, args.profile_steps // 4)):
+        _lib.check(L.st_profile_enable(cap), "st_profile_enable")
+        step()
+        torch.cuda.synchronize()
+        cnt = L.st_profile_collect(kinds, ms, cap)
+        for i in range(cnt):
+            per.setdefault(_lib.KERNEL_KINDS[kinds[i]], []).append(ms[i] * 1e3)
+    L.st_profile_disable()
+    kern = {k: {"launches": len(v), "mean_us": round(float(np.mean(v)), 3), "median_us": round(float(np.median(v)), 3)}
+            for k, v in per.items()}
+    n_mean = float(np.mean(ns))
+    c = 3 if wl.has_gate else 2
+    flops_layer = 2.0 * c * T * n_mean * H
+    gu_flops = 2.0 * (c - 1) * T * n_mean * H
+    gu_us = kern["mlp_prefill_gateup"]["mean_us"]
+    achieved = gu_flops / (gu_us * 1e-6) / 1e12
+    out = {
+        "metric": "sparse_mlp_prefill_tokens_per_s", "value": round(T / (ms_per_step * 1e-3), 1), "unit": "tok/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": {"float16": "f16", "bfloat16": "bf16"}[wl.dtype],
+        "data": "synthetic (seeded weights, inputs and per-row masks; caches at the union of the rows' masks)",
+        "config": {"workload": wl.name + "_prefill", "layers": layers, "hidden": H, "intermediate": I, "rows": T,
+                   "active_rows_mean": n_mean, "act": wl.act, "has_gate": wl.has_gate},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": None, "kernel": "prefill_gateup_kernel",
+                     "flops_per_launch": gu_flops, "mean_us": gu_us},
+        "stack_tflops": round(layers * flops_layer / (ms_per_step * 1e-3) / 1e12, 1),
+        "kernels_us": kern,
+    }
+    print(json.dumps(out))
 
 
 def build_stack(wl, layers, batch, seed, torch, st):
@@ -165,6 +244,9 @@ def main():
         wl = dataclasses.replace(wl, active_frac=args.active_frac if args.active_frac > 0.0 else wl.active_frac,
                                  churn_lo=args.churn if args.churn >= 0.0 else wl.churn_lo,
                                  churn_hi=args.churn if args.churn >= 0.0 else wl.churn_hi)
+    if args.prefill > 0:
+        prefill_bench(args, wl, torch, st, _lib, syn)
+        return
     layers = args.layers or wl.layers
     B = args.batch or wl.batch
     dev = torch.device("cuda:0")
