@@ -17,6 +17,8 @@
 // The reference only runs the sparse path for decode (src/modeling_skip.py:236);
 // this is the same contraction as sparse_mlp_forward_cpu
 // (sparse_transformers/csrc/sparse_mlp_op.cpp:151-161) for B > 1 rows.
+#include <type_traits>
+
 #include "st_mfma.h"
 
 namespace st {
@@ -151,37 +153,59 @@ __global__ __launch_bounds__(2 * BM) void prefill_gateup_kernel(const T *__restr
     sstore(R[0], 0);
     __syncthreads();
     gload(R[0], NS);
-    // stage s = base + u lives in LDS buffer u & 1 and came through register set u % NS (2 NS divides base)
-    for (int base = 0; base < nk; base += 2 * NS) {
+    // stage s = base + u lives in LDS buffer u & 1 and came through register set u % NS (2 NS divides base).
+    // Whole groups of 2 NS stages run without any checks (as straight-line code the compiler interleaves the
+    // loads, LDS stores and MFMAs; with a test per stage the kernel is a quarter slower); the last group tests.
+    int base = 0;
+    for (; base + 2 * NS < nk; base += 2 * NS) {
 #pragma unroll
         for (int u = 0; u < 2 * NS; ++u) {
-            const int s = base + u;
-            if (s >= nk) break;
             mfmas(u & 1);
-            if (s + 1 < nk) sstore(R[(u + 1) % NS], (u + 1) & 1);
+            sstore(R[(u + 1) % NS], (u + 1) & 1);
             __syncthreads();
-            gload(R[(u + 1) % NS], s + 1 + NS);
+            gload(R[(u + 1) % NS], base + u + 1 + NS);
         }
+    }
+#pragma unroll
+    for (int u = 0; u < 2 * NS; ++u) {
+        const int s = base + u;
+        if (s >= nk) break;
+        mfmas(u & 1);
+        if (s + 1 < nk) sstore(R[(u + 1) % NS], (u + 1) & 1);
+        __syncthreads();
+        gload(R[(u + 1) % NS], s + 1 + NS);
     }
 
     // D[m][j]: lane holds rows 4*q + e (e = 0..3) of column l16 in every 16 x 16 block.
     // Columns n .. n_pad are written as zeros so that kernel 2 can run whole K stages.
+    // One copy of the stores per activation, chosen once: with the activation switched per element the
+    // whole kernel was 4 us slower (all five bodies live in the loop's register budget).
+    auto store = [&](auto actc) __attribute__((always_inline)) {
+        constexpr int ACT = decltype(actc)::value;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int col = j0 + 32 * wn + 16 * j + l16;
+            for (int j = 0; j < 2; ++j) {
+                const int col = j0 + 32 * wn + 16 * j + l16;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int m = m0 + 64 * wm + 16 * i + 4 * q + e;
-                if (m < M && col < n_pad) {
-                    float hv = 0.f;
-                    if (col < n) hv = HG ? activate(ag[i][j][e], act) * au[i][j][e] : activate(au[i][j][e], act);
-                    Hh[(size_t)m * ldh + col] = from_float<T>(hv);
-                    if (comb && col < n) comb[(size_t)m * ldc + col] = from_float<T>(hv);
+                for (int e = 0; e < 4; ++e) {
+                    const int m = m0 + 64 * wm + 16 * i + 4 * q + e;
+                    if (m < M && col < n_pad) {
+                        float hv = 0.f;
+                        if (col < n) hv = HG ? activate(ag[i][j][e], ACT) * au[i][j][e] : activate(au[i][j][e], ACT);
+                        Hh[(size_t)m * ldh + col] = from_float<T>(hv);
+                        if (comb && col < n) comb[(size_t)m * ldc + col] = from_float<T>(hv);
+                    }
                 }
             }
-        }
+    };
+    switch (act) {
+    case ST_ACT_RELU: store(std::integral_constant<int, ST_ACT_RELU>{}); break;
+    case ST_ACT_SILU: store(std::integral_constant<int, ST_ACT_SILU>{}); break;
+    case ST_ACT_GELU_TANH: store(std::integral_constant<int, ST_ACT_GELU_TANH>{}); break;
+    case ST_ACT_SIGMOID: store(std::integral_constant<int, ST_ACT_SIGMOID>{}); break;
+    default: store(std::integral_constant<int, ST_ACT_IDENTITY>{}); break;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -308,16 +332,24 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__
         __syncthreads();
         gload(R[0], ks0 + NS);
         // stage ks0 + base + u sits in LDS buffer u & 1 and came through register set u % NS
-        for (int base = 0; base < nst; base += 2 * NS) {
+        int base = 0;
+        for (; base + 2 * NS < nst; base += 2 * NS) {   // whole groups: no checks
 #pragma unroll
             for (int u = 0; u < 2 * NS; ++u) {
-                const int s = base + u;
-                if (s >= nst) break;
                 mfmas(u & 1);
-                if (s + 1 < nst) sstore(R[(u + 1) % NS], (u + 1) & 1);
+                sstore(R[(u + 1) % NS], (u + 1) & 1);
                 __syncthreads();
-                gload(R[(u + 1) % NS], ks0 + s + 1 + NS);
+                gload(R[(u + 1) % NS], ks0 + base + u + 1 + NS);
             }
+        }
+#pragma unroll
+        for (int u = 0; u < 2 * NS; ++u) {
+            const int s = base + u;
+            if (s >= nst) break;
+            mfmas(u & 1);
+            if (s + 1 < nst) sstore(R[(u + 1) % NS], (u + 1) & 1);
+            __syncthreads();
+            gload(R[(u + 1) % NS], ks0 + s + 1 + NS);
         }
     }
 
