@@ -169,6 +169,29 @@ def test_prefill_agrees_with_decode_kernel():
         assert_close(small.float().cpu().numpy(), big[b0:b0 + 8].float().cpu().numpy(), "float16", f"rows {b0}")
 
 
+@pytest.mark.parametrize("name,M,H,n,dtype,act,has_gate", [
+    ("ragged rows and columns, K loop with whole groups and a tail", 300, 1152, 6000, "bfloat16", "silu", True),
+    ("ungated, K loop shorter than one group", 260, 256, 8500, "float16", "relu", False),
+    ("cfg3 prefill, every row active", 512, 3072, 8192, "bfloat16", "silu", True),
+])
+def test_prefill_wide_blocks(name, M, H, n, dtype, act, has_gate):
+    """With more 128-row tiles than CUs the gate/up kernel switches to 256-row blocks.  The oracle checks the
+    first and the last rows (a full and a ragged row tile); every row is compared with the streaming decode
+    kernel, which the tests above hold against the oracle."""
+    x, cw, dn = _case(23, M, H, n, dtype, has_gate)
+    out, _, cb = _run(x, cw, dn, act, has_gate)
+    out, cb = out.float().cpu().numpy().copy(), cb.float().cpu().numpy().copy()
+    for rows in (slice(0, 6), slice(M - 3, M)):
+        want, wantc = oracle.mlp_forward(x[rows].float().numpy(), cw.float().numpy(), dn.float().numpy().T, act, has_gate)
+        assert_close(out[rows], want, dtype, f"{name} rows {rows}")
+        assert_close(cb[rows, :n], wantc[:, :n], dtype, f"{name} combined rows {rows}")
+    step = 8
+    for b0 in range(0, M, 64):   # a sample of row groups through the streaming kernel
+        small, _, cs = _run(x[b0:b0 + step], cw, dn, act, has_gate)
+        assert_close(out[b0:b0 + step], small.float().cpu().numpy(), dtype, f"{name} rows {b0}.. vs decode kernel")
+        assert_close(cb[b0:b0 + step, :n], cs.float().cpu().numpy()[:, :n], dtype, f"{name} combined rows {b0}..")
+
+
 # ---- MFMA batch kernels (3 <= B < 32, fp16 / bf16, H in {2048, 3072, 4096}) ----
 @pytest.mark.parametrize("name,B,H,n,dtype,act,has_gate", [
     ("cfg3 batch 4", 4, 3072, 4620, "bfloat16", "silu", True),
