@@ -74,10 +74,10 @@ const char *st_last_error(void);
  *   workspace          scratch of st_mlp_workspace_bytes(B,H,n) bytes
  * All rows must be 16-byte aligned (H*sizeof(dtype) % 16 == 0). B <= 4096.
  * B <= 2 (and any B < 32 in fp32 or with a hidden size the MFMA kernels do not
- * cover) runs the streaming decode kernel; 3 <= B < 32 in fp16 / bf16 with H in
+ * cover) runs the streaming decode kernel; 3 <= B <= 32 in fp16 / bf16 with H in
  * {2048, 3072, 4096} runs the MFMA batch kernels (still HBM-bound, one pass over
- * the weights per 16 rows); B >= 32 in fp16 / bf16 with H % 128 == 0 runs the
- * MFMA GEMM kernels (then only columns [0,n) of `combined` are written).
+ * the weights per 16 rows); otherwise B >= 32 in fp16 / bf16 with H % 128 == 0
+ * runs the MFMA GEMM kernels (then only columns [0,n) of `combined` are written).
  * ------------------------------------------------------------------------ */
 int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n);
 int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,

@@ -457,7 +457,7 @@ extern "C" int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n)
 {
     const int64_t G = st::mlp_grid();
     int64_t decode = G * st::kMlpMaxBatchPerLaunch * H * 4;
-    if (B >= st::batch_min_rows() && B < st::kPrefillMinRows) {   // dtype is not known here: size for both paths
+    if (B >= st::batch_min_rows() && B <= st::kBatchMaxRows) {   // dtype is not known here: size for both paths
         const int64_t batch = st::batch_workspace_bytes(H, n);
         decode = batch > decode ? batch : decode;
     }
@@ -488,11 +488,12 @@ extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *g
                             (uintptr_t)workspace;
     ST_REQUIRE((align & 15) == 0, "st_mlp_forward: pointers must be 16-byte aligned");
 
-    if (B >= kPrefillMinRows && dtype != ST_F32 && H % 128 == 0 && n >= 1)
+    const bool batch = B >= batch_min_rows() && B <= kBatchMaxRows && batch_supported(dtype, (int)H);
+    if (B >= kPrefillMinRows && !batch && dtype != ST_F32 && H % 128 == 0 && n >= 1)
         return launch_prefill(dtype, x, (int)B, (int)H, gate_rows, up_rows, down_rows, (int)n, n_dev, out, combined,
                               (long)ldc, workspace, act, has_gate ? 1 : 0, static_cast<hipStream_t>(stream));
 
-    if (B >= batch_min_rows() && batch_supported(dtype, (int)H))
+    if (batch)
         return launch_batch(dtype, x, (int)B, (int)H, gate_rows, up_rows, down_rows, (int)n, n_dev, out, combined,
                             (long)ldc, workspace, act, has_gate ? 1 : 0, static_cast<hipStream_t>(stream));
 

@@ -242,12 +242,14 @@ int launch_mlp_reduce(int dtype, const float *partials, int G, int NB, int bcoun
 // Rows of x from which st_mlp_forward switches from the streaming decode
 // kernel to the MFMA kernels (fp16 / bf16 only).
 constexpr int kPrefillMinRows = 32;
+// 32 rows are two passes of the batch kernels, which beat the GEMM kernels at that size where they apply.
+constexpr int kBatchMaxRows = 32;
 int64_t prefill_workspace_bytes(int64_t M, int64_t H, int64_t n);
 int launch_prefill(int dtype, const void *x, int M, int H, const void *gate, const void *up, const void *down, int n,
                    const int *n_dev, void *out, void *comb, long ldc, void *workspace, int act, int has_gate,
                    hipStream_t stream);
 
-// MFMA kernels for a small batch of rows (batch_min_rows() <= B < 32, fp16 / bf16, supported hidden sizes only).
+// MFMA kernels for a small batch of rows (batch_min_rows() <= B <= 32, fp16 / bf16, supported hidden sizes only).
 int batch_min_rows();
 bool batch_supported(int dtype, int H);
 int64_t batch_workspace_bytes(int64_t H, int64_t n);

@@ -151,7 +151,8 @@ def test_argument_errors():
     ("wide hidden", 96, 4096, 600, "float16", "gelu_pytorch_tanh", True),
 ])
 def test_prefill_mfma_vs_oracle(name, M, H, n, dtype, act, has_gate):
-    """B >= 32 rows in fp16 / bf16 run on the MFMA kernels; same tolerance as decode."""
+    """More than 32 rows (32 where the batch kernels do not apply) in fp16 / bf16 run on the MFMA GEMM kernels; same
+    tolerance as decode."""
     x, cw, dn = _case(21, M, H, n, dtype, has_gate)
     out, _, cb = _run(x, cw, dn, act, has_gate)
     want, wantc = oracle.mlp_forward(x.float().numpy(), cw.float().numpy(), dn.float().numpy().T, act, has_gate)
@@ -192,7 +193,7 @@ def test_prefill_wide_blocks(name, M, H, n, dtype, act, has_gate):
         assert_close(cb[b0:b0 + step, :n], cs.float().cpu().numpy()[:, :n], dtype, f"{name} combined rows {b0}..")
 
 
-# ---- MFMA batch kernels (3 <= B < 32, fp16 / bf16, H in {2048, 3072, 4096}) ----
+# ---- MFMA batch kernels (3 <= B <= 32, fp16 / bf16, H in {2048, 3072, 4096}) ----
 @pytest.mark.parametrize("name,B,H,n,dtype,act,has_gate", [
     ("cfg3 batch 4", 4, 3072, 4620, "bfloat16", "silu", True),
     ("cfg3 batch 16", 16, 3072, 7660, "bfloat16", "silu", True),
@@ -200,6 +201,7 @@ def test_prefill_wide_blocks(name, M, H, n, dtype, act, has_gate):
     ("cfg4 batch 4 fp16 ungated relu", 4, 4096, 1100, "float16", "relu", False),
     ("two passes of 16 + ragged tail", 19, 2048, 1237, "float16", "gelu_pytorch_tanh", True),
     ("31 rows, fewer active rows than blocks", 31, 3072, 97, "bfloat16", "sigmoid", True),
+    ("32 rows: two full passes", 32, 3072, 2867, "float16", "silu", True),
     ("one active row", 5, 2048, 1, "float16", "silu", True),
     ("33 rows per block (two tiles)", 3, 2048, 8450, "float16", "silu", False),
 ])
