@@ -52,19 +52,21 @@ constexpr int kPfBK1 = 64;
 constexpr int kPfCh1 = kPfBK1 / 8;   // 16-byte chunks per row and stage
 constexpr int kPfLd1 = kPfCh1 + 1;   // LDS row stride in 16-byte units
 
-template <typename T, bool HG, int BM, int NS>
-__global__ __launch_bounds__(2 * BM) void prefill_gateup_kernel(const T *__restrict__ X, int M, int H,
-                                                                const T *__restrict__ gate,
-                                                                const T *__restrict__ up, int n_host,
-                                                                const int *__restrict__ n_dev,
-                                                                T *__restrict__ Hh, long ldh,
-                                                                T *__restrict__ comb, long ldc, int act, int jt,
-                                                                int mt)
+// KS = 2: two groups of 2 BM threads share a tile, each runs one half of K through LDS buffers of its own, and the
+// second group's accumulators are added to the first's through LDS at the end (for launches with fewer tiles
+// than half the CUs: the K loop of a block, not the chip, is then what takes the time).
+template <typename T, bool HG, int BM, int NS, int KS>
+__global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__restrict__ X, int M, int H,
+                                                                     const T *__restrict__ gate,
+                                                                     const T *__restrict__ up, int n_host,
+                                                                     const int *__restrict__ n_dev,
+                                                                     T *__restrict__ Hh, long ldh,
+                                                                     T *__restrict__ comb, long ldc, int act, int jt,
+                                                                     int mt)
 {
-    constexpr int kThreads = 2 * BM;
-    __shared__ uint4 sX[2][BM][kPfLd1];
-    __shared__ uint4 sG[2][HG ? 64 : 1][kPfLd1];
-    __shared__ uint4 sU[2][64][kPfLd1];
+    constexpr int kThreads = 2 * BM;                     // per K group
+    constexpr int kRows = BM + (HG ? 128 : 64);          // LDS rows of one buffer: x, gate, up
+    __shared__ uint4 lds[KS * 2 * kRows * kPfLd1];
 
     const int n = device_count(n_host, n_dev);
     const int n_pad = (n + kPfBK - 1) / kPfBK * kPfBK;  // kernel 2 runs whole K stages over Hh
@@ -72,7 +74,10 @@ __global__ __launch_bounds__(2 * BM) void prefill_gateup_kernel(const T *__restr
     if (tile < 0) return;
     const int j0 = (tile / mt) * 64, m0 = (tile % mt) * BM;
     if (j0 >= n_pad) return;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kh = KS > 1 ? threadIdx.x / kThreads : 0;  // K group
+    const int tid = threadIdx.x - kh * kThreads, lane = tid & 63, wave = tid >> 6;
+    uint4 (*sX)[kRows][kPfLd1] = reinterpret_cast<uint4 (*)[kRows][kPfLd1]>(lds + (size_t)kh * 2 * kRows * kPfLd1);
+    constexpr int kGRow = BM, kURow = BM + (HG ? 64 : 0);   // first LDS row of the gate and of the up tile
     const int wm = wave >> 1, wn = wave & 1;
     const int l16 = lane & 15, q = lane >> 4;
 
@@ -106,10 +111,10 @@ __global__ __launch_bounds__(2 * BM) void prefill_gateup_kernel(const T *__restr
     }
     struct Stage { uint4 x[kXL], g[kWL], u[kWL]; };
     Stage R[NS];
-    const int nk = H / kPfBK1;   // even: H is a multiple of 128
-    const int klast = (nk - 1) * kPfBK1;
+    const int nk = H / kPfBK1 / KS;   // stages of this K group (H is a multiple of 128)
+    const int kbase = kh * nk * kPfBK1, klast = (nk - 1) * kPfBK1;
     auto gload = [&](Stage &st, int stage) __attribute__((always_inline)) {
-        const int k0 = stage * kPfBK1 <= klast ? stage * kPfBK1 : klast;   // past the end: a harmless repeat
+        const int k0 = kbase + (stage * kPfBK1 <= klast ? stage * kPfBK1 : klast);   // past the end: a harmless repeat
 #pragma unroll
         for (int i = 0; i < kXL; ++i) st.x[i] = ld16(X + xoff[i] + k0);
 #pragma unroll
@@ -123,29 +128,46 @@ __global__ __launch_bounds__(2 * BM) void prefill_gateup_kernel(const T *__restr
         for (int i = 0; i < kXL; ++i) sX[b][r0 + kRowStep * i][ch] = st.x[i];
 #pragma unroll
         for (int i = 0; i < kWL; ++i) {
-            if (HG) sG[b][r0 + kRowStep * i][ch] = st.g[i];
-            sU[b][r0 + kRowStep * i][ch] = st.u[i];
+            if (HG) sX[b][kGRow + r0 + kRowStep * i][ch] = st.g[i];
+            sX[b][kURow + r0 + kRowStep * i][ch] = st.u[i];
         }
     };
-    auto mfmas = [&](int b) __attribute__((always_inline)) {
+    // fragments of one k step (32 of K): x rows of this wave, its gate and up rows
+    struct Frag { uint4 a[4], g[2], u[2]; };
+    Frag F0, F1;
+    auto lfrag = [&](Frag &F, int b, int kb) __attribute__((always_inline)) {
 #pragma unroll
-        for (int kb = 0; kb < kPfBK1 / 32; ++kb) {
-            uint4 fa[4], fg[2], fu[2];
+        for (int i = 0; i < 4; ++i) F.a[i] = sX[b][64 * wm + 16 * i + l16][4 * kb + q];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fa[i] = sX[b][64 * wm + 16 * i + l16][4 * kb + q];
+        for (int j = 0; j < 2; ++j) {
+            if (HG) F.g[j] = sX[b][kGRow + 32 * wn + 16 * j + l16][4 * kb + q];
+            F.u[j] = sX[b][kURow + 32 * wn + 16 * j + l16][4 * kb + q];
+        }
+    };
+    auto mm = [&](const Frag &F) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                if (HG) fg[j] = sG[b][32 * wn + 16 * j + l16][4 * kb + q];
-                fu[j] = sU[b][32 * wn + 16 * j + l16][4 * kb + q];
+                au[i][j] = Mfma<T>::run(F.a[i], F.u[j], au[i][j]);
+                if (HG) ag[i][j] = Mfma<T>::run(F.a[i], F.g[j], ag[i][j]);
             }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    au[i][j] = Mfma<T>::run(fa[i], fu[j], au[i][j]);
-                    if (HG) ag[i][j] = Mfma<T>::run(fa[i], fg[j], ag[i][j]);
-                }
-        }
+    };
+    // One stage: the second k step's fragments are requested before the MFMAs of the first, the next stage's first
+    // fragments (after the barrier that completes its LDS buffer) before the MFMAs of the second.  The scheduling
+    // barriers keep that order: left alone, the compiler sinks every fragment read to just before its first use.
+    auto stage = [&](int u, bool store, int next) __attribute__((always_inline)) {
+        lfrag(F1, u & 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(F0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (store) sstore(R[(u + 1) % NS], (u + 1) & 1);
+        __syncthreads();
+        lfrag(F0, (u + 1) & 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(F1);
+        __builtin_amdgcn_sched_barrier(0);
+        gload(R[(u + 1) % NS], next);
     };
 
 #pragma unroll
@@ -153,27 +175,47 @@ __global__ __launch_bounds__(2 * BM) void prefill_gateup_kernel(const T *__restr
     sstore(R[0], 0);
     __syncthreads();
     gload(R[0], NS);
+    lfrag(F0, 0, 0);
     // stage s = base + u lives in LDS buffer u & 1 and came through register set u % NS (2 NS divides base).
     // Whole groups of 2 NS stages run without any checks (as straight-line code the compiler interleaves the
     // loads, LDS stores and MFMAs; with a test per stage the kernel is a quarter slower); the last group tests.
     int base = 0;
     for (; base + 2 * NS < nk; base += 2 * NS) {
 #pragma unroll
-        for (int u = 0; u < 2 * NS; ++u) {
-            mfmas(u & 1);
-            sstore(R[(u + 1) % NS], (u + 1) & 1);
-            __syncthreads();
-            gload(R[(u + 1) % NS], base + u + 1 + NS);
-        }
+        for (int u = 0; u < 2 * NS; ++u) stage(u, true, base + u + 1 + NS);
     }
 #pragma unroll
     for (int u = 0; u < 2 * NS; ++u) {
         const int s = base + u;
         if (s >= nk) break;
-        mfmas(u & 1);
-        if (s + 1 < nk) sstore(R[(u + 1) % NS], (u + 1) & 1);
+        stage(u, s + 1 < nk, s + 1 + NS);
+    }
+
+    if constexpr (KS > 1) {
+        // the stage loops end with a barrier, so the buffers are free: group 1 hands its sums over
+        float *red = reinterpret_cast<float *>(lds) + (size_t)wave * (HG ? 16 : 8) * 256 + lane;
+        if (kh == 1) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        red[((i * 2 + j) * 4 + e) * 64] = au[i][j][e];
+                        if (HG) red[((8 + i * 2 + j) * 4 + e) * 64] = ag[i][j][e];
+                    }
+        }
         __syncthreads();
-        gload(R[(u + 1) % NS], s + 1 + NS);
+        if (kh == 1) return;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    au[i][j][e] += red[((i * 2 + j) * 4 + e) * 64];
+                    if (HG) ag[i][j][e] += red[((8 + i * 2 + j) * 4 + e) * 64];
+                }
     }
 
     // D[m][j]: lane holds rows 4*q + e (e = 0..3) of column l16 in every 16 x 16 block.
@@ -436,9 +478,12 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
                       static_cast<T *>(comb), ldc, act, jt, mt);
             return ST_OK;
         };
+        // few tiles: two thread groups per tile, half of K each
+        const bool halves = !big && 2 * jt * mt <= device_cu_count();
         int rc;
-        if (big) rc = has_gate ? go(prefill_gateup_kernel<T, true, 256, 2>, 512) : go(prefill_gateup_kernel<T, false, 256, 2>, 512);
-        else rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 4>, 256) : go(prefill_gateup_kernel<T, false, 128, 4>, 256);
+        if (big) rc = has_gate ? go(prefill_gateup_kernel<T, true, 256, 2, 1>, 512) : go(prefill_gateup_kernel<T, false, 256, 2, 1>, 512);
+        else if (halves) rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 2>, 512) : go(prefill_gateup_kernel<T, false, 128, 2, 2>, 512);
+        else rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 4, 1>, 256) : go(prefill_gateup_kernel<T, false, 128, 4, 1>, 256);
         if (rc != ST_OK) return rc;
     }
     ST_HIP(hipGetLastError());
