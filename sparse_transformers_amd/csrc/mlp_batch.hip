@@ -38,6 +38,8 @@ constexpr int kBtRedFloats = kBtWaves * 2 * 256; // kernel 1: 8 waves x (g,u) x 
 constexpr int kBtStagePitch = 72;                // kernel 2: elements per staged row (64 + 8 pad)
 constexpr int kBtStageBytes = kBtTile * kBtStagePitch * 2;
 
+typedef short bt_v4i16_t __attribute__((ext_vector_type(4)));
+
 // Orders this wave's LDS traffic for the compiler (the hardware executes one wave's LDS operations in order).
 __device__ __forceinline__ void wave_lds_fence()
 {
@@ -243,15 +245,18 @@ __global__ __launch_bounds__(kBtThreads) void batch_down_kernel(
             wave_lds_fence();
 #pragma unroll
             for (int ct = 0; ct < 4; ++ct) {
-                const uint16_t *sp = reinterpret_cast<const uint16_t *>(stage) + 16 * ct + c16;
-                uint32_t v[8];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int rr = e < 4 ? 4 * q + e : 16 + 4 * q + (e - 4);
-                    v[e] = sp[rr * kBtStagePitch];
-                }
-                const uint4 bf = make_uint4(v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16),
-                                            v[6] | (v[7] << 16));
+                // transposing LDS read: in its group of 16 lanes, lane j hands in four columns of row j / 4 and
+                // lane i receives column i of the four rows (rows 4q.. and 16 + 4q.. of the staged piece)
+                const uint16_t *sp = reinterpret_cast<const uint16_t *>(stage) +
+                                     (4 * q + (c16 >> 2)) * kBtStagePitch + 16 * ct + 4 * (c16 & 3);
+                const bt_v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) bt_v4i16_t *)sp);
+                const bt_v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) bt_v4i16_t *)(sp + 16 * kBtStagePitch));
+                const uint4 bf = make_uint4((uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16),
+                                            (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16),
+                                            (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16),
+                                            (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16));
                 acc[p * 4 + ct] = Mfma<T>::run(hf, bf, acc[p * 4 + ct]);
             }
         }
