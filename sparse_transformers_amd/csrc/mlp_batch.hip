@@ -1,9 +1,9 @@
-// Sparse MLP over the active set for a small batch of rows of x (3 <= B < 32):
+// Sparse MLP over the active set for a small batch of rows of x (3 <= B <= 32):
 // still bound by the HBM stream of the active rows, but with B rows of x the
 // multiply-adds no longer fit beside it on the vector ALUs, so they go to the
-// matrix cores (fp16 / bf16 MFMA 16x16x32, fp32 accumulate).  Up to 16 rows of
-// x form the N (kernel 1) / M (kernel 2) dimension of one tile; more rows take
-// another pass over the weights.
+// matrix cores (fp16 / bf16 MFMA 16x16x32, fp32 accumulate).  16 rows of x form
+// the N (kernel 1) / M (kernel 2) dimension of one tile; kernel 1 takes two
+// such tiles in one pass over the gate / up rows, kernel 2 one per pass.
 //
 //   kernel 1  h[b][j] = act(x_b . gate_j) * (x_b . up_j)
 //             one block per CU owns a contiguous range of active rows and works
@@ -11,12 +11,14 @@
 //             dimension: weight fragments go from HBM straight into MFMA
 //             operand registers (16 rows x 64 bytes per load instruction, which
 //             streams as fast as fully coalesced loads on this chip), x comes
-//             from LDS, and the 8 partial tiles are summed through LDS.
+//             from LDS (one tile) or from registers that hold the wave's slice
+//             of the hidden dimension (two tiles), and the 8 partial tiles are
+//             summed through LDS.
 //   kernel 2  out[b][:] = sum_j h[b][j] * down_j[:]
 //             K runs down the rows of the packed down matrix, so the operand
 //             has to be transposed: blocks own (column group, row split), each
 //             wave stages 32 rows x 64 columns in LDS and reads the fragment
-//             column-wise.  Split-K partial rows are summed in a fixed order
+//             with the transposing LDS load.  Split-K partial rows are summed in a fixed order
 //             by kernel 3 (mlp_reduce_kernel).
 // Unlike a per-CU fused kernel this writes no per-CU partial [B,H] rows (which
 // would cost B * 3 MB of extra traffic); h (B * n elements) is the only
@@ -31,7 +33,7 @@ namespace st {
 
 constexpr int kBtThreads = 512;
 constexpr int kBtWaves = kBtThreads / kWave;
-constexpr int kBtRows = 16;                      // rows of x per pass
+constexpr int kBtRows = 16;                      // rows of x per MFMA tile (kernel 1 takes two tiles per pass)
 constexpr int kBtXPad = 8;                       // padding elements per x row in LDS (spreads the banks)
 constexpr int kBtTile = 32;                      // active rows per tile / K per MFMA in kernel 2
 constexpr int kBtRedFloats = kBtWaves * 2 * 256; // kernel 1: 8 waves x (g,u) x 16x16, one subtile at a time
@@ -49,20 +51,25 @@ __device__ __forceinline__ void wave_lds_fence()
 }
 
 // ---------------------------------------------------------------------------
-// kernel 1.  KSW = MFMA k-steps per wave = H / 256; HG = gated.
-// h is written as hbuf[b * ldh + row] for all 16 b (rows of x past B are zeros).
+// kernel 1.  KSW = MFMA k-steps per wave = H / 256; HG = gated; NT = tiles of 16 rows of x (1 or 2).
+// h is written as hbuf[b * ldh + row] for all 16 NT b (rows of x past B are zeros).
 // ---------------------------------------------------------------------------
-template <typename T, int KSW, bool HG>
+template <typename T, int KSW, bool HG, int NT>
 __global__ __launch_bounds__(kBtThreads) void batch_gateup_kernel(
     const T *__restrict__ x, int B, const T *__restrict__ gate, const T *__restrict__ up, int n_host,
     const int *__restrict__ n_dev, T *__restrict__ hbuf, int ldh, T *__restrict__ combined, long ldc, int act)
 {
     constexpr int H = KSW * 256;
+    // k-steps of weight loads in flight per wave (the x fragments take 4 NT KSW registers)
+    constexpr int DEPTH = NT == 1 ? (KSW < 6 ? KSW : 6) : (KSW > 12 ? 4 : 5);
+    // One tile of x (NT == 1) is staged in LDS by the whole block with full-line loads and read from there;
+    // two tiles do not fit, so every wave keeps the fragments of its K slice in registers (measured 0.4-1.2 us
+    // slower per launch for one tile: a fragment load touches 16 half lines).
+    constexpr bool XREG = NT > 1;
     constexpr int XP = H + kBtXPad;
-    constexpr int DEPTH = KSW < 6 ? KSW : 6;   // k-steps of loads in flight per wave
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    T *xs = reinterpret_cast<T *>(lds_raw);                                        // [16][XP]
-    float *red = reinterpret_cast<float *>(lds_raw + (size_t)kBtRows * XP * 2);    // [8][2][4][64]
+    T *xs = reinterpret_cast<T *>(lds_raw);                                                      // [16][XP]
+    float *red = reinterpret_cast<float *>(lds_raw + (XREG ? 0 : (size_t)kBtRows * XP * 2));     // [NT][8][2][4][64]
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), w = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
@@ -74,7 +81,6 @@ __global__ __launch_bounds__(kBtThreads) void batch_gateup_kernel(
     const int jcount = n - row0 < R ? n - row0 : R;
     if (jcount <= 0) return;
 
-    const T *xfrag = xs + (size_t)r * XP + 8 * q + 32 * w;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
     const int ntile = (jcount + kBtTile - 1) / kBtTile;
 
@@ -102,9 +108,26 @@ __global__ __launch_bounds__(kBtThreads) void batch_gateup_kernel(
         }
     };
 
-    // x is requested first, then the first weight loads, so that staging x waits for x alone
-    // (16 rows x H/8 chunks = KSW chunks per thread; rows past B are zeros)
-    {
+    // x is requested first, then the first weight loads.  XREG: lane (r, q) of wave w holds columns
+    // 256 j + 32 w + 8 q .. + 7 of row 16 t + r (rows past B are zeros).
+    const T *xfrag = xs + (size_t)r * XP + 8 * q + 32 * w;
+    uint4 xr[XREG ? NT : 1][XREG ? KSW : 1];
+    if constexpr (XREG) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const bool ok = 16 * t + r < B;
+            const T *xp = x + (size_t)(ok ? 16 * t + r : 0) * H + 8 * q + 32 * w;
+#pragma unroll
+            for (int j = 0; j < KSW; ++j) {
+                xr[t][j] = zero4;
+                if (ok) xr[t][j] = ld16(xp + 256 * j);
+            }
+        }
+        setup(0);
+#pragma unroll
+        for (int j = 0; j < DEPTH; ++j) issue(j);
+    } else {
+        // 16 rows x H/8 chunks = KSW chunks per thread; staging x waits for x alone
         constexpr int chunks = H / 8;
         uint4 xv[KSW];
 #pragma unroll
@@ -123,8 +146,8 @@ __global__ __launch_bounds__(kBtThreads) void batch_gateup_kernel(
             const int b = idx / chunks, c = idx - b * chunks;
             *reinterpret_cast<uint4 *>(xs + (size_t)b * XP + c * 8) = xv[i];
         }
+        __syncthreads();
     }
-    __syncthreads();
 
     for (int t = 0; t < ntile; ++t) {
         if (t > 0) {
@@ -133,39 +156,52 @@ __global__ __launch_bounds__(kBtThreads) void batch_gateup_kernel(
             for (int j = 0; j < DEPTH; ++j) issue(j);
         }
 
-        f32x4_t dg0 = {0.f, 0.f, 0.f, 0.f}, du0 = dg0, dg1 = dg0, du1 = dg0;
+        f32x4_t dg0[NT], du0[NT], dg1[NT], du1[NT];
+#pragma unroll
+        for (int xt = 0; xt < NT; ++xt) {
+            dg0[xt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            du0[xt] = dg0[xt]; dg1[xt] = dg0[xt]; du1[xt] = dg0[xt];
+        }
 #pragma unroll
         for (int j = 0; j < KSW; ++j) {
-            const uint4 xf = *reinterpret_cast<const uint4 *>(xfrag + 256 * j);
-            du0 = Mfma<T>::run(u0[j], xf, du0);
-            if (HG) dg0 = Mfma<T>::run(g0[j], xf, dg0);
-            du1 = Mfma<T>::run(u1[j], xf, du1);
-            if (HG) dg1 = Mfma<T>::run(g1[j], xf, dg1);
+#pragma unroll
+            for (int xt = 0; xt < NT; ++xt) {
+                uint4 xf;
+                if constexpr (XREG) xf = xr[xt][j];
+                else xf = *reinterpret_cast<const uint4 *>(xfrag + 256 * j);
+                du0[xt] = Mfma<T>::run(u0[j], xf, du0[xt]);
+                if (HG) dg0[xt] = Mfma<T>::run(g0[j], xf, dg0[xt]);
+                du1[xt] = Mfma<T>::run(u1[j], xf, du1[xt]);
+                if (HG) dg1[xt] = Mfma<T>::run(g1[j], xf, dg1[xt]);
+            }
             if (j + DEPTH < KSW) issue(j + DEPTH);
         }
 
-        // sum the 8 waves' partial tiles, one 16-row subtile at a time: red[w][g|u][e][lane]
+        // sum the 8 waves' partial tiles, one 16-row subtile at a time: red[xt][w][g|u][e][lane]
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
             if (s == 1 && jcount - t * kBtTile <= 16) break;   // the second subtile is empty (uniform)
-            float *mine = red + (size_t)w * 512 + lane;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                if (HG) mine[e * 64] = s == 0 ? dg0[e] : dg1[e];
-                mine[(4 + e) * 64] = s == 0 ? du0[e] : du1[e];
+            for (int xt = 0; xt < NT; ++xt) {
+                float *mine = red + (size_t)(xt * kBtWaves + w) * 512 + lane;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (HG) mine[e * 64] = s == 0 ? dg0[xt][e] : dg1[xt][e];
+                    mine[(4 + e) * 64] = s == 0 ? du0[xt][e] : du1[xt][e];
+                }
             }
             __syncthreads();
-            if (tid < 256) {
-                // thread -> one element of the 16x16 tile: D register e of D lane dl
-                const int e = tid >> 6, dl = tid & 63;
+            if (tid < 256 * NT) {
+                // thread -> one element of a 16x16 tile: D register e of D lane dl of x tile xt
+                const int xt = tid >> 8, e = (tid >> 6) & 3, dl = tid & 63;
                 float sg = 0.f, su = 0.f;
 #pragma unroll
                 for (int ww = 0; ww < kBtWaves; ++ww) {
-                    if (HG) sg += red[(size_t)ww * 512 + e * 64 + dl];
-                    su += red[(size_t)ww * 512 + (4 + e) * 64 + dl];
+                    if (HG) sg += red[(size_t)(xt * kBtWaves + ww) * 512 + e * 64 + dl];
+                    su += red[(size_t)(xt * kBtWaves + ww) * 512 + (4 + e) * 64 + dl];
                 }
                 const int j = t * kBtTile + 16 * s + 4 * (dl >> 4) + e;   // D rows are 4 * (lane / 16) + e
-                const int b = dl & 15;
+                const int b = 16 * xt + (dl & 15);
                 if (j < jcount) {
                     const float hv = HG ? activate(sg, act) * su : activate(su, act);
                     const int row = row0 + j;
@@ -326,16 +362,16 @@ static int64_t batch_ldh(int64_t n) { return (n + kBtTile - 1) / kBtTile * kBtTi
 
 int64_t batch_workspace_bytes(int64_t H, int64_t n)
 {
-    const int64_t hh = ((int64_t)kBtRows * batch_ldh(n) * 2 + 255) & ~(int64_t)255;
+    const int64_t hh = ((int64_t)2 * kBtRows * batch_ldh(n) * 2 + 255) & ~(int64_t)255;   // h of up to 32 rows of x
     return hh + (int64_t)32 * kBtRows * H * 4;
 }
 
-template <typename T, int KSW, bool HG>
+template <typename T, int KSW, bool HG, int NT>
 static int launch_gateup(const T *x, int B, const T *gate, const T *up, int n, const int *n_dev, T *hbuf, int ldh,
                          T *comb, long ldc, int act, hipStream_t stream)
 {
-    auto kern = batch_gateup_kernel<T, KSW, HG>;
-    const size_t lds = (size_t)kBtRows * (KSW * 256 + kBtXPad) * 2 + (size_t)kBtRedFloats * 4;
+    auto kern = batch_gateup_kernel<T, KSW, HG, NT>;
+    const size_t lds = (NT == 1 ? (size_t)kBtRows * (KSW * 256 + kBtXPad) * 2 : 0) + (size_t)NT * kBtRedFloats * 4;
     static bool attr_set = false;
     if (!attr_set) {
         ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -376,34 +412,42 @@ static int launch_batch_t(const void *x_, int B, int H, const void *gate_, const
     ST_REQUIRE(batch_shape(H, s), "st_mlp_forward: hidden size %d is not supported by the batch kernels", H);
     const int ldh = (int)batch_ldh(n);
     T *hbuf = static_cast<T *>(workspace);
-    const int64_t hh_bytes = ((int64_t)kBtRows * ldh * 2 + 255) & ~(int64_t)255;
+    const int64_t hh_bytes = ((int64_t)2 * kBtRows * ldh * 2 + 255) & ~(int64_t)255;
     float *partial = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + hh_bytes);
     const T *gate = static_cast<const T *>(gate_), *up = static_cast<const T *>(up_);
     const T *down = static_cast<const T *>(down_);
-    for (int b0 = 0; b0 < B; b0 += kBtRows) {
-        const int bc = B - b0 < kBtRows ? B - b0 : kBtRows;
+    // gate / up: one pass over the weights per 32 rows of x; down: one per 16
+    for (int b0 = 0; b0 < B; b0 += 2 * kBtRows) {
+        const int bc = B - b0 < 2 * kBtRows ? B - b0 : 2 * kBtRows;
         const T *x = static_cast<const T *>(x_) + (size_t)b0 * H;
         T *comb = comb_ ? static_cast<T *>(comb_) + (size_t)b0 * ldc : nullptr;
-        T *out = static_cast<T *>(out_) + (size_t)b0 * H;
         int rc;
-#define ST_BT_GATEUP(KSW)                                                                                          \
-    rc = has_gate ? launch_gateup<T, KSW, true>(x, bc, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream)      \
-                  : launch_gateup<T, KSW, false>(x, bc, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream)
+#define ST_BT_GATEUP(KSW)                                                                                              \
+    rc = bc > kBtRows                                                                                                 \
+             ? (has_gate ? launch_gateup<T, KSW, true, 2>(x, bc, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream)   \
+                         : launch_gateup<T, KSW, false, 2>(x, bc, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream)) \
+             : (has_gate ? launch_gateup<T, KSW, true, 1>(x, bc, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream)   \
+                         : launch_gateup<T, KSW, false, 1>(x, bc, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream))
         if (s.ksw == 8) ST_BT_GATEUP(8);
         else if (s.ksw == 12) ST_BT_GATEUP(12);
         else ST_BT_GATEUP(16);
 #undef ST_BT_GATEUP
         if (rc != ST_OK) return rc;
         ST_HIP(hipGetLastError());
-        rc = s.np == 3 ? launch_down<T, 3>(hbuf, ldh, bc, down, H, n, n_dev, partial, s, stream)
-                       : launch_down<T, 2>(hbuf, ldh, bc, down, H, n, n_dev, partial, s, stream);
-        if (rc != ST_OK) return rc;
-        ST_HIP(hipGetLastError());
-        // kernel 3: the row splits' partial rows [rs][16][H] summed in a fixed order (the streaming kernels'
-        // reduce kernel: one memory round trip, 32-column blocks)
-        rc = launch_mlp_reduce(sizeof(T) == 2 && __is_same(T, f16_t) ? ST_F16 : ST_BF16, partial, s.rs, kBtRows, bc, H,
-                               out, stream);
-        if (rc != ST_OK) return rc;
+        for (int t0 = 0; t0 < bc; t0 += kBtRows) {
+            const int tc = bc - t0 < kBtRows ? bc - t0 : kBtRows;
+            const T *ht = hbuf + (size_t)t0 * ldh;
+            T *out = static_cast<T *>(out_) + (size_t)(b0 + t0) * H;
+            rc = s.np == 3 ? launch_down<T, 3>(ht, ldh, tc, down, H, n, n_dev, partial, s, stream)
+                           : launch_down<T, 2>(ht, ldh, tc, down, H, n, n_dev, partial, s, stream);
+            if (rc != ST_OK) return rc;
+            ST_HIP(hipGetLastError());
+            // kernel 3: the row splits' partial rows [rs][16][H] summed in a fixed order (the streaming kernels'
+            // reduce kernel: one memory round trip, 32-column blocks)
+            rc = launch_mlp_reduce(sizeof(T) == 2 && __is_same(T, f16_t) ? ST_F16 : ST_BF16, partial, s.rs, kBtRows, tc,
+                                   H, out, stream);
+            if (rc != ST_OK) return rc;
+        }
     }
     return ST_OK;
 }
