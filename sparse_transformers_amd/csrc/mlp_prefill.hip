@@ -46,16 +46,17 @@ __device__ __forceinline__ int xcd_tile_id(int bid, int ntiles)
 // ---------------------------------------------------------------------------
 // K stages of 64 (one 128-byte line of every row), two LDS buffers and NS register sets: stage s is
 // requested from memory NS stages ahead, goes from registers into the LDS buffer of its parity while the
-// MFMAs of stage s - 1 run, and costs one barrier.  BM rows of x by 64 gate + 64 up rows per block,
-// 2 BM threads, every wave a 64 x (32 + 32) tile.  HG: gated.
+// MFMAs of stage s - 1 run, and costs one barrier.  BM rows of x by 64 (or 32) gate + as many up rows per
+// block, 2 BM threads, every wave a 64 x (32 + 32) (or 64 x (16 + 16)) tile.  HG: gated.
 constexpr int kPfBK1 = 64;
 constexpr int kPfCh1 = kPfBK1 / 8;   // 16-byte chunks per row and stage
 constexpr int kPfLd1 = kPfCh1 + 1;   // LDS row stride in 16-byte units
 
 // KS = 2: two groups of 2 BM threads share a tile, each runs one half of K through LDS buffers of its own, and the
-// second group's accumulators are added to the first's through LDS at the end (for launches with fewer tiles
-// than half the CUs: the K loop of a block, not the chip, is then what takes the time).
-template <typename T, bool HG, int BM, int NS, int KS>
+// second group's accumulators are added to the first's through LDS at the end.
+// JN = 16-row tiles of gate and of up per wave: 2 (64 rows of each per block) or, to make more blocks out of
+// few rows, 1 (32 rows of each).
+template <typename T, bool HG, int BM, int NS, int KS, int JN>
 __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__restrict__ X, int M, int H,
                                                                      const T *__restrict__ gate,
                                                                      const T *__restrict__ up, int n_host,
@@ -65,19 +66,20 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
                                                                      int mt)
 {
     constexpr int kThreads = 2 * BM;                     // per K group
-    constexpr int kRows = BM + (HG ? 128 : 64);          // LDS rows of one buffer: x, gate, up
+    constexpr int kWR = 32 * JN;                         // rows of gate and of up per block
+    constexpr int kRows = BM + (HG ? 2 : 1) * kWR;       // LDS rows of one buffer: x, gate, up
     __shared__ uint4 lds[KS * 2 * kRows * kPfLd1];
 
     const int n = device_count(n_host, n_dev);
     const int n_pad = (n + kPfBK - 1) / kPfBK * kPfBK;  // kernel 2 runs whole K stages over Hh
     const int tile = xcd_tile_id(blockIdx.x, jt * mt);   // row tiles of x fastest: they share the weight rows
     if (tile < 0) return;
-    const int j0 = (tile / mt) * 64, m0 = (tile % mt) * BM;
+    const int j0 = (tile / mt) * kWR, m0 = (tile % mt) * BM;
     if (j0 >= n_pad) return;
     const int kh = KS > 1 ? threadIdx.x / kThreads : 0;  // K group
     const int tid = threadIdx.x - kh * kThreads, lane = tid & 63, wave = tid >> 6;
     uint4 (*sX)[kRows][kPfLd1] = reinterpret_cast<uint4 (*)[kRows][kPfLd1]>(lds + (size_t)kh * 2 * kRows * kPfLd1);
-    constexpr int kGRow = BM, kURow = BM + (HG ? 64 : 0);   // first LDS row of the gate and of the up tile
+    constexpr int kGRow = BM, kURow = BM + (HG ? kWR : 0);   // first LDS row of the gate and of the up tile
     const int wm = wave >> 1, wn = wave & 1;
     const int l16 = lane & 15, q = lane >> 4;
 
@@ -85,13 +87,13 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
     const int ch = tid & (kPfCh1 - 1), r0 = tid / kPfCh1;
     constexpr int kRowStep = kThreads / kPfCh1;
     constexpr int kXL = BM / kRowStep;             // loads for x
-    constexpr int kWL = 64 / kRowStep;             // loads for gate and for up
+    constexpr int kWL = kWR / kRowStep;            // loads for gate and for up
 
-    f32x4_t ag[4][2], au[4][2];
+    f32x4_t ag[4][JN], au[4][JN];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < JN; ++j) {
             ag[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             au[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
@@ -133,22 +135,22 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
         }
     };
     // fragments of one k step (32 of K): x rows of this wave, its gate and up rows
-    struct Frag { uint4 a[4], g[2], u[2]; };
+    struct Frag { uint4 a[4], g[JN], u[JN]; };
     Frag F0, F1;
     auto lfrag = [&](Frag &F, int b, int kb) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) F.a[i] = sX[b][64 * wm + 16 * i + l16][4 * kb + q];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            if (HG) F.g[j] = sX[b][kGRow + 32 * wn + 16 * j + l16][4 * kb + q];
-            F.u[j] = sX[b][kURow + 32 * wn + 16 * j + l16][4 * kb + q];
+        for (int j = 0; j < JN; ++j) {
+            if (HG) F.g[j] = sX[b][kGRow + 16 * JN * wn + 16 * j + l16][4 * kb + q];
+            F.u[j] = sX[b][kURow + 16 * JN * wn + 16 * j + l16][4 * kb + q];
         }
     };
     auto mm = [&](const Frag &F) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < JN; ++j) {
                 au[i][j] = Mfma<T>::run(F.a[i], F.u[j], au[i][j]);
                 if (HG) ag[i][j] = Mfma<T>::run(F.a[i], F.g[j], ag[i][j]);
             }
@@ -193,16 +195,16 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
 
     if constexpr (KS > 1) {
         // the stage loops end with a barrier, so the buffers are free: group 1 hands its sums over
-        float *red = reinterpret_cast<float *>(lds) + (size_t)wave * (HG ? 16 : 8) * 256 + lane;
+        float *red = reinterpret_cast<float *>(lds) + (size_t)wave * (HG ? 8 : 4) * JN * 256 + lane;
         if (kh == 1) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < JN; ++j)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        red[((i * 2 + j) * 4 + e) * 64] = au[i][j][e];
-                        if (HG) red[((8 + i * 2 + j) * 4 + e) * 64] = ag[i][j][e];
+                        red[((i * JN + j) * 4 + e) * 64] = au[i][j][e];
+                        if (HG) red[((4 * JN + i * JN + j) * 4 + e) * 64] = ag[i][j][e];
                     }
         }
         __syncthreads();
@@ -210,11 +212,11 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < JN; ++j)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    au[i][j][e] += red[((i * 2 + j) * 4 + e) * 64];
-                    if (HG) ag[i][j][e] += red[((8 + i * 2 + j) * 4 + e) * 64];
+                    au[i][j][e] += red[((i * JN + j) * 4 + e) * 64];
+                    if (HG) ag[i][j][e] += red[((4 * JN + i * JN + j) * 4 + e) * 64];
                 }
     }
 
@@ -227,8 +229,8 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int col = j0 + 32 * wn + 16 * j + l16;
+            for (int j = 0; j < JN; ++j) {
+                const int col = j0 + 16 * JN * wn + 16 * j + l16;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int m = m0 + 64 * wm + 16 * i + 4 * q + e;
@@ -466,11 +468,15 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
     const int split_k = prefill_split_k(M, H, n);
     {
         ProfScope ps(ST_K_MLP_PREFILL_GATEUP, stream);
-        const int jt = (int)(ldh / 64);
-        // 256-row blocks (one per CU, 25 % less operand traffic) once 128-row tiles outnumber the CUs;
-        // below that a CU holds one block at most and the deeper register pipeline of the small form pays
-        const bool big = M > 128 && jt * ((M + 127) / 128) > device_cu_count();
-        const int mt = big ? (M + 255) / 256 : (M + 127) / 128;
+        const int cus = device_cu_count();
+        const int jt64 = (int)(ldh / 64), mt128 = (M + 127) / 128;
+        // 256-row blocks with 64 + 64 weight rows (one per CU, 25 % less operand traffic) once 128-row tiles
+        // outnumber the CUs; below that, 128-row blocks with 32 + 32 weight rows, and while even those number no
+        // more than the CUs, two thread groups per tile with half of K each (the K loop of a block, not the
+        // chip, is then what takes the time)
+        const bool big = M > 128 && jt64 * mt128 > cus;
+        const bool halves = !big && 2 * jt64 * mt128 <= cus;
+        const int jt = big ? jt64 : 2 * jt64, mt = big ? (M + 255) / 256 : mt128;
         const int grid = (jt * mt + kXcds - 1) / kXcds * kXcds;
         auto go = [&](auto kern, int threads) -> int {
             ST_LAUNCH(ps, kern, dim3(grid), dim3(threads), 0, stream, static_cast<const T *>(x), M, H,
@@ -478,12 +484,10 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
                       static_cast<T *>(comb), ldc, act, jt, mt);
             return ST_OK;
         };
-        // few tiles: two thread groups per tile, half of K each
-        const bool halves = !big && 2 * jt * mt <= device_cu_count();
         int rc;
-        if (big) rc = has_gate ? go(prefill_gateup_kernel<T, true, 256, 2, 1>, 512) : go(prefill_gateup_kernel<T, false, 256, 2, 1>, 512);
-        else if (halves) rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 2>, 512) : go(prefill_gateup_kernel<T, false, 128, 2, 2>, 512);
-        else rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 4, 1>, 256) : go(prefill_gateup_kernel<T, false, 128, 4, 1>, 256);
+        if (big) rc = has_gate ? go(prefill_gateup_kernel<T, true, 256, 2, 1, 2>, 512) : go(prefill_gateup_kernel<T, false, 256, 2, 1, 2>, 512);
+        else if (halves) rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 2, 1>, 512) : go(prefill_gateup_kernel<T, false, 128, 2, 2, 1>, 512);
+        else rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 1, 1>, 256) : go(prefill_gateup_kernel<T, false, 128, 2, 1, 1>, 256);
         if (rc != ST_OK) return rc;
     }
     ST_HIP(hipGetLastError());

@@ -149,6 +149,9 @@ def test_argument_errors():
     ("ungated", 77, 512, 333, "float16", "relu", False),
     ("cfg3 prefill shape, part of the active set", 512, 3072, 1000, "bfloat16", "silu", True),
     ("wide hidden", 96, 4096, 600, "float16", "gelu_pytorch_tanh", True),
+    ("narrow tiles, two K groups, many tiles", 100, 512, 7000, "bfloat16", "silu", True),
+    ("narrow tiles, one K group", 512, 256, 2457, "float16", "silu", True),
+    ("the same, ungated", 500, 384, 2300, "bfloat16", "relu", False),
 ])
 def test_prefill_mfma_vs_oracle(name, M, H, n, dtype, act, has_gate):
     """More than 32 rows (32 where the batch kernels do not apply) in fp16 / bf16 run on the MFMA GEMM kernels; same
