@@ -471,12 +471,14 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         const int cus = device_cu_count();
         const int jt64 = (int)(ldh / 64), mt128 = (M + 127) / 128;
         // 256-row blocks with 64 + 64 weight rows (one per CU, 25 % less operand traffic) once 128-row tiles
-        // outnumber the CUs; below that, 128-row blocks with 32 + 32 weight rows, and while even those number no
-        // more than the CUs, two thread groups per tile with half of K each (the K loop of a block, not the
-        // chip, is then what takes the time)
+        // outnumber the CUs.  Below that the K loop of a block, not the chip, is what takes the time: two thread
+        // groups per tile with half of K each, on 128 x (64 + 64) tiles while those number more than half the
+        // CUs and on 128 x (32 + 32) tiles (twice the blocks) when there are fewer.  What is left (one row tile
+        // and more than 16384 active rows) takes 128 x (32 + 32) tiles without K groups.
         const bool big = M > 128 && jt64 * mt128 > cus;
         const bool halves = !big && 2 * jt64 * mt128 <= cus;
-        const int jt = big ? jt64 : 2 * jt64, mt = big ? (M + 255) / 256 : mt128;
+        const bool wide_halves = !big && !halves && jt64 * mt128 <= cus;   // K groups on 64 + 64 rows: one block per CU
+        const int jt = big || wide_halves ? jt64 : 2 * jt64, mt = big ? (M + 255) / 256 : mt128;
         const int grid = (jt * mt + kXcds - 1) / kXcds * kXcds;
         auto go = [&](auto kern, int threads) -> int {
             ST_LAUNCH(ps, kern, dim3(grid), dim3(threads), 0, stream, static_cast<const T *>(x), M, H,
@@ -487,6 +489,7 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         int rc;
         if (big) rc = has_gate ? go(prefill_gateup_kernel<T, true, 256, 2, 1, 2>, 512) : go(prefill_gateup_kernel<T, false, 256, 2, 1, 2>, 512);
         else if (halves) rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 2, 1>, 512) : go(prefill_gateup_kernel<T, false, 128, 2, 2, 1>, 512);
+        else if (wide_halves) rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 2, 2>, 512) : go(prefill_gateup_kernel<T, false, 128, 2, 2, 2>, 512);
         else rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 1, 1>, 256) : go(prefill_gateup_kernel<T, false, 128, 2, 1, 1>, 256);
         if (rc != ST_OK) return rc;
     }

@@ -150,7 +150,8 @@ def test_argument_errors():
     ("cfg3 prefill shape, part of the active set", 512, 3072, 1000, "bfloat16", "silu", True),
     ("wide hidden", 96, 4096, 600, "float16", "gelu_pytorch_tanh", True),
     ("narrow tiles, two K groups, many tiles", 100, 512, 7000, "bfloat16", "silu", True),
-    ("narrow tiles, one K group", 512, 256, 2457, "float16", "silu", True),
+    ("64-row weight tiles, two K groups", 512, 256, 2457, "float16", "silu", True),
+    ("narrow tiles, one K group (more tiles than CUs, one row tile)", 64, 256, 17000, "float16", "silu", True),
     ("the same, ungated", 500, 384, 2300, "bfloat16", "relu", False),
 ])
 def test_prefill_mfma_vs_oracle(name, M, H, n, dtype, act, has_gate):
