@@ -76,6 +76,7 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
     if (tile < 0) return;
     const int j0 = (tile / mt) * kWR, m0 = (tile % mt) * BM;
     if (j0 >= n_pad) return;
+    ST_TL(0);
     const int kh = KS > 1 ? threadIdx.x / kThreads : 0;  // K group
     const int tid = threadIdx.x - kh * kThreads, lane = tid & 63, wave = tid >> 6;
     uint4 (*sX)[kRows][kPfLd1] = reinterpret_cast<uint4 (*)[kRows][kPfLd1]>(lds + (size_t)kh * 2 * kRows * kPfLd1);
@@ -178,6 +179,7 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
     __syncthreads();
     gload(R[0], NS);
     lfrag(F0, 0, 0);
+    ST_TL(1);
     // stage s = base + u lives in LDS buffer u & 1 and came through register set u % NS (2 NS divides base).
     // Whole groups of 2 NS stages run without any checks (as straight-line code the compiler interleaves the
     // loads, LDS stores and MFMAs; with a test per stage the kernel is a quarter slower); the last group tests.
@@ -186,12 +188,14 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
 #pragma unroll
         for (int u = 0; u < 2 * NS; ++u) stage(u, true, base + u + 1 + NS);
     }
+    ST_TL(2);
 #pragma unroll
     for (int u = 0; u < 2 * NS; ++u) {
         const int s = base + u;
         if (s >= nk) break;
         stage(u, s + 1 < nk, s + 1 + NS);
     }
+    ST_TL(3);
 
     if constexpr (KS > 1) {
         // the stage loops end with a barrier, so the buffers are free: group 1 hands its sums over
@@ -222,8 +226,15 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
 
     // D[m][j]: lane holds rows 4*q + e (e = 0..3) of column l16 in every 16 x 16 block.
     // Columns n .. n_pad are written as zeros so that kernel 2 can run whole K stages.
-    // One copy of the stores per activation, chosen once: with the activation switched per element the
-    // whole kernel was 4 us slower (all five bodies live in the loop's register budget).
+    // The wave's 64 x 16 JN results go through a tile of its own in LDS (free now: the stage loops end with a
+    // barrier) and leave as whole 16-byte chunks, 64 bytes of a row per four lanes; storing every element by
+    // itself took 5.2 us of the 57 the kernel ran.
+    // One copy per activation, chosen once: with the activation switched per element the whole kernel was
+    // 4 us slower (all five bodies live in the loop's register budget).
+    constexpr int kSP = 16 * JN + 8;   // elements per staged row (16-byte multiple, spreads the banks)
+    T *stg = reinterpret_cast<T *>(lds) + (KS > 1 ? (size_t)4 * (HG ? 8 : 4) * JN * 256 * (4 / sizeof(T)) : 0) +
+             (size_t)wave * 64 * kSP;
+    const bool comb16 = comb && ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(comb) & 15) == 0;
     auto store = [&](auto actc) __attribute__((always_inline)) {
         constexpr int ACT = decltype(actc)::value;
 #pragma unroll
@@ -233,15 +244,31 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
                 const int col = j0 + 16 * JN * wn + 16 * j + l16;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const int m = m0 + 64 * wm + 16 * i + 4 * q + e;
-                    if (m < M && col < n_pad) {
-                        float hv = 0.f;
-                        if (col < n) hv = HG ? activate(ag[i][j][e], ACT) * au[i][j][e] : activate(au[i][j][e], ACT);
-                        Hh[(size_t)m * ldh + col] = from_float<T>(hv);
-                        if (comb && col < n) comb[(size_t)m * ldc + col] = from_float<T>(hv);
-                    }
+                    float hv = 0.f;
+                    if (col < n) hv = HG ? activate_fast(ag[i][j][e], ACT) * au[i][j][e] : activate_fast(au[i][j][e], ACT);
+                    stg[(16 * i + 4 * q + e) * kSP + 16 * j + l16] = from_float<T>(hv);
                 }
             }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int c = 0; c < 2 * JN; ++c) {
+            const int idx = lane + 64 * c, row = idx / (2 * JN), ch = idx % (2 * JN);
+            const int m = m0 + 64 * wm + row, col0 = j0 + 16 * JN * wn + 8 * ch;
+            if (m < M && col0 < n_pad) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(stg + row * kSP + 8 * ch);
+                *reinterpret_cast<uint4 *>(Hh + (size_t)m * ldh + col0) = v;
+                if (comb16 && col0 + 8 <= n) {
+                    *reinterpret_cast<uint4 *>(comb + (size_t)m * ldc + col0) = v;
+                } else if (comb) {
+                    const T *sv = stg + row * kSP + 8 * ch;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        if (col0 + k < n) comb[(size_t)m * ldc + col0 + k] = sv[k];
+                }
+            }
+        }
     };
     switch (act) {
     case ST_ACT_RELU: store(std::integral_constant<int, ST_ACT_RELU>{}); break;
@@ -250,6 +277,7 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
     case ST_ACT_SIGMOID: store(std::integral_constant<int, ST_ACT_SIGMOID>{}); break;
     default: store(std::integral_constant<int, ST_ACT_IDENTITY>{}); break;
     }
+    ST_TL(4);
 }
 
 // ---------------------------------------------------------------------------
