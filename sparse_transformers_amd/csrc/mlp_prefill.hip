@@ -302,8 +302,9 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__
                                                                      int split_k, int ct, int mt)
 {
     constexpr int NS = 2;
-    __shared__ uint4 sA[2][kPfBM][kPfLd1];
-    __shared__ uint4 sB[2][kPfBK2][kPfLdB];
+    __shared__ uint4 lds[2 * kPfBM * kPfLd1 + 2 * kPfBK2 * kPfLdB];
+    uint4 (*sA)[kPfBM][kPfLd1] = reinterpret_cast<uint4 (*)[kPfBM][kPfLd1]>(lds);
+    uint4 (*sB)[kPfBK2][kPfLdB] = reinterpret_cast<uint4 (*)[kPfBK2][kPfLdB]>(lds + 2 * kPfBM * kPfLd1);
 
     const int n = device_count(n_host, n_dev);
     const int tile = xcd_tile_id(blockIdx.x, ct * mt * split_k);  // row tiles fastest, then column tiles, then splits
@@ -425,20 +426,41 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__
         }
     }
 
+    if (split_k == 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = c0 + 64 * wn + 16 * j + l16;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int m = m0 + 64 * wm + 16 * i + 4 * q + e;
+                    if (m < M && col < H) Out[(size_t)m * H + col] = from_float<T>(acc[i][j][e]);
+                }
+            }
+        return;
+    }
+    // Partial sums: the wave's 64 x 64 floats go through a tile of its own in LDS (the stage loop ends with a
+    // barrier, so the buffers are free) and leave as 16-byte chunks, 256 bytes of a row per 16 lanes.
+    constexpr int kSP = 64 + 4;   // floats per staged row
+    static_assert(4 * 64 * kSP * 4 <= (int)sizeof(lds), "staging tiles exceed the stage buffers");
+    float *stg = reinterpret_cast<float *>(lds) + (size_t)wave * 64 * kSP;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int col = c0 + 64 * wn + 16 * j + l16;
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int m = m0 + 64 * wm + 16 * i + 4 * q + e;
-                if (m < M && col < H) {
-                    if (split_k == 1) Out[(size_t)m * H + col] = from_float<T>(acc[i][j][e]);
-                    else partial[((size_t)z * M + m) * H + col] = acc[i][j][e];
-                }
-            }
-        }
+            for (int e = 0; e < 4; ++e) stg[(16 * i + 4 * q + e) * kSP + 16 * j + l16] = acc[i][j][e];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+        const int row = 4 * c + q, m = m0 + 64 * wm + row, col = c0 + 64 * wn + 4 * l16;
+        if (m < M && col < H)
+            *reinterpret_cast<float4 *>(partial + ((size_t)z * M + m) * H + col) =
+                *reinterpret_cast<const float4 *>(stg + row * kSP + 4 * l16);
+    }
 }
 
 // out[m, c] = sum over splits of partial[z][m][c]
