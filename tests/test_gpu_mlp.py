@@ -164,6 +164,35 @@ def test_prefill_mfma_vs_oracle(name, M, H, n, dtype, act, has_gate):
     assert_close(cb.float().cpu().numpy()[:, :n], wantc[:, :n], dtype, name + " combined[:, :n]")
 
 
+@pytest.mark.parametrize("M", [40, 200, 512])
+def test_prefill_device_count(M):
+    """The GEMM kernels with the active count read on the device: the tile geometry is laid out for the host's
+    upper bound, rows beyond the device count may hold anything (here NaN), and the result is the one for the
+    exact count."""
+    I, H, n = 6144, 1024, 1500
+    g = torch.Generator().manual_seed(31)
+    gate = (torch.randn(I, H, generator=g) * 0.02).half().to(DEV)
+    up = (torch.randn(I, H, generator=g) * 0.02).half().to(DEV)
+    dn = (torch.randn(I, H, generator=g) * 0.02).half().to(DEV)
+    x = torch.randn(M, H, generator=g).half().to(DEV)
+    ref = torch.empty(M, H, dtype=torch.float16, device=DEV)
+    mlp_forward_rows(x, gate, up, dn, n, None, ref, None, "silu", True)
+    for t in (gate, up, dn):
+        t[n:] = float("nan")
+    n_dev = torch.tensor([n], dtype=torch.int32, device=DEV)
+    out = torch.full((M, H), float("nan"), dtype=torch.float16, device=DEV)
+    mlp_forward_rows(x, gate, up, dn, I, n_dev, out, None, "silu", True)
+    torch.cuda.synchronize()
+    assert_close(out.float().cpu().numpy(), ref.float().cpu().numpy(), "float16", f"device count, {M} rows")
+    want, _ = oracle.mlp_forward(x[:4].float().cpu().numpy(), torch.cat([gate[:n], up[:n]]).float().cpu().numpy(),
+                                 dn[:n].float().cpu().numpy().T, "silu", True)
+    assert_close(out[:4].float().cpu().numpy(), want, "float16", "device count vs oracle")
+    n_dev.fill_(0)
+    out.fill_(1.0)
+    mlp_forward_rows(x, gate, up, dn, I, n_dev, out, None, "silu", True)
+    assert not out.any()                                       # empty active set -> zeros
+
+
 def test_prefill_agrees_with_decode_kernel():
     """The MFMA path (B = 40) and the streaming path (the same rows, 4 at a time) agree to rounding."""
     x, cw, dn = _case(22, 40, 1024, 700, "float16", True)
