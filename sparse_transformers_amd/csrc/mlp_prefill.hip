@@ -50,7 +50,13 @@ __device__ __forceinline__ int xcd_tile_id(int bid, int ntiles)
 // block, 2 BM threads, every wave a 64 x (32 + 32) (or 64 x (16 + 16)) tile.  HG: gated.
 constexpr int kPfBK1 = 64;
 constexpr int kPfCh1 = kPfBK1 / 8;   // 16-byte chunks per row and stage
-constexpr int kPfLd1 = kPfCh1 + 1;   // LDS row stride in 16-byte units
+constexpr int kPfLd1 = kPfCh1;       // LDS row stride in 16-byte units: 128 bytes, no padding
+// K-contiguous tiles in LDS: chunk c of row r sits at position c ^ pf_swz(r).  Rows are 128 bytes, so even and
+// odd rows take the two halves of the 64 banks and the XOR spreads eight row pairs over a half: the 16 rows of a
+// fragment read (one chunk each) and the two rows of a 16-lane store (eight chunks each) both meet every bank
+// once.  (With 144-byte rows the reads were free of conflicts but the stores were not: a third of the LDS
+// cycles of kernel 1 were bank conflicts.)
+__device__ __forceinline__ int pf_swz(int row) { return (row >> 1) & 7; }
 
 // KS = 2: two groups of 2 BM threads share a tile, each runs one half of K through LDS buffers of its own, and the
 // second group's accumulators are added to the first's through LDS at the end.
@@ -87,6 +93,9 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
     // global -> register staging: thread owns chunk `ch` of rows r0 + kRowStep i
     const int ch = tid & (kPfCh1 - 1), r0 = tid / kPfCh1;
     constexpr int kRowStep = kThreads / kPfCh1;
+    static_assert(kRowStep % 16 == 0 && BM % 16 == 0, "the swizzle of a thread's rows must not depend on i");
+    const int chs = ch ^ pf_swz(r0);               // where this thread's chunk sits in its LDS rows
+    const int fsw = pf_swz(l16);                   // the same for the rows this lane reads fragments from
     constexpr int kXL = BM / kRowStep;             // loads for x
     constexpr int kWL = kWR / kRowStep;            // loads for gate and for up
 
@@ -128,11 +137,11 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
     };
     auto sstore = [&](const Stage &st, int b) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < kXL; ++i) sX[b][r0 + kRowStep * i][ch] = st.x[i];
+        for (int i = 0; i < kXL; ++i) sX[b][r0 + kRowStep * i][chs] = st.x[i];
 #pragma unroll
         for (int i = 0; i < kWL; ++i) {
-            if (HG) sX[b][kGRow + r0 + kRowStep * i][ch] = st.g[i];
-            sX[b][kURow + r0 + kRowStep * i][ch] = st.u[i];
+            if (HG) sX[b][kGRow + r0 + kRowStep * i][chs] = st.g[i];
+            sX[b][kURow + r0 + kRowStep * i][chs] = st.u[i];
         }
     };
     // fragments of one k step (32 of K): x rows of this wave, its gate and up rows
@@ -140,11 +149,11 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
     Frag F0, F1;
     auto lfrag = [&](Frag &F, int b, int kb) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) F.a[i] = sX[b][64 * wm + 16 * i + l16][4 * kb + q];
+        for (int i = 0; i < 4; ++i) F.a[i] = sX[b][64 * wm + 16 * i + l16][(4 * kb + q) ^ fsw];
 #pragma unroll
         for (int j = 0; j < JN; ++j) {
-            if (HG) F.g[j] = sX[b][kGRow + 16 * JN * wn + 16 * j + l16][4 * kb + q];
-            F.u[j] = sX[b][kURow + 16 * JN * wn + 16 * j + l16][4 * kb + q];
+            if (HG) F.g[j] = sX[b][kGRow + 16 * JN * wn + 16 * j + l16][(4 * kb + q) ^ fsw];
+            F.u[j] = sX[b][kURow + 16 * JN * wn + 16 * j + l16][(4 * kb + q) ^ fsw];
         }
     };
     auto mm = [&](const Frag &F) __attribute__((always_inline)) {
@@ -361,7 +370,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__
     };
     auto sstore = [&](const Stage &st, int b) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) sA[b][ar0 + 32 * i][ach] = st.a[i];
+        for (int i = 0; i < 4; ++i) sA[b][ar0 + 32 * i][ach ^ pf_swz(ar0)] = st.a[i];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int k = br0 + 16 * i;
@@ -373,7 +382,7 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__
         for (int kb = 0; kb < kPfBK2 / 32; ++kb) {
             uint4 fa[4], fb[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fa[i] = sA[b][64 * wm + 16 * i + l16][4 * kb + q];
+            for (int i = 0; i < 4; ++i) fa[i] = sA[b][64 * wm + 16 * i + l16][(4 * kb + q) ^ pf_swz(l16)];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 pf_v4i16_t h[2];
