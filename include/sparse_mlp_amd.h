@@ -76,7 +76,7 @@ const char *st_last_error(void);
  * B <= 2 (and any B < 32 in fp32 or with a hidden size the MFMA kernels do not
  * cover) runs the streaming decode kernel; 3 <= B <= 32 in fp16 / bf16 with H in
  * {2048, 3072, 4096} runs the MFMA batch kernels (still HBM-bound, one pass over
- * the gate / up rows per 32 rows of x and over the down rows per 16); otherwise B >= 32 in fp16 / bf16 with H % 128 == 0
+ * the weights); otherwise B >= 32 in fp16 / bf16 with H % 128 == 0
  * runs the MFMA GEMM kernels (then only columns [0,n) of `combined` are written).
  * ------------------------------------------------------------------------ */
 int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n);

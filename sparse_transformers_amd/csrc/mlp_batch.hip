@@ -2,8 +2,8 @@
 // still bound by the HBM stream of the active rows, but with B rows of x the
 // multiply-adds no longer fit beside it on the vector ALUs, so they go to the
 // matrix cores (fp16 / bf16 MFMA 16x16x32, fp32 accumulate).  16 rows of x form
-// the N (kernel 1) / M (kernel 2) dimension of one tile; kernel 1 takes two
-// such tiles in one pass over the gate / up rows, kernel 2 one per pass.
+// the N (kernel 1) / M (kernel 2) dimension of one tile; both kernels take up
+// to two such tiles in one pass over the weights.
 //
 //   kernel 1  h[b][j] = act(x_b . gate_j) * (x_b . up_j)
 //             one block per CU owns a contiguous range of active rows and works
@@ -219,9 +219,9 @@ __global__ __launch_bounds__(kBtThreads) void batch_gateup_kernel(
 
 // ---------------------------------------------------------------------------
 // kernel 2.  Block = (column group cg, row split rs); NP = 64-column pieces per
-// block.  partial[(rs * 16 + b) * H + col], fp32.
+// block; NX = tiles of 16 rows of x.  partial[(rs * 16 NX + b) * H + col], fp32.
 // ---------------------------------------------------------------------------
-template <typename T, int NP>
+template <typename T, int NP, int NX>
 __global__ __launch_bounds__(kBtThreads) void batch_down_kernel(
     const T *__restrict__ hbuf, int ldh, int B, const T *__restrict__ down, int H, int n_host,
     const int *__restrict__ n_dev, float *__restrict__ partial, int CG, int RS)
@@ -241,11 +241,13 @@ __global__ __launch_bounds__(kBtThreads) void batch_down_kernel(
 
     T *stage = reinterpret_cast<T *>(lds_raw + (size_t)w * kBtStageBytes);
 
-    f32x4_t acc[NT];
+    f32x4_t acc[NX][NT];
 #pragma unroll
-    for (int i = 0; i < NT; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < NX; ++t)
+#pragma unroll
+        for (int i = 0; i < NT; ++i) acc[t][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    struct Chunk { uint4 d[NP][4]; uint2 hlo, hhi; };
+    struct Chunk { uint4 d[NP][4]; uint2 hlo[NX], hhi[NX]; };
     // 8 rows x 128 bytes per load instruction
     auto load_chunk = [&](Chunk &k, int c) __attribute__((always_inline)) {
 #pragma unroll
@@ -257,21 +259,28 @@ __global__ __launch_bounds__(kBtThreads) void batch_down_kernel(
             for (int p = 0; p < NP; ++p) k.d[p][kk] = ld16(rp + 64 * p);
         }
         // h fragment: k-slots 0..3 <-> rows 4q..4q+3, slots 4..7 <-> rows 16+4q..16+4q+3 of the chunk
-        const T *hp = hbuf + (size_t)c16 * ldh + c * kBtTile + 4 * q;
-        k.hlo = *reinterpret_cast<const uint2 *>(hp);
-        k.hhi = *reinterpret_cast<const uint2 *>(hp + 16);
+#pragma unroll
+        for (int t = 0; t < NX; ++t) {
+            const T *hp = hbuf + (size_t)(16 * t + c16) * ldh + c * kBtTile + 4 * q;
+            k.hlo[t] = *reinterpret_cast<const uint2 *>(hp);
+            k.hhi[t] = *reinterpret_cast<const uint2 *>(hp + 16);
+        }
     };
     auto process = [&](const Chunk &k, int c) __attribute__((always_inline)) {
-        uint32_t a[4] = {k.hlo.x, k.hlo.y, k.hhi.x, k.hhi.y};
-        if (c * kBtTile + kBtTile > n) {   // rows past the count hold nothing defined
+        uint4 hf[NX];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int rlo = c * kBtTile + (i < 2 ? 4 * q + 2 * i : 16 + 4 * q + 2 * (i - 2));
-                if (rlo >= n) a[i] = 0u;
-                else if (rlo + 1 >= n) a[i] &= 0xffffu;
+        for (int t = 0; t < NX; ++t) {
+            uint32_t a[4] = {k.hlo[t].x, k.hlo[t].y, k.hhi[t].x, k.hhi[t].y};
+            if (c * kBtTile + kBtTile > n) {   // rows past the count hold nothing defined
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int rlo = c * kBtTile + (i < 2 ? 4 * q + 2 * i : 16 + 4 * q + 2 * (i - 2));
+                    if (rlo >= n) a[i] = 0u;
+                    else if (rlo + 1 >= n) a[i] &= 0xffffu;
+                }
             }
+            hf[t] = make_uint4(a[0], a[1], a[2], a[3]);
         }
-        const uint4 hf = make_uint4(a[0], a[1], a[2], a[3]);
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             wave_lds_fence();   // the previous piece's reads come first
@@ -293,7 +302,8 @@ __global__ __launch_bounds__(kBtThreads) void batch_down_kernel(
                                             (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16),
                                             (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16),
                                             (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16));
-                acc[p * 4 + ct] = Mfma<T>::run(hf, bf, acc[p * 4 + ct]);
+#pragma unroll
+                for (int t = 0; t < NX; ++t) acc[t][p * 4 + ct] = Mfma<T>::run(hf[t], bf, acc[t][p * 4 + ct]);
             }
         }
     };
@@ -313,23 +323,26 @@ __global__ __launch_bounds__(kBtThreads) void batch_down_kernel(
         c = cn;
     }
 
-    // sum the 8 waves' accumulators through LDS (reuses the staging area)
-    __syncthreads();
-    float *red = reinterpret_cast<float *>(lds_raw);   // [8][NT][4][64]
+    // sum the 8 waves' accumulators through LDS (reuses the staging area), one tile of x at a time
 #pragma unroll
-    for (int i = 0; i < NT; ++i)
+    for (int t = 0; t < NX; ++t) {
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(lds_raw);   // [8][NT][4][64]
 #pragma unroll
-        for (int e = 0; e < 4; ++e) red[((size_t)(w * NT + i) * 4 + e) * 64 + lane] = acc[i][e];
-    __syncthreads();
+        for (int i = 0; i < NT; ++i)
 #pragma unroll
-    for (int m = 0; m < NT * 256 / kBtThreads; ++m) {
-        const int idx = tid + kBtThreads * m;
-        float s = 0.f;
+            for (int e = 0; e < 4; ++e) red[((size_t)(w * NT + i) * 4 + e) * 64 + lane] = acc[t][i][e];
+        __syncthreads();
 #pragma unroll
-        for (int ww = 0; ww < kBtWaves; ++ww) s += red[(size_t)ww * NT * 256 + idx];
-        const int tile = idx >> 8, e = (idx >> 6) & 3, dl = idx & 63;
-        const int b = 4 * (dl >> 4) + e;   // D rows are the rows of x
-        if (b < B) partial[((size_t)rs * kBtRows + b) * H + col0 + 16 * tile + (dl & 15)] = s;
+        for (int m = 0; m < NT * 256 / kBtThreads; ++m) {
+            const int idx = tid + kBtThreads * m;
+            float s = 0.f;
+#pragma unroll
+            for (int ww = 0; ww < kBtWaves; ++ww) s += red[(size_t)ww * NT * 256 + idx];
+            const int tile = idx >> 8, e = (idx >> 6) & 3, dl = idx & 63;
+            const int b = 16 * t + 4 * (dl >> 4) + e;   // D rows are the rows of x
+            if (b < B) partial[((size_t)rs * (kBtRows * NX) + b) * H + col0 + 16 * tile + (dl & 15)] = s;
+        }
     }
 }
 
@@ -384,11 +397,11 @@ static int launch_gateup(const T *x, int B, const T *gate, const T *up, int n, c
     return ST_OK;
 }
 
-template <typename T, int NP>
+template <typename T, int NP, int NX>
 static int launch_down(const T *hbuf, int ldh, int B, const T *down, int H, int n, const int *n_dev, float *partial,
-                       const BatchShape &s, hipStream_t stream)
+                       int cg, int rs, hipStream_t stream)
 {
-    auto kern = batch_down_kernel<T, NP>;
+    auto kern = batch_down_kernel<T, NP, NX>;
     const size_t red = (size_t)kBtWaves * NP * 4 * 256 * 4, stage = (size_t)kBtWaves * kBtStageBytes;
     const size_t lds = red > stage ? red : stage;
     static bool attr_set = false;
@@ -398,8 +411,7 @@ static int launch_down(const T *hbuf, int ldh, int B, const T *down, int H, int 
         attr_set = true;
     }
     ProfScope ps(ST_K_MLP_BATCH_DOWN, stream);
-    ST_LAUNCH(ps, kern, dim3(s.cg * s.rs), dim3(kBtThreads), lds, stream, hbuf, ldh, B, down, H, n, n_dev, partial,
-                       s.cg, s.rs);
+    ST_LAUNCH(ps, kern, dim3(cg * rs), dim3(kBtThreads), lds, stream, hbuf, ldh, B, down, H, n, n_dev, partial, cg, rs);
     return ST_OK;
 }
 
@@ -434,20 +446,26 @@ static int launch_batch_t(const void *x_, int B, int H, const void *gate_, const
 #undef ST_BT_GATEUP
         if (rc != ST_OK) return rc;
         ST_HIP(hipGetLastError());
-        for (int t0 = 0; t0 < bc; t0 += kBtRows) {
-            const int tc = bc - t0 < kBtRows ? bc - t0 : kBtRows;
-            const T *ht = hbuf + (size_t)t0 * ldh;
-            T *out = static_cast<T *>(out_) + (size_t)(b0 + t0) * H;
-            rc = s.np == 3 ? launch_down<T, 3>(ht, ldh, tc, down, H, n, n_dev, partial, s, stream)
-                           : launch_down<T, 2>(ht, ldh, tc, down, H, n, n_dev, partial, s, stream);
-            if (rc != ST_OK) return rc;
-            ST_HIP(hipGetLastError());
-            // kernel 3: the row splits' partial rows [rs][16][H] summed in a fixed order (the streaming kernels'
-            // reduce kernel: one memory round trip, 32-column blocks)
-            rc = launch_mlp_reduce(sizeof(T) == 2 && __is_same(T, f16_t) ? ST_F16 : ST_BF16, partial, s.rs, kBtRows, tc,
-                                   H, out, stream);
-            if (rc != ST_OK) return rc;
+        // kernel 2 takes both tiles of x in one pass with two 64-column pieces per block (three would not leave
+        // registers for a second set of accumulators); kernel 3 sums the row splits' partial rows
+        // [rs][16 or 32][H] in a fixed order (the streaming kernels' reduce kernel)
+        T *out = static_cast<T *>(out_) + (size_t)b0 * H;
+        int rs = s.rs, nbrows = kBtRows;
+        if (bc > kBtRows) {
+            const int cg = H / 128;
+            rs = device_cu_count() / cg;
+            rs = rs < 1 ? 1 : (rs > 16 ? 16 : rs);
+            nbrows = 2 * kBtRows;
+            rc = launch_down<T, 2, 2>(hbuf, ldh, bc, down, H, n, n_dev, partial, cg, rs, stream);
+        } else {
+            rc = s.np == 3 ? launch_down<T, 3, 1>(hbuf, ldh, bc, down, H, n, n_dev, partial, s.cg, s.rs, stream)
+                           : launch_down<T, 2, 1>(hbuf, ldh, bc, down, H, n, n_dev, partial, s.cg, s.rs, stream);
         }
+        if (rc != ST_OK) return rc;
+        ST_HIP(hipGetLastError());
+        rc = launch_mlp_reduce(sizeof(T) == 2 && __is_same(T, f16_t) ? ST_F16 : ST_BF16, partial, rs, nbrows, bc, H, out,
+                               stream);
+        if (rc != ST_OK) return rc;
     }
     return ST_OK;
 }
