@@ -58,8 +58,8 @@ constexpr int kPfLd1 = kPfCh1;       // LDS row stride in 16-byte units: 128 byt
 // cycles of kernel 1 were bank conflicts.)
 __device__ __forceinline__ int pf_swz(int row) { return (row >> 1) & 7; }
 
-// KS = 2: two groups of 2 BM threads share a tile, each runs one half of K through LDS buffers of its own, and the
-// second group's accumulators are added to the first's through LDS at the end.
+// KS = 2 or 4: as many groups of 2 BM threads share a tile, each runs its part of K through LDS buffers of its own,
+// and the other groups' accumulators are added to the first's through LDS at the end.
 // JN = 16-row tiles of gate and of up per wave: 2 (64 rows of each per block) or, to make more blocks out of
 // few rows, 1 (32 rows of each).
 template <typename T, bool HG, int BM, int NS, int KS, int JN>
@@ -206,10 +206,12 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
     }
     ST_TL(3);
 
+    constexpr int kWG = kThreads / 64;                      // waves per K group
+    constexpr int kRedWave = (HG ? 8 : 4) * JN * 256;       // floats one wave hands over
     if constexpr (KS > 1) {
-        // the stage loops end with a barrier, so the buffers are free: group 1 hands its sums over
-        float *red = reinterpret_cast<float *>(lds) + (size_t)wave * (HG ? 8 : 4) * JN * 256 + lane;
-        if (kh == 1) {
+        // the stage loops end with a barrier, so the buffers are free: the other groups hand their sums over
+        float *red = reinterpret_cast<float *>(lds) + ((size_t)(kh > 0 ? kh - 1 : 0) * kWG + wave) * kRedWave + lane;
+        if (kh > 0) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -221,16 +223,18 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
                     }
         }
         __syncthreads();
-        if (kh == 1) return;
+        if (kh > 0) return;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int g = 0; g < KS - 1; ++g)
 #pragma unroll
-            for (int j = 0; j < JN; ++j)
+            for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    au[i][j][e] += red[((i * JN + j) * 4 + e) * 64];
-                    if (HG) ag[i][j][e] += red[((4 * JN + i * JN + j) * 4 + e) * 64];
-                }
+                for (int j = 0; j < JN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        au[i][j][e] += red[(size_t)g * kWG * kRedWave + ((i * JN + j) * 4 + e) * 64];
+                        if (HG) ag[i][j][e] += red[(size_t)g * kWG * kRedWave + ((4 * JN + i * JN + j) * 4 + e) * 64];
+                    }
     }
 
     // D[m][j]: lane holds rows 4*q + e (e = 0..3) of column l16 in every 16 x 16 block.
@@ -241,8 +245,9 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
     // One copy per activation, chosen once: with the activation switched per element the whole kernel was
     // 4 us slower (all five bodies live in the loop's register budget).
     constexpr int kSP = 16 * JN + 8;   // elements per staged row (16-byte multiple, spreads the banks)
-    T *stg = reinterpret_cast<T *>(lds) + (KS > 1 ? (size_t)4 * (HG ? 8 : 4) * JN * 256 * (4 / sizeof(T)) : 0) +
-             (size_t)wave * 64 * kSP;
+    constexpr size_t kStgOff = KS > 1 ? (size_t)(KS - 1) * kWG * kRedWave * (4 / sizeof(T)) : 0;   // past the sums
+    static_assert((kStgOff + (size_t)kWG * 64 * kSP) * sizeof(T) <= sizeof(lds), "epilogue tiles exceed the stage buffers");
+    T *stg = reinterpret_cast<T *>(lds) + kStgOff + (size_t)wave * 64 * kSP;
     const bool comb16 = comb && ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(comb) & 15) == 0;
     auto store = [&](auto actc) __attribute__((always_inline)) {
         constexpr int ACT = decltype(actc)::value;
@@ -532,10 +537,12 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         // 256-row blocks with 64 + 64 weight rows (one per CU, 25 % less operand traffic) once 128-row tiles
         // outnumber the CUs.  Below that the K loop of a block, not the chip, is what takes the time: two thread
         // groups per tile with half of K each, on 128 x (64 + 64) tiles while those number more than half the
-        // CUs and on 128 x (32 + 32) tiles (twice the blocks) when there are fewer.  What is left (one row tile
-        // and more than 16384 active rows) takes 128 x (32 + 32) tiles without K groups.
+        // CUs and on 128 x (32 + 32) tiles (twice the blocks) when there are fewer -- four groups with a quarter
+        // of K each on 64 x (32 + 32) tiles for up to 64 rows of x.  What is left (one row tile and more than
+        // 16384 active rows) takes 128 x (32 + 32) tiles without K groups.
         const bool big = M > 128 && jt64 * mt128 > cus;
         const bool halves = !big && 2 * jt64 * mt128 <= cus;
+        const bool quarters = halves && M <= 64 && H % 256 == 0;   // 64 rows of x: four K groups fit the LDS
         const bool wide_halves = !big && !halves && jt64 * mt128 <= cus;   // K groups on 64 + 64 rows: one block per CU
         const int jt = big || wide_halves ? jt64 : 2 * jt64, mt = big ? (M + 255) / 256 : mt128;
         const int grid = (jt * mt + kXcds - 1) / kXcds * kXcds;
@@ -547,6 +554,7 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         };
         int rc;
         if (big) rc = has_gate ? go(prefill_gateup_kernel<T, true, 256, 2, 1, 2>, 512) : go(prefill_gateup_kernel<T, false, 256, 2, 1, 2>, 512);
+        else if (quarters) rc = has_gate ? go(prefill_gateup_kernel<T, true, 64, 2, 4, 1>, 512) : go(prefill_gateup_kernel<T, false, 64, 2, 4, 1>, 512);
         else if (halves) rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 2, 1>, 512) : go(prefill_gateup_kernel<T, false, 128, 2, 2, 1>, 512);
         else if (wide_halves) rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 2, 2>, 512) : go(prefill_gateup_kernel<T, false, 128, 2, 2, 2>, 512);
         else rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 1, 1>, 256) : go(prefill_gateup_kernel<T, false, 128, 2, 1, 1>, 256);

@@ -153,6 +153,8 @@ def test_argument_errors():
     ("64-row weight tiles, two K groups", 512, 256, 2457, "float16", "silu", True),
     ("narrow tiles, one K group (more tiles than CUs, one row tile)", 64, 256, 17000, "float16", "silu", True),
     ("the same, ungated", 500, 384, 2300, "bfloat16", "relu", False),
+    ("up to 64 rows of x: four K groups", 50, 768, 900, "bfloat16", "silu", True),
+    ("four K groups, ungated", 64, 512, 333, "float16", "sigmoid", False),
 ])
 def test_prefill_mfma_vs_oracle(name, M, H, n, dtype, act, has_gate):
     """More than 32 rows (32 where the batch kernels do not apply) in fp16 / bf16 run on the MFMA GEMM kernels; same
