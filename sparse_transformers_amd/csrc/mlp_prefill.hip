@@ -538,13 +538,15 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         // outnumber the CUs.  Below that the K loop of a block, not the chip, is what takes the time: two thread
         // groups per tile with half of K each, on 128 x (64 + 64) tiles while those number more than half the
         // CUs and on 128 x (32 + 32) tiles (twice the blocks) when there are fewer -- four groups with a quarter
-        // of K each on 64 x (32 + 32) tiles for up to 64 rows of x.  What is left (one row tile and more than
-        // 16384 active rows) takes 128 x (32 + 32) tiles without K groups.
+        // of K each on 64 x (32 + 32) tiles while those fit one per CU.  What is left (one row tile and more
+        // than 16384 active rows) takes 128 x (32 + 32) tiles without K groups.
         const bool big = M > 128 && jt64 * mt128 > cus;
         const bool halves = !big && 2 * jt64 * mt128 <= cus;
-        const bool quarters = halves && M <= 64 && H % 256 == 0;   // 64 rows of x: four K groups fit the LDS
+        // 64-row tiles: four K groups fit the LDS
+        const bool quarters = !big && H % 256 == 0 && 2 * jt64 * ((M + 63) / 64) <= cus;
         const bool wide_halves = !big && !halves && jt64 * mt128 <= cus;   // K groups on 64 + 64 rows: one block per CU
-        const int jt = big || wide_halves ? jt64 : 2 * jt64, mt = big ? (M + 255) / 256 : mt128;
+        const int jt = big || (wide_halves && !quarters) ? jt64 : 2 * jt64;
+        const int mt = big ? (M + 255) / 256 : quarters ? (M + 63) / 64 : mt128;
         const int grid = (jt * mt + kXcds - 1) / kXcds * kXcds;
         auto go = [&](auto kern, int threads) -> int {
             ST_LAUNCH(ps, kern, dim3(grid), dim3(threads), 0, stream, static_cast<const T *>(x), M, H,
