@@ -77,7 +77,7 @@ def test_fused_equals_update_then_forward(dtype, H, I, has_gate):
 
 
 def test_fused_full_size_trace_and_errors():
-    """BASELINE config 2 shape with its churn, then the corner cases: unchanged mask, an update that empties the
+    """The Llama-3.2-3B layer shape (H 3072, I 8192, 35 % active) with 5-15 % churn, then the corner cases: unchanged mask, an update that empties the
     cache (status reported at the next sync, zeros out), recovery from empty."""
     H, I, n = 3072, 8192, 2867
     trace = syn.mask_trace(21, 1, I, n, 12, 0.05, 0.15)[:, 0]
