@@ -48,14 +48,14 @@ def test_forward_vs_oracle_small(dtype, act, has_gate):
 
 
 @pytest.mark.parametrize("name,B,H,n,dtype,act,has_gate", [
-    ("cfg1 llama-1b layer", 1, 2048, 2457, "float32", "silu", True),
-    ("cfg2 llama-3b layer", 1, 3072, 2867, "float16", "silu", True),
-    ("cfg3 batched decode", 4, 3072, 4620, "bfloat16", "silu", True),
-    ("cfg3 batched decode 8", 8, 3072, 6300, "bfloat16", "silu", True),
-    ("cfg4 mistral-7b layer", 1, 4096, 3584, "bfloat16", "silu", True),
-    ("cfg4 mistral-7b batch 2", 2, 4096, 3584, "bfloat16", "silu", True),
-    ("cfg5 relu-llama gated", 1, 4096, 1100, "float16", "relu", True),
-    ("cfg5 relu-llama ungated", 1, 4096, 1100, "float16", "relu", False),
+    ("llama-1b layer fp32", 1, 2048, 2457, "float32", "silu", True),
+    ("llama-3b layer fp16", 1, 3072, 2867, "float16", "silu", True),
+    ("llama-3b bf16, 4 rows, union of masks", 4, 3072, 4620, "bfloat16", "silu", True),
+    ("llama-3b bf16, 8 rows, union of masks", 8, 3072, 6300, "bfloat16", "silu", True),
+    ("mistral-7b layer", 1, 4096, 3584, "bfloat16", "silu", True),
+    ("mistral-7b layer, 2 rows", 2, 4096, 3584, "bfloat16", "silu", True),
+    ("relu-llama-7b gated", 1, 4096, 1100, "float16", "relu", True),
+    ("relu-llama-7b ungated", 1, 4096, 1100, "float16", "relu", False),
     ("fp32 wide rows (two chunks per thread)", 1, 4096, 700, "float32", "silu", True),
     ("fp32 8192 hidden", 1, 8192, 300, "float32", "relu", True),
     ("fp16 8192 hidden", 3, 8192, 900, "float16", "silu", True),
@@ -147,7 +147,7 @@ def test_argument_errors():
     ("small ragged", 130, 256, 200, "float16", "silu", True),
     ("one row tile, n below a K step", 32, 128, 20, "bfloat16", "relu", True),
     ("ungated", 77, 512, 333, "float16", "relu", False),
-    ("cfg3 prefill shape, part of the active set", 512, 3072, 1000, "bfloat16", "silu", True),
+    ("llama-3b prefill shape, part of the active set", 512, 3072, 1000, "bfloat16", "silu", True),
     ("wide hidden", 96, 4096, 600, "float16", "gelu_pytorch_tanh", True),
     ("narrow tiles, two K groups, many tiles", 100, 512, 7000, "bfloat16", "silu", True),
     ("64-row weight tiles, two K groups", 512, 256, 2457, "float16", "silu", True),
@@ -208,7 +208,7 @@ def test_prefill_agrees_with_decode_kernel():
 @pytest.mark.parametrize("name,M,H,n,dtype,act,has_gate", [
     ("ragged rows and columns, K loop with whole groups and a tail", 300, 1152, 6000, "bfloat16", "silu", True),
     ("ungated, K loop shorter than one group", 260, 256, 8500, "float16", "relu", False),
-    ("cfg3 prefill, every row active", 512, 3072, 8192, "bfloat16", "silu", True),
+    ("llama-3b prefill, every row active", 512, 3072, 8192, "bfloat16", "silu", True),
 ])
 def test_prefill_wide_blocks(name, M, H, n, dtype, act, has_gate):
     """With more 128-row tiles than CUs the gate/up kernel switches to 256-row blocks.  The oracle checks the
@@ -230,10 +230,10 @@ def test_prefill_wide_blocks(name, M, H, n, dtype, act, has_gate):
 
 # ---- MFMA batch kernels (3 <= B <= 32, fp16 / bf16, H in {2048, 3072, 4096}) ----
 @pytest.mark.parametrize("name,B,H,n,dtype,act,has_gate", [
-    ("cfg3 batch 4", 4, 3072, 4620, "bfloat16", "silu", True),
-    ("cfg3 batch 16", 16, 3072, 7660, "bfloat16", "silu", True),
-    ("cfg4 batch 8", 8, 4096, 3584, "bfloat16", "silu", True),
-    ("cfg4 batch 4 fp16 ungated relu", 4, 4096, 1100, "float16", "relu", False),
+    ("llama-3b bf16, 4 rows", 4, 3072, 4620, "bfloat16", "silu", True),
+    ("llama-3b bf16, 16 rows", 16, 3072, 7660, "bfloat16", "silu", True),
+    ("mistral-7b bf16, 8 rows", 8, 4096, 3584, "bfloat16", "silu", True),
+    ("4096-wide fp16, 4 rows, ungated relu", 4, 4096, 1100, "float16", "relu", False),
     ("two passes of 16 + ragged tail", 19, 2048, 1237, "float16", "gelu_pytorch_tanh", True),
     ("31 rows, fewer active rows than blocks", 31, 3072, 97, "bfloat16", "sigmoid", True),
     ("32 rows: two full passes", 32, 3072, 2867, "float16", "silu", True),

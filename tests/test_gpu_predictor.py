@@ -23,11 +23,11 @@ def _weights(seed, B, H, r, I, dtype):
 
 
 @pytest.mark.parametrize("B,H,r,I,dtype,frac", [
-    (1, 2048, 64, 8192, "float32", 0.30),      # cfg1
-    (1, 3072, 128, 8192, "float16", 0.35),     # cfg2
-    (8, 4096, 256, 14336, "bfloat16", 0.25),   # cfg4, batch union
-    (1, 4096, 440, 11008, "float16", 0.10),    # cfg5: rank int(0.04 * I), 55 chunks per row
-    (16, 3072, 128, 8192, "bfloat16", 0.30),   # cfg3 decode batch 16
+    (1, 2048, 64, 8192, "float32", 0.30),      # Llama-3.2-1B layer, fp32
+    (1, 3072, 128, 8192, "float16", 0.35),     # Llama-3.2-3B layer, fp16
+    (8, 4096, 256, 14336, "bfloat16", 0.25),   # Mistral-7B layer, bf16, batch union
+    (1, 4096, 440, 11008, "float16", 0.10),    # ReLU-Llama-7B layer: rank int(0.04 * I), 55 chunks per row
+    (16, 3072, 128, 8192, "bfloat16", 0.30),   # Llama-3.2-3B layer, bf16, decode batch 16
     (3, 128, 8, 50, "float16", 0.5),           # tiny / ragged
     (2, 64, 4, 17, "float32", 0.5),
     (1, 1024, 1024, 300, "float16", 0.4),      # rank rows longer than one pass of the wave
