@@ -155,6 +155,8 @@ def test_argument_errors():
     ("the same, ungated", 500, 384, 2300, "bfloat16", "relu", False),
     ("up to 64 rows of x: four K groups", 50, 768, 900, "bfloat16", "silu", True),
     ("four K groups, ungated", 64, 512, 333, "float16", "sigmoid", False),
+    ("one active row", 40, 256, 1, "float16", "silu", True),
+    ("three active rows, several row tiles", 300, 256, 3, "bfloat16", "silu", True),
 ])
 def test_prefill_mfma_vs_oracle(name, M, H, n, dtype, act, has_gate):
     """More than 32 rows (32 where the batch kernels do not apply) in fp16 / bf16 run on the MFMA GEMM kernels; same
