@@ -1,0 +1,43 @@
+"""bench.py prints one JSON line with the fields its callers rely on (short runs in a child process)."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _run(*args):
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), *args], capture_output=True, text=True,
+                       timeout=280, cwd=ROOT)
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = [l for l in p.stdout.splitlines() if l.startswith("{")]
+    assert len(lines) == 1, p.stdout[-2000:]
+    return json.loads(lines[0])
+
+
+def test_decode_line():
+    d = _run("--layers", "2", "--steps", "6", "--warmup", "2", "--profile-steps", "2", "--cpu-layers", "1",
+             "--cpu-steps", "4")
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 6 and d["warmup"] == 2 and d["vs_baseline"] is None
+    assert d["unit"] == "tok/s" and d["value"] > 0 and d["higher_is_better"] is True
+    assert d["config"]["workload"] == "llama3b_stack_fp16" and d["dtype"] == "f16"
+    r = d["roofline"]
+    assert r["bound"] == "hbm" and r["peak"] == 8000.0 and r["unit"] == "GB/s"
+    assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3 and 0 < r["frac"] < 1
+    c = d["cpu_baseline"]
+    assert c["value"] > 0 and c["cores"] >= 1 and c["kind"] in ("reference", "port") and c["sample"]
+
+
+def test_prefill_line():
+    d = _run("--workload", "llama3b_stack_bf16_overlap06", "--prefill", "128", "--layers", "1", "--steps", "3",
+             "--warmup", "1", "--profile-steps", "4")
+    r = d["roofline"]
+    assert d["dtype"] == "bf16" and r["bound"] == "mfma" and r["unit"] == "TFLOP/s" and r["peak"] == 2500.0
+    assert 0 < r["frac"] < 1 and d["value"] > 0 and d["config"]["rows"] == 128

@@ -106,3 +106,14 @@ def test_layer_constants_from_sparsity():
     assert (layer.method, layer.k, layer.std_multiplier) == ("naive", 0, 0.0)
     with pytest.raises(ValueError):
         st.SparseDecodeLayer.from_sparsity(pred, cache, 0.7, "magnitude")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py --gpus N with N > 1 exits with a message before anything touches a GPU."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120, cwd=root)
+    assert p.returncode != 0 and "ONE GPU" in p.stderr
