@@ -364,10 +364,10 @@ def main():
             for l, layer in enumerate(stack.layers):
                 out = stack._pingpong[l & 1]
                 if stack.fused:
-                    layer.cache.update_and_forward(stack.mask_stage[l], x, layer.act, out=out)
+                    layer.cache.update_and_forward(stack.mask_stage[l], x, layer.act, out=out, workspace=stack._mlp_ws)
                 else:
                     layer.cache.update_active_weights_async(stack.mask_stage[l])
-                    layer.cache.forward(x, layer.act, out=out)
+                    layer.cache.forward(x, layer.act, out=out, workspace=stack._mlp_ws)
                 x = out
 
         wall_parts = {}

@@ -958,6 +958,9 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
                "st_cache_update_forward: workspace too small (%lld < %lld)", (long long)workspace_bytes,
                (long long)st_mlp_workspace_bytes(B, c->H, c->I));
     ST_REQUIRE((((uintptr_t)x | (uintptr_t)workspace) & 15) == 0, "st_cache_update_forward: pointers must be 16-byte aligned");
+    // the count after the update is only known on the device: `combined` has to hold the largest possible one
+    ST_REQUIRE(!combined || ldc >= (c->has_gate ? 2 : 1) * c->I,
+               "st_cache_update_forward: ldc=%lld too small for %lld intermediate rows", (long long)ldc, (long long)c->I);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int I = (int)c->I, H = (int)c->H;
     const int row_bytes = (int)(c->H * c->esz), chunks = row_bytes >> 4;

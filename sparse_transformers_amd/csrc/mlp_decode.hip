@@ -451,6 +451,57 @@ int launch_mlp_reduce(int dtype, const float *partials, int G, int NB, int bcoun
     return ST_OK;
 }
 
+// Argument checks shared by the MLP entry points (everything but the workspace size).
+static int check_mlp_args(const char *who, const void *x, int64_t B, int64_t H, const void *gate_rows,
+                          const void *up_rows, const void *down_rows, int64_t n, const void *out, const void *combined,
+                          int64_t ldc, const void *workspace, int act, int dtype, int has_gate)
+{
+    ST_REQUIRE(x && up_rows && down_rows && out && workspace, "%s: null pointer", who);
+    ST_REQUIRE(!has_gate || gate_rows, "%s: has_gate set but gate_rows is null", who);
+    ST_REQUIRE(B >= 1 && B <= 4096, "%s: B=%lld out of range [1,4096]", who, (long long)B);
+    ST_REQUIRE(n >= 0 && n <= (1 << 24), "%s: n=%lld out of range", who, (long long)n);
+    ST_REQUIRE(act >= ST_ACT_RELU && act <= ST_ACT_IDENTITY, "%s: unknown activation %d", who, act);
+    ST_REQUIRE(dtype >= ST_F32 && dtype <= ST_BF16, "%s: unknown dtype %d", who, dtype);
+    const int esz = dtype == ST_F32 ? 4 : 2;
+    ST_REQUIRE(H >= 1 && (H * esz) % 16 == 0, "%s: H=%lld rows are not 16-byte multiples", who, (long long)H);
+    ST_REQUIRE(!combined || ldc >= (has_gate ? 2 * n : n), "%s: ldc=%lld too small for n=%lld", who, (long long)ldc,
+               (long long)n);
+    const uintptr_t align = (uintptr_t)x | (uintptr_t)gate_rows | (uintptr_t)up_rows | (uintptr_t)down_rows |
+                            (uintptr_t)workspace;
+    ST_REQUIRE((align & 15) == 0, "%s: pointers must be 16-byte aligned", who);
+    return ST_OK;
+}
+
+// The streaming decode kernel (+ its reduce) on `workspace`, which holds at least
+// blocks x min(B, 8) x H fp32 partial rows.  Allocates nothing.
+static int mlp_forward_decode(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
+                              const void *down_rows, int64_t n, const int32_t *n_dev, int64_t n_hint, void *out,
+                              void *combined, int64_t ldc, void *workspace, int64_t workspace_bytes, int act,
+                              int dtype, int has_gate, void *stream, const char *who)
+{
+    const int rc = check_mlp_args(who, x, B, H, gate_rows, up_rows, down_rows, n, out, combined, ldc, workspace, act,
+                                  dtype, has_gate);
+    if (rc != ST_OK) return rc;
+    MlpLaunch a;
+    a.G = mlp_grid();
+    const int64_t rows = B <= 2 ? B : (B <= 4 ? 4 : kMlpMaxBatchPerLaunch);   // rows of x per pass (launch_nb)
+    ST_REQUIRE(workspace_bytes >= (int64_t)a.G * rows * H * 4, "%s: workspace too small (%lld < %lld)", who,
+               (long long)workspace_bytes, (long long)((int64_t)a.G * rows * H * 4));
+    a.x = x; a.B = (int)B; a.H = (int)H;
+    a.gate = gate_rows; a.up = up_rows; a.down = down_rows;
+    a.n = (int)n; a.n_dev = n_dev;
+    a.n_hint = (int)(n_hint < 0 ? 0 : (n_hint > n ? n : n_hint));
+    a.out = out; a.combined = combined; a.ldc = (long)ldc;
+    a.partials = static_cast<float *>(workspace);
+    a.act = act; a.has_gate = has_gate ? 1 : 0;
+    a.stream = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+    case ST_F32: return launch_nb<float>(a);
+    case ST_F16: return launch_nb<f16_t>(a);
+    default: return launch_nb<bf16_t>(a);
+    }
+}
+
 }  // namespace st
 
 extern "C" int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n)
@@ -472,21 +523,11 @@ extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *g
                               int dtype, int has_gate, void *stream)
 {
     using namespace st;
-    ST_REQUIRE(x && up_rows && down_rows && out && workspace, "st_mlp_forward: null pointer");
-    ST_REQUIRE(!has_gate || gate_rows, "st_mlp_forward: has_gate set but gate_rows is null");
-    ST_REQUIRE(B >= 1 && B <= 4096, "st_mlp_forward: B=%lld out of range [1,4096]", (long long)B);
-    ST_REQUIRE(n >= 0 && n <= (1 << 24), "st_mlp_forward: n=%lld out of range", (long long)n);
-    ST_REQUIRE(act >= ST_ACT_RELU && act <= ST_ACT_IDENTITY, "st_mlp_forward: unknown activation %d", act);
-    ST_REQUIRE(dtype >= ST_F32 && dtype <= ST_BF16, "st_mlp_forward: unknown dtype %d", dtype);
-    const int esz = dtype == ST_F32 ? 4 : 2;
-    ST_REQUIRE(H >= 1 && (H * esz) % 16 == 0, "st_mlp_forward: H=%lld rows are not 16-byte multiples", (long long)H);
+    const int rc = check_mlp_args("st_mlp_forward", x, B, H, gate_rows, up_rows, down_rows, n, out, combined, ldc,
+                                  workspace, act, dtype, has_gate);
+    if (rc != ST_OK) return rc;
     ST_REQUIRE(workspace_bytes >= st_mlp_workspace_bytes(B, H, n), "st_mlp_forward: workspace too small (%lld < %lld)",
                (long long)workspace_bytes, (long long)st_mlp_workspace_bytes(B, H, n));
-    ST_REQUIRE(!combined || ldc >= (has_gate ? 2 * n : n), "st_mlp_forward: ldc=%lld too small for n=%lld",
-               (long long)ldc, (long long)n);
-    const uintptr_t align = (uintptr_t)x | (uintptr_t)gate_rows | (uintptr_t)up_rows | (uintptr_t)down_rows |
-                            (uintptr_t)workspace;
-    ST_REQUIRE((align & 15) == 0, "st_mlp_forward: pointers must be 16-byte aligned");
 
     const bool batch = B >= batch_min_rows() && B <= kBatchMaxRows && batch_supported(dtype, (int)H);
     if (B >= kPrefillMinRows && !batch && dtype != ST_F32 && H % 128 == 0 && n >= 1)
@@ -497,19 +538,6 @@ extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *g
         return launch_batch(dtype, x, (int)B, (int)H, gate_rows, up_rows, down_rows, (int)n, n_dev, out, combined,
                             (long)ldc, workspace, act, has_gate ? 1 : 0, static_cast<hipStream_t>(stream));
 
-    MlpLaunch a;
-    a.x = x; a.B = (int)B; a.H = (int)H;
-    a.gate = gate_rows; a.up = up_rows; a.down = down_rows;
-    a.n = (int)n; a.n_dev = n_dev;
-    a.n_hint = (int)(n_hint < 0 ? 0 : (n_hint > n ? n : n_hint));
-    a.out = out; a.combined = combined; a.ldc = (long)ldc;
-    a.partials = static_cast<float *>(workspace);
-    a.act = act; a.has_gate = has_gate ? 1 : 0;
-    a.stream = static_cast<hipStream_t>(stream);
-    a.G = mlp_grid();
-    switch (dtype) {
-    case ST_F32: return launch_nb<float>(a);
-    case ST_F16: return launch_nb<f16_t>(a);
-    default: return launch_nb<bf16_t>(a);
-    }
+    return mlp_forward_decode(x, B, H, gate_rows, up_rows, down_rows, n, n_dev, n_hint, out, combined, ldc, workspace,
+                              workspace_bytes, act, dtype, has_gate, stream, "st_mlp_forward");
 }

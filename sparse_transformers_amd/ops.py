@@ -56,30 +56,92 @@ def current_stream_ptr(device: torch.device) -> int:
 _workspaces: dict = {}
 
 
+def mlp_workspace_bytes(B: int, H: int, n: int) -> int:
+    return int(_lib.lib().st_mlp_workspace_bytes(B, H, n))
+
+
 def mlp_workspace(device: torch.device, B: int, H: int, n: int) -> torch.Tensor:
-    need = int(_lib.lib().st_mlp_workspace_bytes(B, H, n))
-    key = (device.index if device.index is not None else torch.cuda.current_device())
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < need:
-        ws = torch.empty(need, dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
+    """Scratch for one forward on the current stream of ``device``.
+
+    One list of buffers per (device, stream): two streams never share scratch, and a buffer that has been
+    handed out is kept for the life of the process -- a HIP graph captured earlier may have its address
+    baked in, so growing must not free it.  Callers that replay graphs or know their largest batch should
+    own a buffer instead (``torch.empty(mlp_workspace_bytes(B, H, I), dtype=torch.uint8)``) and pass it as
+    ``workspace=``."""
+    need = mlp_workspace_bytes(B, H, n)
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    bufs = _workspaces.setdefault(key, [])
+    if not bufs or bufs[-1].numel() < need:
+        grow = max(need, 2 * bufs[-1].numel() if bufs else 0)
+        bufs.append(torch.empty(grow, dtype=torch.uint8, device=device))
+    return bufs[-1]
+
+
+def _check_workspace(ws: torch.Tensor, device: torch.device, need: int) -> torch.Tensor:
+    if ws.dtype != torch.uint8 or not ws.is_cuda or ws.device != device or not ws.is_contiguous():
+        raise ValueError("workspace must be a contiguous uint8 tensor on the cache's GPU")
+    if ws.numel() < need:
+        raise ValueError(f"workspace holds {ws.numel()} bytes, this call needs {need}")
     return ws
+
+
+def check_mlp_args(x2: torch.Tensor, out: torch.Tensor, combined: Optional[torch.Tensor], dtype: torch.dtype,
+                   device: torch.device, H: int, min_cols: int) -> None:
+    """Host-side checks shared by every MLP launch: the kernels index x, out and combined as [B,H] / [B,ldc]
+    arrays of the weights' element type, so a wrong dtype or a short buffer must never reach them."""
+    B = x2.size(0)
+    for name, t in (("x", x2), ("out", out), ("combined", combined)):
+        if t is None:
+            continue
+        if t.dtype != dtype:
+            raise TypeError(f"{name} has dtype {t.dtype}, the weights are {dtype}")
+        if t.device != device:
+            raise RuntimeError(f"{name} is on {t.device}, the weights are on {device}")
+    if x2.dim() != 2 or x2.size(1) != H or not x2.is_contiguous():
+        raise ValueError(f"x must be a contiguous [B,{H}] tensor, got {tuple(x2.shape)}")
+    if out.dim() != 2 or tuple(out.shape) != (B, H) or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous [{B},{H}] tensor, got {tuple(out.shape)}")
+    if combined is not None:
+        if combined.dim() != 2 or combined.size(0) < B or combined.stride(1) != 1 or combined.size(1) < min_cols \
+                or combined.stride(0) < combined.size(1):
+            raise ValueError(f"combined must be [>={B}, >={min_cols}] with unit column stride, got "
+                             f"{tuple(combined.shape)} strides {combined.stride()}")
 
 
 def mlp_forward_rows(x2: torch.Tensor, gate_rows: Optional[torch.Tensor], up_rows: torch.Tensor,
                      down_rows: torch.Tensor, n: int, n_dev: Optional[torch.Tensor], out: torch.Tensor,
-                     combined: Optional[torch.Tensor], act: str, has_gate: bool, n_hint: int = 0) -> None:
+                     combined: Optional[torch.Tensor], act: str, has_gate: bool, n_hint: int = 0,
+                     workspace: Optional[torch.Tensor] = None) -> None:
     """Raw launch on packed rows: gate/up/down are [>=n, H] row-major, x2/out are [B, H].
     With ``n_dev`` (device int32 count) the kernels use min(*n_dev, n); ``n_hint`` is the count the host
     expects, used only to request rows before the device count has arrived."""
     dev = require_gpu(x2, gate_rows, up_rows, down_rows, out, combined, n_dev)
+    if x2.dim() != 2:
+        raise ValueError(f"x must be [B,H], got {tuple(x2.shape)}")
     B, H = x2.shape
-    ws = mlp_workspace(dev, B, H, int(n))
+    n = int(n)
+    for name, t in (("gate_rows", gate_rows if has_gate else None), ("up_rows", up_rows), ("down_rows", down_rows)):
+        if t is None:
+            if name == "gate_rows" and has_gate:
+                raise ValueError("has_gate=True needs gate_rows")
+            continue
+        if t.dim() != 2 or t.size(1) != H or t.size(0) < n or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous [>={n},{H}] tensor, got {tuple(t.shape)}")
+        if t.dtype != x2.dtype:
+            raise TypeError(f"{name} has dtype {t.dtype}, x is {x2.dtype}")
+    if has_gate and gate_rows is None:
+        raise ValueError("has_gate=True needs gate_rows")
+    check_mlp_args(x2, out, combined, up_rows.dtype, dev, H, (2 if has_gate else 1) * n)
+    if n_dev is not None and (n_dev.dtype != torch.int32 or n_dev.numel() < 1):
+        raise TypeError("n_dev must be an int32 GPU tensor")
+    need = mlp_workspace_bytes(B, H, n)
+    ws = mlp_workspace(dev, B, H, n) if workspace is None else _check_workspace(workspace, dev, need)
     if act not in _lib.ACT_CODES:
         raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
     rc = _lib.lib().st_mlp_forward(
         x2.data_ptr(), B, H, gate_rows.data_ptr() if has_gate else None, up_rows.data_ptr(), down_rows.data_ptr(),
-        int(n), n_dev.data_ptr() if n_dev is not None else None, int(n_hint), out.data_ptr(),
+        n, n_dev.data_ptr() if n_dev is not None else None, int(n_hint), out.data_ptr(),
         combined.data_ptr() if combined is not None else None, combined.stride(0) if combined is not None else 0,
         ws.data_ptr(), ws.numel(), _lib.ACT_CODES[act], dtype_code(x2), int(bool(has_gate)), current_stream_ptr(dev))
     _lib.check(rc, "st_mlp_forward")

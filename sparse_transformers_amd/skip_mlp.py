@@ -14,7 +14,8 @@ from typing import List, Optional, Sequence
 
 import torch
 
-from .ops import mask_select, predictor_mask, predictor_scores, select_workspace, sparse_mlp_forward
+from .ops import (mask_select, mlp_workspace_bytes, predictor_mask, predictor_scores, select_workspace,
+                  sparse_mlp_forward)
 from .weight_cache import WeightCache
 
 
@@ -172,15 +173,17 @@ class SparseDecodeLayer:
         self.predict_mask(x_pred, t_ws)
         self.cache.update_active_weights_async(self.mask if mask_override is None else mask_override)
 
-    def mlp(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        return self.cache.forward(x, self.act, out=out)
+    def mlp(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
+            workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return self.cache.forward(x, self.act, out=out, workspace=workspace)
 
     def step(self, x_pred: torch.Tensor, x: torch.Tensor, mask_override: Optional[torch.Tensor] = None,
-             out: Optional[torch.Tensor] = None, t_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+             out: Optional[torch.Tensor] = None, t_ws: Optional[torch.Tensor] = None,
+             workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Predictor mask, then cache update and MLP in one call (``WeightCache.update_and_forward``)."""
         self.predict_mask(x_pred, t_ws)
         return self.cache.update_and_forward(self.mask if mask_override is None else mask_override, x, self.act,
-                                             out=out)
+                                             out=out, workspace=workspace)
 
 
 class SparseMLPStack:
@@ -201,6 +204,8 @@ class SparseMLPStack:
         self._pingpong = [torch.empty(batch, H, dtype=dt, device=dev) for _ in range(2)]
         rmax = max(layer.predictor.lora_size for layer in self.layers)
         self._t_ws = torch.empty(batch * rmax, dtype=torch.float32, device=dev)
+        # the stack owns its MLP scratch: a captured step keeps this address, whatever other callers do later
+        self._mlp_ws = torch.empty(mlp_workspace_bytes(batch, H, I), dtype=torch.uint8, device=dev)
         self.out = self._pingpong[0]
         self.graph = None
         self.use_trace_masks = True
@@ -225,7 +230,7 @@ class SparseMLPStack:
             mask = self.mask_stage[l] if self.use_trace_masks else None
             if self.fused:
                 out = self._pingpong[l & 1]
-                layer.step(self.xp_stage[l], x, mask, out=out, t_ws=self._t_ws)
+                layer.step(self.xp_stage[l], x, mask, out=out, t_ws=self._t_ws, workspace=self._mlp_ws)
                 x = out
                 continue
             if side is not None:
@@ -236,7 +241,7 @@ class SparseMLPStack:
             else:
                 layer.compute_mask_and_update(self.xp_stage[l], mask, t_ws=self._t_ws)
             out = self._pingpong[l & 1]
-            layer.cache.forward(x, layer.act, out=out)
+            layer.cache.forward(x, layer.act, out=out, workspace=self._mlp_ws)
             x = out
         self.out = x
 

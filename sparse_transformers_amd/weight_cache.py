@@ -13,7 +13,8 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .ops import current_stream_ptr, dtype_code, mlp_forward_rows, mlp_workspace, require_gpu
+from .ops import (_check_workspace, check_mlp_args, current_stream_ptr, dtype_code, mlp_forward_rows, mlp_workspace,
+                  mlp_workspace_bytes, require_gpu)
 
 
 class WeightCache:
@@ -158,25 +159,35 @@ class WeightCache:
         return self.down_active[: int(st["n_active"])].t()
 
     # ---------------------------------------------------------------- fast path
+    def _x_rows(self, x: torch.Tensor) -> torch.Tensor:
+        H = self.hidden_size
+        if x.shape[-1] != H:
+            raise ValueError(f"x must have {H} columns, got {tuple(x.shape)}")
+        if x.dtype != self.dtype or x.device != self.device:
+            raise TypeError(f"x must be {self.dtype} on {self.device}, got {x.dtype} on {x.device}")
+        x2 = x.reshape(-1, H)
+        return x2 if x2.is_contiguous() else x2.contiguous()
+
     def update_and_forward(self, mask: torch.Tensor, x: torch.Tensor, act: str = "silu",
                            out: Optional[torch.Tensor] = None, combined: Optional[torch.Tensor] = None,
-                           n_hint: Optional[int] = None) -> torch.Tensor:
+                           n_hint: Optional[int] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``update_active_weights(mask)`` followed by the sparse MLP on x, enqueued as one call and never
         touching the host.  For one row of x this is a single kernel that takes the rows whose index
         changed straight from the pool (and writes them back to the active buffers on the way); the
         cache state and the result equal those of the two separate calls bit for bit.  ``n_hint`` (default:
-        the last count the host saw) only steers what the kernel requests before it knows the true count."""
+        the last count the host saw) only steers what the kernel requests before it knows the true count.
+        ``workspace``: a caller-owned uint8 buffer of ``mlp_workspace_bytes(B, H, I)`` bytes (default: one
+        kept per device and stream)."""
         m = self._mask_arg(mask)
-        H = self.hidden_size
-        x2 = x.reshape(-1, H)
-        if not x2.is_contiguous():
-            x2 = x2.contiguous()
-        if x2.dtype != self.dtype or x2.device != self.device:
-            raise TypeError(f"x must be {self.dtype} on {self.device}")
+        H, I = self.hidden_size, self.intermediate_size
+        x2 = self._x_rows(x)
         B = x2.size(0)
         if out is None:
             out = torch.empty_like(x2)
-        ws = mlp_workspace(self.device, B, H, self.intermediate_size)
+        # the count after the update is not known on the host: `combined` must hold the largest possible one
+        check_mlp_args(x2, out, combined, self.dtype, self.device, H, (2 if self.has_gate else 1) * I)
+        need = mlp_workspace_bytes(B, H, I)
+        ws = mlp_workspace(self.device, B, H, I) if workspace is None else _check_workspace(workspace, self.device, need)
         if act not in _lib.ACT_CODES:
             raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
         rc = _lib.lib().st_cache_update_forward(
@@ -189,16 +200,14 @@ class WeightCache:
         return out.view(x.shape)
 
     def forward(self, x: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor] = None,
-                combined: Optional[torch.Tensor] = None) -> torch.Tensor:
+                combined: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Sparse MLP on the cache's packed rows; the active count is read on the device."""
-        H = self.hidden_size
-        x2 = x.reshape(-1, H)
-        if not x2.is_contiguous():
-            x2 = x2.contiguous()
+        x2 = self._x_rows(x)
         if out is None:
             out = torch.empty_like(x2)
         # the last count the host saw is only a prefetch hint; the kernels read the true one on the device
+        # (mlp_forward_rows checks out / combined against the cache's dtype, device and capacity I)
         mlp_forward_rows(x2, self.gate_active, self.up_active, self.down_active, self.intermediate_size,
                          self.n_active_dev, out, combined, act, self.has_gate,
-                         n_hint=int(self._host_state[_lib.STATE_N_ACTIVE]))
+                         n_hint=int(self._host_state[_lib.STATE_N_ACTIVE]), workspace=workspace)
         return out.view(x.shape)

@@ -162,3 +162,40 @@ def test_constructor_validation():
     assert wc.get_concat_weight().shape == (I, H)
     with pytest.raises(ValueError):                                                   # rows must be 16-byte multiples
         st.WeightCache(ones, 6, _t(gate[:, :6]), _t(up[:, :6]), _t(down[:6]), True)
+
+
+def test_fast_path_argument_errors():
+    """forward / update_and_forward check x, out and combined against the cache on the host: a wrong dtype, a
+    short output or a combined buffer that cannot hold every possible count raises instead of reaching a kernel."""
+    I, H = 256, 128
+    g = torch.Generator().manual_seed(3)
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.05).half().to(DEV)
+    cache = st.WeightCache(torch.ones(I, dtype=torch.bool, device=DEV), H, mk(I, H), mk(I, H), mk(H, I), True)
+    mask = (torch.rand(I, generator=g) < 0.5).to(DEV)
+    x = mk(1, H)
+    for call in (lambda **kw: cache.forward(kw.pop("x", x), "silu", **kw),
+                 lambda **kw: cache.update_and_forward(mask, kw.pop("x", x), "silu", **kw)):
+        with pytest.raises(TypeError):
+            call(x=x.float())                                   # fp32 x on an fp16 cache
+        with pytest.raises(ValueError):
+            call(x=mk(1, H // 2))                               # wrong hidden size
+        with pytest.raises(TypeError):
+            call(out=torch.empty(1, H, dtype=torch.float32, device=DEV))
+        with pytest.raises(ValueError):
+            call(out=torch.empty(1, H // 2, dtype=torch.float16, device=DEV))
+        with pytest.raises(ValueError):
+            call(combined=torch.empty(1, I, dtype=torch.float16, device=DEV))   # gated: needs 2*I columns
+        with pytest.raises(ValueError):
+            call(workspace=torch.empty(16, dtype=torch.uint8, device=DEV))
+        with pytest.raises((TypeError, RuntimeError)):
+            call(x=x.cpu())
+    # and the C entry point itself refuses a short row pitch for `combined`
+    from sparse_transformers_amd import _lib
+    comb = torch.empty(1, I, dtype=torch.float16, device=DEV)
+    out = torch.empty(1, H, dtype=torch.float16, device=DEV)
+    ws = torch.empty(int(_lib.lib().st_mlp_workspace_bytes(1, H, I)), dtype=torch.uint8, device=DEV)
+    rc = _lib.lib().st_cache_update_forward(cache._h, mask.data_ptr(), x.data_ptr(), 1, 0, out.data_ptr(), comb.data_ptr(),
+                                            I, ws.data_ptr(), ws.numel(), 1, torch.cuda.current_stream().cuda_stream)
+    assert rc == _lib.ST_ERR_ARG and "ldc" in _lib.last_error()
+    # nothing above changed the cache
+    assert cache.get_num_active() == I

@@ -101,3 +101,35 @@ def test_predictor_argument_errors():
     sd = {"down.weight": A, "up.weight": Bm}
     p = st.FastLoRAProjection.from_state_dict(sd, device=DEV, dtype=torch.float32)   # the reference's checkpoint keys
     assert p.lora_size == 8 and p.intermediate_size == 32
+
+
+def test_loaded_checkpoints_drive_the_hip_predictor(tmp_path):
+    """Predictor files as the reference's trainer writes them (fp32 state dicts with keys down.weight [r,H] and
+    up.weight [I,r] under final_predictor_layer_{i}_lora_{pct}pct.pt, src/trainer.py:569-585), loaded the way
+    benchmark.py:460-468 consumes them, here onto the GPU in fp16: the loaded predictors' scores and masks against
+    the oracle on the same (fp16-rounded) weights."""
+    H, I = 3072, 8192
+    r = int(I * 0.016)          # the trainer's sizing rule int(I * pct / 100) at 1.6 % -> 131 -> not a multiple of 8
+    r = (r // 8) * 8            # 128: rank rows must be 16-byte multiples in fp16
+    g = torch.Generator().manual_seed(21)
+    want = []
+    for layer in range(2):
+        sd = {"down.weight": torch.randn(r, H, generator=g) * 0.02, "up.weight": torch.randn(I, r, generator=g) * 0.02}
+        torch.save(sd, tmp_path / st.FastLoRAProjection.checkpoint_name(layer, 1.6))
+        want.append(sd)
+    preds = st.load_predictors(str(tmp_path), 2, 1.6, device=DEV, dtype=torch.float16)
+    x = torch.randn(2, H, generator=g).half()
+    for p, sd in zip(preds, want):
+        assert p.down_weight.is_cuda and p.down_weight.dtype == torch.float16 and p.lora_size == r
+        A, Bm = sd["down.weight"].half().float().numpy(), sd["up.weight"].half().float().numpy()
+        s_ref = oracle.predictor_scores(x.float().numpy(), A, Bm)
+        s = p(x.to(DEV)).cpu().numpy()
+        scale = np.abs(s_ref).max()
+        assert np.abs(s - s_ref).max() <= 2e-6 * scale
+        thr = syn.threshold_for_fraction(s_ref.max(0), 0.35)
+        near = (np.abs(s_ref - thr) < 8e-6 * scale).any(0)
+        got = p.mask(x.to(DEV), "threshold", thr=thr).cpu().numpy()
+        assert np.array_equal(got[~near], oracle.mask_threshold(s_ref, thr, True)[~near]) and near.sum() <= 3
+        got_naive = p.mask(x.to(DEV), "naive").cpu().numpy()
+        safe = np.abs(s_ref).min(0) > 8e-6 * scale
+        assert np.array_equal(got_naive[safe], oracle.mask_threshold(s_ref, 0.0, True)[safe]) and safe.mean() > 0.999
