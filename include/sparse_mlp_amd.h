@@ -85,6 +85,23 @@ int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, c
                    int64_t ldc, void *workspace, int64_t workspace_bytes, int act, int dtype, int has_gate,
                    void *stream);
 
+/* The same forward for callers that cannot allocate or bring a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  Arguments as for
+ * st_mlp_forward without the workspace; only B <= 2 (the streaming decode
+ * kernel).  The fp32 partial rows go to a scratch array that is part of the
+ * library image (st_mlp_static_scratch_bytes() = 8 MiB per GPU, resident until
+ * the process ends); a call needs blocks * B * H * 4 bytes of it (one block per
+ * CU) and is refused with ST_ERR_ARG beyond that.  Every element the reduction
+ * reads is written by the same call first, so nothing has to be cleared between
+ * calls.  All calls on one GPU share the array: calls that overlap in time on
+ * the same GPU (two streams, two threads) race.  No hipMalloc / hipFree or
+ * other allocating call is made. */
+int64_t st_mlp_static_scratch_bytes(void);
+int st_mlp_forward_static(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
+                          const void *down_rows, int64_t n, const int32_t *n_dev, int64_t n_hint, void *out,
+                          void *combined, int64_t ldc, int act, int dtype, int has_gate, void *stream);
+
 /* ------------------------------------------------------------------------
  * LoRA predictor -> threshold mask -> union over rows, on the device.
  * Replaces FastLoRAProjection.forward (src/modeling_skip.py:52-53) and the

@@ -21,8 +21,16 @@
 #include "st_common.h"
 
 #include <cstdlib>
+#include <mutex>
 
 namespace st {
+
+// Scratch of the entry point that allocates nothing (st_mlp_forward_static): the fp32 partial rows
+// [blocks][rows of x][H] of the streaming decode kernel.  One copy per GPU the library runs on, held until
+// the process ends.  In host code this name is only a handle for hipGetSymbolAddress; kernels get the
+// address that call returns.
+constexpr size_t kStaticScratchBytes = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 template <int RB, int CPT> struct RowBatch {
     uint4 g[RB][CPT], u[RB][CPT], d[RB][CPT];
@@ -503,6 +511,49 @@ static int mlp_forward_decode(const void *x, int64_t B, int64_t H, const void *g
 }
 
 }  // namespace st
+
+// Device address of `scratch` on the current device, resolved once per device.
+static int static_scratch_ptr(void **out)
+{
+    static std::mutex mu;
+    static void *ptrs[64] = {nullptr};
+    int dev = 0;
+    ST_HIP(hipGetDevice(&dev));
+    ST_REQUIRE(dev >= 0 && dev < 64, "st_mlp_forward_static: device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void *p = nullptr;
+        ST_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(st::scratch)));   // the copy of the array on the current device
+        ST_REQUIRE(p != nullptr, "st_mlp_forward_static: hipGetSymbolAddress returned a null address");
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return ST_OK;
+}
+
+extern "C" int64_t st_mlp_static_scratch_bytes(void) { return (int64_t)st::kStaticScratchBytes; }
+
+extern "C" int st_mlp_forward_static(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
+                                     const void *down_rows, int64_t n, const int32_t *n_dev, int64_t n_hint,
+                                     void *out, void *combined, int64_t ldc, int act, int dtype, int has_gate,
+                                     void *stream)
+{
+    using namespace st;
+    ST_REQUIRE(B >= 1 && B <= 2, "st_mlp_forward_static: B=%lld outside [1,2] (use st_mlp_forward with a workspace)",
+               (long long)B);
+    ST_REQUIRE(H >= 1, "st_mlp_forward_static: H=%lld", (long long)H);
+    // what the streaming kernel writes: one fp32 row per block and row of x
+    const int64_t need = (int64_t)mlp_grid() * B * H * 4;
+    ST_REQUIRE(need <= (int64_t)kStaticScratchBytes,
+               "st_mlp_forward_static: %lld blocks x %lld rows x H=%lld needs %lld bytes of scratch, the static buffer "
+               "holds %lld", (long long)mlp_grid(), (long long)B, (long long)H, (long long)need,
+               (long long)kStaticScratchBytes);
+    void *ws = nullptr;
+    const int rc = static_scratch_ptr(&ws);
+    if (rc != ST_OK) return rc;
+    return mlp_forward_decode(x, B, H, gate_rows, up_rows, down_rows, n, n_dev, n_hint, out, combined, ldc, ws,
+                              (int64_t)kStaticScratchBytes, act, dtype, has_gate, stream, "st_mlp_forward_static");
+}
 
 extern "C" int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n)
 {
