@@ -6,7 +6,7 @@ Unlike the reference's ``sparse_transformers/__init__.py`` nothing global is cha
 fallback: without the built library, or without a GPU tensor, calls raise.
 """
 from .ops import approx_topk_threshold, mask_select, predictor_mask, predictor_scores, sparse_mlp_forward
-from .skip_mlp import FastLoRAProjection, SkipMLP, SparseDecodeLayer, SparseMLPStack, load_predictors
+from .skip_mlp import FastLoRAProjection, OPTSkipMLP, SkipMLP, SparseDecodeLayer, SparseMLPStack, load_predictors
 from .weight_cache import WeightCache
 
 __all__ = [
@@ -18,6 +18,7 @@ __all__ = [
     "approx_topk_threshold",
     "FastLoRAProjection",
     "SkipMLP",
+    "OPTSkipMLP",
     "SparseDecodeLayer",
     "SparseMLPStack",
     "load_predictors",

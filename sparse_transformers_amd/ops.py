@@ -163,6 +163,10 @@ def sparse_mlp_forward(x: torch.Tensor, concat_weight: torch.Tensor, active_down
     "relu" reproduces that operator, "silu" reproduces src/modeling_skip.py:114-117.
     """
     global _warned_layout
+    from .weight_cache import ConcatWeightHandle
+    handle = concat_weight if isinstance(concat_weight, ConcatWeightHandle) and concat_weight._real is None else None
+    if isinstance(concat_weight, ConcatWeightHandle) and handle is None:
+        concat_weight = concat_weight.materialize()
     dev = require_gpu(x, concat_weight, active_down_weight, down_proj_buffer, combined_proj_buffer)
     H = x.shape[-1]
     rows = concat_weight.size(0)
@@ -180,8 +184,6 @@ def sparse_mlp_forward(x: torch.Tensor, concat_weight: torch.Tensor, active_down
     x2 = x.reshape(-1, H)
     if not x2.is_contiguous():
         x2 = x2.contiguous()
-    if not concat_weight.is_contiguous():
-        concat_weight = concat_weight.contiguous()
     B = x2.size(0)
     # [H, n] with strides (1, H) is a packed [n, H] buffer underneath
     if n > 0 and active_down_weight.stride() == (1, H):
@@ -196,8 +198,20 @@ def sparse_mlp_forward(x: torch.Tensor, concat_weight: torch.Tensor, active_down
         down_proj_buffer.resize_(B, H)
     if combined_proj_buffer.dim() != 2 or combined_proj_buffer.size(0) != B or combined_proj_buffer.size(1) != rows:
         combined_proj_buffer.resize_(B, rows)
-    gate_rows = concat_weight[:n] if has_gate else None
-    up_rows = concat_weight[n:] if has_gate else concat_weight
+    if handle is not None:
+        # the cache's own handle: its packed gate / up rows are read in place (no [2n,H] copy)
+        cache = handle._cache
+        if has_gate != cache.has_gate:
+            raise ValueError("has_gate does not match the cache the concat weight comes from")
+        if not handle.fresh():
+            raise RuntimeError("concat_weight was fetched before the cache's last update; call get_concat_weight() again")
+        gate_rows = cache.gate_active if has_gate else None
+        up_rows = cache.up_active
+    else:
+        if not concat_weight.is_contiguous():
+            concat_weight = concat_weight.contiguous()
+        gate_rows = concat_weight[:n] if has_gate else None
+        up_rows = concat_weight[n:] if has_gate else concat_weight
     mlp_forward_rows(x2, gate_rows, up_rows, down_rows, n, None, down_proj_buffer, combined_proj_buffer, act,
                      has_gate)
     return down_proj_buffer.view(x.shape) if x.dim() != 2 else down_proj_buffer

@@ -1,12 +1,13 @@
 """Host-side mirror of the reference's callers of the sparse-MLP path.
 
   * ``FastLoRAProjection`` — src/modeling_skip.py:32-53 (the importance predictor's two bias-free maps)
-  * ``SkipMLP``            — src/modeling_skip.py:55-128 (buffers, ``initialize_weight_cache``, sparse forward)
+  * ``SkipMLP`` / ``OPTSkipMLP`` — src/modeling_skip.py:55-128, src/models/opt/modelling_opt_skip.py:60-119
+    (``nn.Module`` with the reference's sub-modules and buffers, ``initialize_weight_cache``, ``reset_cache``)
   * ``SparseDecodeLayer`` / ``SparseMLPStack`` — the per-layer order of SkipDecoderLayer.forward
     (src/modeling_skip.py:204-219,234-261): predictor -> mask -> union -> cache update -> sparse MLP,
     without attention or normalisation, which are outside this path.
 
-No HuggingFace dependency; parameters are plain tensors on the GPU.
+No HuggingFace dependency.
 """
 from __future__ import annotations
 
@@ -87,43 +88,124 @@ def load_predictors(directory: str, num_layers: int, lora_pct: float, device=Non
                                          device=device, dtype=dtype) for l in range(num_layers)]
 
 
-class SkipMLP:
-    """Gated (or ungated) MLP whose decode path runs on the differential weight cache."""
+_TORCH_ACTS = {
+    "relu": torch.relu,
+    "silu": torch.nn.functional.silu,
+    "gelu_pytorch_tanh": lambda v: torch.nn.functional.gelu(v, approximate="tanh"),
+    "sigmoid": torch.sigmoid,
+    "identity": lambda v: v,
+}
 
-    def __init__(self, gate_weight: Optional[torch.Tensor], up_weight: torch.Tensor, down_weight: torch.Tensor,
-                 sparsity: float = 0.5, act_fn: str = "silu", has_gate: bool = True):
-        self.gate_weight, self.up_weight, self.down_weight = gate_weight, up_weight, down_weight
-        self.intermediate_size, self.hidden_size = up_weight.shape
+
+class SkipMLP(torch.nn.Module):
+    """Drop-in for the reference's ``SkipMLP`` (src/modeling_skip.py:55-128) and, with ``has_gate=False``, for
+    ``OPTSkipMLP`` (src/models/opt/modelling_opt_skip.py:60-119): same constructor arguments, the same
+    sub-modules ``gate_proj`` / ``up_proj`` / ``down_proj`` (bias-free by default) and registered buffers
+    ``init_mask``, ``down_proj_buffer``, ``combined_proj_buffer`` -- so a checkpoint of the reference loads
+    with ``load_state_dict`` -- and the same methods.
+
+    ``forward(x, use_sparse=True)`` runs the HIP decode kernels on the cache's packed rows
+    (``WeightCache.forward``: no host read-back, no ``[2n,H]`` copy).  The reference's own sparse forward
+    multiplies ``x`` with ``get_concat_weight()`` in torch (src/modeling_skip.py:114-117) and therefore never
+    reaches ``sparse_mlp_forward``; replacing the module is what puts the kernels on the path.
+    ``use_sparse=False`` is the dense MLP in torch, which is what the reference runs for prefill.
+    Like the reference's cache path, the sparse forward ignores biases."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, sparsity: float, bias: bool = False,
+                 act_fn: str = "silu", use_weight_cache: bool = True, has_gate: bool = True):
+        super().__init__()
+        if act_fn not in _TORCH_ACTS:
+            raise ValueError(f"unknown activation {act_fn!r}; expected one of {sorted(_TORCH_ACTS)}")
+        self.has_gate = bool(has_gate)
+        if self.has_gate:
+            self.gate_proj = torch.nn.Linear(hidden_size, intermediate_size, bias=bias)
+        self.up_proj = torch.nn.Linear(hidden_size, intermediate_size, bias=bias)
+        self.down_proj = torch.nn.Linear(intermediate_size, hidden_size, bias=bias)
         self.sparsity = sparsity
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.act_fn_name = act_fn
-        self.has_gate = has_gate
-        dev, dt = up_weight.device, up_weight.dtype
-        self.init_mask = torch.ones(self.intermediate_size, dtype=torch.bool, device=dev)
+        self.act_fn = _TORCH_ACTS[act_fn]
+        self.use_weight_cache = use_weight_cache
+        self.weight_mask: Optional[torch.Tensor] = None      # only used by the cache-less debugging forward
         self.weight_cache: Optional[WeightCache] = None
-        cols = (2 if has_gate else 1) * int(self.intermediate_size * sparsity)
-        self.down_proj_buffer = torch.zeros(1, self.hidden_size, dtype=dt, device=dev)
-        self.combined_proj_buffer = torch.zeros(1, max(cols, 1), dtype=dt, device=dev)
+        self.register_buffer("init_mask", torch.ones(self.intermediate_size, dtype=torch.bool))
+        cols = (2 if self.has_gate else 1) * int(self.intermediate_size * sparsity)
+        self.register_buffer("down_proj_buffer", torch.zeros(1, self.hidden_size))
+        self.register_buffer("combined_proj_buffer", torch.zeros(1, max(cols, 1)))
+
+    @classmethod
+    def from_weights(cls, gate_weight: Optional[torch.Tensor], up_weight: torch.Tensor, down_weight: torch.Tensor,
+                     sparsity: float = 0.5, act_fn: str = "silu", has_gate: bool = True) -> "SkipMLP":
+        """The module around existing weight tensors (gate/up [I,H], down [H,I]); device and dtype follow them."""
+        I, H = up_weight.shape
+        with torch.device("meta"):
+            m = cls(H, I, sparsity, False, act_fn, True, has_gate)
+        m = m.to_empty(device=up_weight.device).to(up_weight.dtype)
+        with torch.no_grad():
+            if has_gate:
+                m.gate_proj.weight.copy_(gate_weight)
+            m.up_proj.weight.copy_(up_weight)
+            m.down_proj.weight.copy_(down_weight)
+            m.init_mask.fill_(True)
+            m.down_proj_buffer.zero_()
+            m.combined_proj_buffer.zero_()
+        return m
 
     def initialize_weight_cache(self) -> None:
-        if self.weight_cache is None:
-            self.weight_cache = WeightCache(self.init_mask, self.hidden_size, self.gate_weight, self.up_weight,
-                                            self.down_weight, self.has_gate)
+        """Builds the cache from the current weights (they are copied), all rows active: called once the weights
+        are loaded and the module sits on its GPU, as the reference does from ``post_init``."""
+        if self.weight_cache is None and self.use_weight_cache:
+            self.weight_cache = WeightCache(self.init_mask, self.hidden_size,
+                                            self.gate_proj.weight if self.has_gate else None, self.up_proj.weight,
+                                            self.down_proj.weight, self.has_gate)
 
     def reset_cache(self) -> None:
-        """Back to the all-ones mask of a fresh cache (every row active, order 0..I-1)."""
+        """What the reference's model-level ``reset_cache`` does per layer (src/modeling_skip.py:492-497): drop
+        the cache and build a fresh one (every row active, order 0..I-1)."""
         self.weight_cache = None
         self.initialize_weight_cache()
 
+    def _apply(self, fn, *args, **kwargs):
+        # .to() / .half() / .cuda(): parameters and the registered buffers move with the module; a cache built
+        # on the old device or dtype no longer matches them and has to be rebuilt
+        out = super()._apply(fn, *args, **kwargs)
+        wc = self.weight_cache
+        if wc is not None and (wc.device != self.up_proj.weight.device or wc.dtype != self.up_proj.weight.dtype):
+            self.weight_cache = None
+        return out
+
     def forward(self, x: torch.Tensor, use_sparse: bool = True) -> torch.Tensor:
         if not use_sparse:
-            raise NotImplementedError("the dense (prefill) MLP is outside this package's path")
+            return self._forward_dense(x)
+        if self.use_weight_cache:
+            return self._forward_sparse_weight_cache(x)
+        return self._forward_sparse_no_cache(x)
+
+    def _forward_sparse_weight_cache(self, x: torch.Tensor) -> torch.Tensor:
         wc = self.weight_cache
         if wc is None:
             raise RuntimeError("call initialize_weight_cache() first")
-        return sparse_mlp_forward(x, wc.get_concat_weight(), wc.get_active_down_weight(), self.down_proj_buffer,
-                                  self.combined_proj_buffer, self.act_fn_name, self.has_gate)
+        return wc.forward(x, self.act_fn_name)
 
-    __call__ = forward
+    def _forward_sparse_no_cache(self, x: torch.Tensor) -> torch.Tensor:
+        up = self.up_proj(x)
+        h = self.act_fn(self.gate_proj(x)) * up if self.has_gate else self.act_fn(up)
+        if self.weight_mask is not None:
+            h = h * self.weight_mask
+        return self.down_proj(h)
+
+    def _forward_dense(self, x: torch.Tensor) -> torch.Tensor:
+        up = self.up_proj(x)
+        return self.down_proj(self.act_fn(self.gate_proj(x)) * up if self.has_gate else self.act_fn(up))
+
+
+class OPTSkipMLP(SkipMLP):
+    """The ungated variant (src/models/opt/modelling_opt_skip.py:60-119): ``up_proj`` / ``down_proj`` only,
+    ReLU by default."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, sparsity: float, bias: bool = False,
+                 act_fn: str = "relu", use_weight_cache: bool = True):
+        super().__init__(hidden_size, intermediate_size, sparsity, bias, act_fn, use_weight_cache, has_gate=False)
 
 
 class SparseDecodeLayer:

@@ -17,6 +17,53 @@ from .ops import (_check_workspace, check_mlp_args, current_stream_ptr, dtype_co
                   mlp_workspace_bytes, require_gpu)
 
 
+class ConcatWeightHandle(torch.Tensor):
+    """What ``WeightCache.get_concat_weight()`` returns: a tensor of shape ``[2n,H]`` (``[n,H]`` ungated) that
+    owns no memory until something reads it.  ``sparse_mlp_forward`` recognises it and reads the cache's packed
+    gate / up rows in place, so the reference's call sequence costs no ``[2n,H]`` copy (the reference pays a
+    ``torch::cat`` per update, weight_cache.h:138).  Any other torch operation on it (``.t()``, ``matmul``,
+    indexing, ``.cpu()`` ...) first materialises the contiguous tensor with one device copy and then runs on
+    that.  Like the reference's tensor it describes the cache as of the update it was fetched after; using it
+    after a later update raises instead of silently showing newer rows under the old shape."""
+
+    @staticmethod
+    def __new__(cls, cache: "WeightCache", n: int, serial: int):
+        rows = (2 if cache.has_gate else 1) * n
+        t = torch.Tensor._make_wrapper_subclass(cls, (rows, cache.hidden_size), dtype=cache.dtype,
+                                                device=cache.device, requires_grad=False)
+        t._cache, t._n, t._serial, t._real = cache, n, serial, None
+        return t
+
+    def fresh(self) -> bool:
+        """True while no update has changed the cache since this handle was fetched."""
+        c = self._cache
+        return not c._dirty and c._host_state[_lib.STATE_SERIAL] == self._serial
+
+    def materialize(self) -> torch.Tensor:
+        if self._real is None:
+            c = self._cache
+            if not self.fresh():
+                raise RuntimeError("this concat weight was fetched before the cache's last update; "
+                                   "call get_concat_weight() again")
+            buf = torch.empty(self.shape[0], c.hidden_size, dtype=c.dtype, device=c.device)
+            if self._n > 0:
+                rc = _lib.lib().st_cache_materialize_concat(c._h, buf.data_ptr(), self._n, current_stream_ptr(c.device))
+                _lib.check(rc, "st_cache_materialize_concat")
+            self._real = buf
+        return self._real
+
+    def __repr__(self):
+        return f"ConcatWeightHandle(shape={tuple(self.shape)}, dtype={self.dtype}, materialized={self._real is not None})"
+
+    @classmethod
+    def __torch_dispatch__(cls, func, types, args=(), kwargs=None):
+        from torch.utils._pytree import tree_map
+
+        def real(t):
+            return t.materialize() if isinstance(t, cls) else t
+        return func(*tree_map(real, args), **tree_map(real, kwargs or {}))
+
+
 class WeightCache:
     """Drop-in for the reference WeightCache, plus a zero-copy fast path.
 
@@ -141,16 +188,11 @@ class WeightCache:
         return st
 
     def get_concat_weight(self) -> torch.Tensor:
-        """Contiguous [2n,H] (gate rows then up rows; [n,H] when ungated), valid until the next update."""
+        """``[2n,H]`` (gate rows then up rows; ``[n,H]`` when ungated), valid until the next update.  Returned
+        as a ``ConcatWeightHandle``: no copy is made unless something other than ``sparse_mlp_forward`` reads it."""
         st = self._require_valid()
-        n = int(st["n_active"])
         if self._concat is None or self._concat_serial != st["serial"]:
-            rows = (2 if self.has_gate else 1) * n
-            buf = torch.empty(rows, self.hidden_size, dtype=self.dtype, device=self.device)
-            if n > 0:
-                rc = _lib.lib().st_cache_materialize_concat(self._h, buf.data_ptr(), n, current_stream_ptr(self.device))
-                _lib.check(rc, "st_cache_materialize_concat")
-            self._concat, self._concat_serial = buf, st["serial"]
+            self._concat, self._concat_serial = ConcatWeightHandle(self, int(st["n_active"]), st["serial"]), st["serial"]
         return self._concat
 
     def get_active_down_weight(self) -> torch.Tensor:

@@ -98,26 +98,128 @@ def test_graph_replay_equals_eager(overlap):
 
 
 def test_skip_mlp_module_surface():
-    """SkipMLP mirrors the reference module: buffers, initialize_weight_cache, sparse forward."""
+    """SkipMLP mirrors the reference module (src/modeling_skip.py:55-128): constructor arguments, sub-modules,
+    registered buffers, state-dict keys, initialize_weight_cache / reset_cache, the three forwards."""
     H, I = 128, 320
     g = torch.Generator().manual_seed(0)
+    mlp = st.SkipMLP(H, I, 0.5, bias=False, act_fn="silu", use_weight_cache=True)
+    assert isinstance(mlp, torch.nn.Module)
+    assert sorted(mlp.state_dict()) == sorted(["gate_proj.weight", "up_proj.weight", "down_proj.weight", "init_mask",
+                                               "down_proj_buffer", "combined_proj_buffer"])
+    assert tuple(mlp.down_proj_buffer.shape) == (1, H) and tuple(mlp.combined_proj_buffer.shape) == (1, 2 * 160)
+    assert mlp.init_mask.dtype == torch.bool and bool(mlp.init_mask.all())
     gate, up, down = (torch.randn(I, H, generator=g) * 0.05), (torch.randn(I, H, generator=g) * 0.05), \
         (torch.randn(H, I, generator=g) * 0.05)
-    mlp = st.SkipMLP(gate.to(DEV), up.to(DEV), down.to(DEV), sparsity=0.5, act_fn="silu")
-    assert tuple(mlp.down_proj_buffer.shape) == (1, H) and tuple(mlp.combined_proj_buffer.shape) == (1, 2 * 160)
+    mlp.load_state_dict({"gate_proj.weight": gate, "up_proj.weight": up, "down_proj.weight": down}, strict=False)
+    mlp = mlp.to(DEV)
+    assert mlp.init_mask.is_cuda and mlp.down_proj_buffer.is_cuda and mlp.combined_proj_buffer.is_cuda
     with pytest.raises(RuntimeError):
         mlp(torch.randn(1, 1, H, device=DEV))
     mlp.initialize_weight_cache()
+    wc0 = mlp.weight_cache
+    mlp.initialize_weight_cache()
+    assert mlp.weight_cache is wc0                        # only built once
     m = torch.rand(I, generator=g) < 0.5
     mlp.weight_cache.update_active_weights(m.to(DEV))
     x = torch.randn(2, 1, H, generator=g)
     out = mlp(x.to(DEV))
+    assert out.shape == x.shape
     idx = torch.nonzero(m).flatten()
     oc = oracle.OracleWeightCache(np.ones(I, bool), H, gate.numpy(), up.numpy(), down.numpy(), True)
     oc.update_active_weights(m.numpy())
     want, _ = oracle.mlp_forward(x.numpy(), oc.get_concat_weight(), oc.get_active_down_weight(), "silu", True)
     assert_close(out.cpu().numpy(), want, "float32", "SkipMLP")
     assert sorted(mlp.weight_cache.get_active_indices().cpu().tolist()) == idx.tolist()
+    # dense forward (the reference's prefill path) = the full MLP in torch
+    dense = mlp(x.to(DEV), use_sparse=False).detach().cpu()
+    ref = (torch.nn.functional.silu(x @ gate.t()) * (x @ up.t())) @ down.t()
+    assert torch.allclose(dense, ref, rtol=1e-4, atol=1e-5)
+    # reset_cache: back to every row active in order 0..I-1 (src/modeling_skip.py:492-497)
+    mlp.reset_cache()
+    assert mlp.weight_cache is not wc0
+    assert mlp.weight_cache.get_active_indices().cpu().tolist() == list(range(I))
+    # a move to another dtype invalidates the cache (its rows would no longer match the parameters)
+    mlp = mlp.half()
+    assert mlp.weight_cache is None and mlp.down_proj_buffer.dtype == torch.float16
+    mlp.initialize_weight_cache()
+    assert mlp.weight_cache.dtype == torch.float16
+    # the cache-less debugging forward with a weight mask
+    dbg = st.SkipMLP.from_weights(gate.to(DEV), up.to(DEV), down.to(DEV), 0.5, "silu")
+    dbg.use_weight_cache = False
+    dbg.weight_mask = m.to(DEV).float()
+    assert_close(dbg(x.to(DEV)).detach().cpu().numpy(), want, "float32", "masked dense forward")
+
+
+@pytest.mark.parametrize("variant", ["llama3b_gated_fp16", "opt_ungated_fp16"])
+def test_skip_mlp_full_shape_vs_oracle(variant):
+    """The module at a benchmark shape (H = 3072, I = 8192, 35 % active, fp16), gated with SiLU and OPT-style
+    ungated with ReLU, decode with one row and with several: sparse forward against the oracle."""
+    H, I, dtype = 3072, 8192, "float16"
+    gated = variant.startswith("llama")
+    rng = np.random.default_rng(12)
+    w = syn.layer_weights(rng, H, I, 8, std=0.02, has_gate=gated)
+    w = {k: (None if v is None else round_to(v, dtype)) for k, v in w.items()}
+    if gated:
+        mlp = st.SkipMLP(H, I, 0.65, act_fn="silu")
+        mlp.gate_proj.weight.data = torch.from_numpy(w["gate"])
+    else:
+        mlp = st.OPTSkipMLP(H, I, 0.65)
+        assert not hasattr(mlp, "gate_proj") and mlp.act_fn_name == "relu"
+    mlp.up_proj.weight.data = torch.from_numpy(w["up"])
+    mlp.down_proj.weight.data = torch.from_numpy(w["down"])
+    mlp = mlp.to(DEV).half()
+    mlp.initialize_weight_cache()
+    oc = oracle.OracleWeightCache(np.ones(I, bool), H, w["gate"], w["up"], w["down"], gated)
+    act = "silu" if gated else "relu"
+    for step, B in enumerate((1, 1, 4, 1)):
+        m = syn.initial_mask(rng, I, int(0.35 * I))
+        mlp.weight_cache.update_active_weights(torch.from_numpy(m).to(DEV))
+        oc.update_active_weights(m)
+        x = round_to(rng.standard_normal((B, 1, H)).astype(np.float32), dtype)
+        got = mlp(torch.from_numpy(x).to(DEV, torch.float16))
+        want, _ = oracle.mlp_forward(x, oc.get_concat_weight(), oc.get_active_down_weight(), act, gated)
+        assert_close(got.float().cpu().numpy(), want, dtype, f"{variant} step {step}")
+        assert mlp.weight_cache.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist()
+
+
+def test_reference_call_sequence_reads_the_cache_in_place():
+    """update_active_weights -> get_concat_weight -> get_active_down_weight -> sparse_mlp_forward, as a caller of
+    the reference's operator writes it: the concat weight is a handle that sparse_mlp_forward resolves to the
+    cache's packed rows (no [2n,H] copy); anything else that touches it gets the real contiguous tensor; a handle
+    kept across a later update is refused."""
+    H, I = 256, 512
+    g = torch.Generator().manual_seed(2)
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.05).half().to(DEV)
+    gate, up, down = mk(I, H), mk(I, H), mk(H, I)
+    wc = st.WeightCache(torch.ones(I, dtype=torch.bool, device=DEV), H, gate, up, down, True)
+    m = (torch.rand(I, generator=g) < 0.4).to(DEV)
+    wc.update_active_weights(m)
+    n = int(m.sum())
+    cw, dw = wc.get_concat_weight(), wc.get_active_down_weight()
+    assert tuple(cw.shape) == (2 * n, H) and cw.dtype == torch.float16 and cw.is_cuda and cw.is_contiguous()
+    assert cw._real is None and wc.get_concat_weight() is cw
+    x = mk(3, H)
+    db, cb = torch.zeros(1, H, dtype=torch.float16, device=DEV), torch.zeros(1, 2, dtype=torch.float16, device=DEV)
+    y = st.sparse_mlp_forward(x, cw, dw, db, cb, "silu").clone()
+    assert cw._real is None                                   # still no copy
+    order = wc.get_active_indices()
+    real = cw + 0                                             # any torch op materialises it
+    assert cw._real is not None and torch.equal(real, torch.cat([gate[order], up[order]]))
+    assert torch.equal(cw.t().contiguous(), real.t().contiguous()) and torch.equal(cw[:n], gate[order])
+    y2 = st.sparse_mlp_forward(x, cw, dw, db, cb, "silu")     # now through the materialised tensor: same bits
+    assert torch.equal(y, y2)
+    wc.update_active_weights(~m)
+    stale = cw
+    fresh = wc.get_concat_weight()
+    assert fresh is not stale and tuple(fresh.shape) == (2 * (I - n), H)
+    with pytest.raises(RuntimeError):
+        st.sparse_mlp_forward(x, ConcatStale(stale, wc, n), dw, db, cb, "silu")
+
+
+def ConcatStale(stale, wc, n):
+    """A handle fetched before the last update that has never been read."""
+    from sparse_transformers_amd.weight_cache import ConcatWeightHandle
+    return ConcatWeightHandle(wc, n, stale._serial)
 
 
 @pytest.mark.parametrize("method,B", [("topk", 1), ("topk", 3), ("statistical_topk", 1), ("statistical_topk", 2)])
