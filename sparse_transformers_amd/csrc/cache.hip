@@ -25,6 +25,7 @@
 
 #include <cstdlib>
 #include <new>
+#include <type_traits>
 
 namespace st {
 
@@ -51,6 +52,24 @@ __device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v, int lane)
         if (lane >= off) v += o;
     }
     return v;
+}
+
+// The same with DPP row shifts (no LDS crossbar traffic): four steps scan each row of 16 lanes, the row totals
+// travel through scalar registers.
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_shr_add(uint32_t v)
+{
+    return v + (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);   // lanes shifted in from outside the row read 0
+}
+__device__ __forceinline__ uint32_t wave_incl_scan_dpp(uint32_t v, int lane)
+{
+    v = dpp_shr_add<0x111>(v);   // row_shr:1
+    v = dpp_shr_add<0x112>(v);   // row_shr:2
+    v = dpp_shr_add<0x114>(v);   // row_shr:4
+    v = dpp_shr_add<0x118>(v);   // row_shr:8
+    const uint32_t t0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 15), t1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 31),
+                   t2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 47);
+    const int row = lane >> 4;
+    return v + (row >= 1 ? t0 : 0u) + (row >= 2 ? t1 : 0u) + (row >= 3 ? t2 : 0u);
 }
 
 // Exclusive scan of one uint32 per thread over WAVES waves; *total receives the sum.  `sync` is the
@@ -780,6 +799,446 @@ __global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
     ST_TL(7);
 }
 
+// ---------------------------------------------------------------------------
+// update + sparse MLP in ONE kernel, with the plan worked out per POSITION
+// instead of per index.
+//
+// A block only has to know, for each of the <= ceil(I / G) positions it owns,
+// which row to read: position p held index e before the update; if e left the
+// mask it is the i-th removed index (i = its rank among the removed, ascending)
+// and the position receives the i-th added index (weight_cache.h:248-277);
+// positions n_old .. n_new-1 receive the surplus additions in ascending order
+// (:280-307).  Ranks come from bitmaps of the two masks and per-word prefix
+// counts (one wave, no block-wide scans), the i-th added index from a binary
+// search over those counts -- no index -> position map, no lists, no atomics,
+// three LDS-only barriers, and straight-line code, so the rows a block requests
+// on the caller's guess right after its (few) bookkeeping loads stay in flight
+// through all of it.  Every block publishes its own positions of the new
+// ordered list and a slice of the remembered mask into the other bookkeeping
+// buffer; block 0 writes the state words; the last block to arrive flips the
+// epoch (as in cache_plan).
+// When removals outnumber additions (:310-353 is sequential) the block falls
+// back to cache_plan above, for that launch only.
+// ---------------------------------------------------------------------------
+constexpr int kSparseMaxQ = 64;       // positions a block can own
+constexpr int kSparseMaxW32 = 512;    // mask words: I <= 16384
+constexpr int kSparseWords = 2;       // 8-byte mask words per thread, at most
+constexpr int kSrcPool = 0x40000000;  // src[]: bit 30 = read the pool row (low bits) and write it back; else active row
+
+struct SparseShared {
+    uint32_t newbits[kSparseMaxW32], oldbits[kSparseMaxW32];
+    uint16_t pr[kSparseMaxW32];   // removed indices below each word
+    int na, nr, n;
+    int src[kSparseMaxQ];
+};
+
+// 0x01-per-element bytes -> 8 bits (element k -> bit k)
+__device__ __forceinline__ uint32_t pack_bits8(uint64_t ones)
+{
+    return (uint32_t)((ones * 0x0102040810204080ull) >> 56);
+}
+
+template <typename T, int RB, int TPB, int NB = 1, int NW = 1, int SPECN = RB / 2>
+__global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
+    FusedRows fr, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
+    int32_t *__restrict__ state, int I, const T *__restrict__ x, int B, int H, T *__restrict__ combined, long ldc,
+    float *__restrict__ partials, int act, int gs_log2, int plan_bytes, int n_hint)
+{
+    constexpr int VEC = Elem<T>::kVec;
+    // Slots of the first batch that are requested ahead of the plan, on the caller's guess of the count and from the
+    // active buffers.  A slot whose row turns out to have changed is requested again into the same registers, which
+    // has to wait until its first request has arrived; requests return in order, so for the last slots that wait
+    // would be the whole stream plus one more round trip, and every row requested in vain is traffic.  The later
+    // slots are therefore requested after the plan (first, so that they queue right behind the rows already
+    // requested).  Half the batch ahead of the plan measured best (against a third, two thirds and all of it).
+    constexpr int SPEC = SPECN;
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float red[TPB / kWave][RB][NB][2];  // per-wave partial (g,u)
+    __shared__ float hs[TPB / kWave][RB][NB];      // h of the rows being computed
+    __shared__ SparseShared sh;
+    __shared__ PlanShared plan_shared;
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int G = gridDim.x, blk = blockIdx.x;
+    const int chunks = H / VEC;
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+    const int GS = 1 << gs_log2, ngrp = TPB >> gs_log2, wpg = GS >> 6;
+    const int grp = tid >> gs_log2, cc = tid & (GS - 1);
+    const bool valid = cc < chunks;
+    const size_t coff = valid ? (size_t)cc * 16 : 0;
+    const bool wave_live = __builtin_amdgcn_readfirstlane(cc & ~(kWave - 1)) < chunks;
+    const bool has_gate = fr.has_gate != 0;
+    const int row_bytes = fr.row_bytes;
+    const unsigned char *const pool_g = fr.pool_g, *const pool_u = fr.pool_u, *const pool_d = fr.pool_d;
+    unsigned char *const act_g = fr.act_g, *const act_u = fr.act_u, *const act_d = fr.act_d;
+    const int Q = (I + G - 1) / G;        // positions of this block: blk + G * q, q < Q (host: Q <= kSparseMaxQ)
+    const int W32 = (I + 31) >> 5;
+
+    ST_TL(0);
+    // ---- bookkeeping loads: one round trip, all unconditional (clamped addresses).  The state words are read
+    // through a lane offset the compiler cannot see through (always zero): as loads from one address for the whole
+    // wave they would be moved to scalar registers at once, which means waiting for them before anything else
+    // is requested.
+    int lane_zero = 0;
+    asm volatile("" : "+v"(lane_zero));
+    const int32_t *state_v = state + lane_zero;
+    const uint32_t tword = __hip_atomic_load(reinterpret_cast<const uint32_t *>(&state_v[ST_STATE_TICKET]),
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int n_buf0 = state_v[ST_STATE_N_BUF0], n_buf1 = state_v[ST_STATE_N_BUF1];
+    const int serial_old = state_v[ST_STATE_SERIAL];
+    constexpr int nw_rt = NW;   // 8-byte mask words per thread (host: I <= 8 * TPB * NW)
+    uint64_t v_new[NW], v_c0[NW], v_c1[NW];
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        const int e = (tid * nw_rt + w) * 8;
+        const int ec = e + 8 <= I ? e : I - 8;
+        v_new[w] = *reinterpret_cast<const uint64_t *>(new_mask + ec);
+        v_c0[w] = *reinterpret_cast<const uint64_t *>(cur_mask2 + ec);
+        v_c1[w] = *reinterpret_cast<const uint64_t *>(cur_mask2 + (size_t)I + ec);
+    }
+    // The plan is worked out by ONE wave, the last of the block (with 6 KB rows a wave that owns no columns), while
+    // the others already request rows; its lanes own the block's positions.
+    constexpr int PW = TPB / kWave - 1;
+    const bool plan_wave = wave == PW;
+    static_assert(kSparseMaxQ == kWave, "one lane of the planning wave per position of the block");
+    const int my_p = blk + G * lane;
+    const int my_pc = my_p < I ? my_p : I - 1;
+    const int i_old0 = indices2[my_pc], i_old1 = indices2[(size_t)I + my_pc];
+    uint4 xr[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+        xr[b] = ld16(reinterpret_cast<const unsigned char *>(x) + (size_t)(b < B ? b : 0) * row_bytes + coff);
+
+    // ---- the first batch of rows, on the caller's guess of the count, from the active buffers
+    auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
+    const int n_spec = n_hint < I ? n_hint : I;
+    uint4 wg[RB], wu[RB], wd[RB];
+    // (every wave issues the same number of loads whatever its role: a wave without columns, and the gate loads
+    // of an ungated cache, read one line of x instead -- with branches around the loads the compiler could no
+    // longer tell how many requests are younger than the bookkeeping loads and would wait for all of them)
+    // Addresses are a uniform base (scalar registers) plus a 32-bit lane offset, one offset per row for its three
+    // matrices: with a 64-bit address per load the 18 requests alone would need 36 registers more.
+    const uint32_t coff32 = (uint32_t)coff;
+    const unsigned char *const dummy = reinterpret_cast<const unsigned char *>(x);
+    const unsigned char *const sp_u = wave_live ? act_u : dummy, *const sp_d = wave_live ? act_d : dummy,
+                        *const sp_g = wave_live && has_gate ? act_g : dummy;
+    auto speculate = [&](auto lo_c, auto hi_c) __attribute__((always_inline)) {
+        constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
+#pragma unroll
+        for (int k = LO; k < HI; ++k) {
+            const int p = row_of(0, k);
+            // (a slot past the expected count reads one 16-byte piece for the whole wave: a single request instead of
+            // a row's worth of traffic that nobody needs)
+            const uint32_t off = wave_live && p < n_spec ? (uint32_t)p * (uint32_t)row_bytes + coff32 : 0u;
+            wu[k] = ld16_stream(sp_u + off);
+            wd[k] = ld16_stream(sp_d + off);
+            wg[k] = ld16_stream(sp_g + (has_gate ? off : 0u));   // (the stand-in line of x has no rows to index)
+        }
+    };
+    // Half of the rows that are requested ahead of the plan go out right behind the bookkeeping loads -- few enough
+    // that the memory system is not yet saturated when those loads are served -- the other half once they have
+    // arrived.  The barrier only orders the issue: every wave's bookkeeping loads are queued before any wave's rows.
+    constexpr int SPEC_A = SPEC / 2;
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    speculate(std::integral_constant<int, 0>{}, std::integral_constant<int, SPEC_A>{});
+    __builtin_amdgcn_sched_barrier(0);
+    ST_TL(1);
+
+    // ---- masks -> bitmaps in LDS
+    const int ep = (int)((tword >> 16) & 1u);
+    const int n_old = ep ? n_buf1 : n_buf0;
+    uint64_t w_new[NW], w_cur[NW];
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        const int bi = tid * nw_rt + w;            // byte of the bitmaps = elements [8 bi, 8 bi + 8)
+        const bool in = w < nw_rt && bi * 8 < I;
+        w_new[w] = in ? nonzero_bytes(v_new[w]) : 0ull;
+        w_cur[w] = in ? nonzero_bytes(ep ? v_c1[w] : v_c0[w]) : 0ull;
+        if (w < nw_rt && bi < W32 * 4) {
+            reinterpret_cast<uint8_t *>(sh.newbits)[bi] = (uint8_t)pack_bits8(w_new[w]);
+            reinterpret_cast<uint8_t *>(sh.oldbits)[bi] = (uint8_t)pack_bits8(w_cur[w]);
+        }
+    }
+    lds_barrier();
+    // ---- Rows are requested from here on, i.e. once every wave's bookkeeping loads have ARRIVED: loads issued into
+    // a memory system that is already saturated with row requests take several times longer to come back (measured:
+    // 5.7 us instead of under 2 when the rows were requested right behind them), and the plan hangs on them.  From
+    // here on the plan needs LDS only.  It is one wave's work, so that it does not wait for the other waves either:
+    // a wave's requests are accepted only as fast as the memory system takes them (the last wave of sixteen gets its
+    // first batch out 3 us after the first), and a block barrier inside the plan would wait for all of that.
+    ST_TL(2);
+    int n = n_old;      // count after the update
+    uint32_t arrival = 0;
+    __builtin_amdgcn_sched_barrier(0);
+    if (plan_wave) {
+        // ---- per-word prefix counts of added / removed indices, eight words per lane at most
+        const int wpl = (W32 + kWave - 1) >> 6;
+        uint32_t la[kSparseMaxW32 / kWave], lr[kSparseMaxW32 / kWave];
+        uint32_t ca = 0, cr = 0;
+#pragma unroll
+        for (int j = 0; j < kSparseMaxW32 / kWave; ++j) {
+            const int t = lane * wpl + j;
+            const bool in = j < wpl && t < W32;
+            const uint32_t nwd = in ? sh.newbits[t] : 0u, owd = in ? sh.oldbits[t] : 0u;
+            la[j] = ca; lr[j] = cr;
+            ca += (uint32_t)__popc(nwd & ~owd);
+            cr += (uint32_t)__popc(owd & ~nwd);
+        }
+        const uint32_t packed = ca | (cr << 16);
+        const uint32_t incl = wave_incl_scan_dpp(packed, lane);
+        const uint32_t excl = incl - packed;
+        // removed: per-word prefix counts (a position looks its old index's rank up); added: the ascending list itself
+        uint16_t *added_list = reinterpret_cast<uint16_t *>(smem);   // (the region of the per-index plan, unused on this path)
+#pragma unroll
+        for (int j = 0; j < kSparseMaxW32 / kWave; ++j) {
+            const int t = lane * wpl + j;
+            if (j < wpl && t < W32) {
+                sh.pr[t] = (uint16_t)((excl >> 16) + lr[j]);
+                uint32_t aw = sh.newbits[t] & ~sh.oldbits[t];
+                int o = (int)((excl & 0xffffu) + la[j]);
+                while (aw) {
+                    added_list[o++] = (uint16_t)(t * 32 + __ffs((int)aw) - 1);
+                    aw &= aw - 1u;
+                }
+            }
+        }
+        const uint32_t tot = (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+        const int na_w = (int)(tot & 0xffffu), nr_w = (int)(tot >> 16);
+        // (LDS operations of one wave execute in order: the lanes below read what other lanes of this wave wrote above)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+        int s = -1;
+        if (nr_w <= na_w) {
+            // ---- every removed index is paired with an added one: the positions' sources follow per position
+            int nn = n_old + (na_w - nr_w);
+            if (nn > I) nn = I;
+            if (lane < Q && my_p < nn) {
+                int newidx;
+                if (my_p < n_old) {
+                    const int e = ep ? i_old1 : i_old0;
+                    const int word = (e >> 5) & (kSparseMaxW32 - 1), bit = e & 31;
+                    const uint32_t remw = sh.oldbits[word] & ~sh.newbits[word];
+                    if ((remw >> bit) & 1u) {
+                        const int rank = (int)sh.pr[word] + __popc(remw & ((1u << bit) - 1u));
+                        newidx = (int)added_list[rank];
+                        s = newidx | kSrcPool;
+                    } else {
+                        newidx = e;
+                        s = my_p;
+                    }
+                } else {
+                    newidx = (int)added_list[nr_w + (my_p - n_old)];
+                    s = newidx | kSrcPool;
+                }
+                if ((na_w | nr_w) != 0) indices2[(size_t)(ep ^ 1) * I + my_p] = newidx;
+            }
+            if (lane == 0) sh.n = nn;
+        }
+        sh.src[lane] = s;
+        if (lane == 0) { sh.na = na_w; sh.nr = nr_w; }
+    }
+    speculate(std::integral_constant<int, SPEC_A>{}, std::integral_constant<int, SPEC>{});
+    __builtin_amdgcn_sched_barrier(0);
+    lds_barrier();
+    ST_TL(3);
+    const int na = sh.na, nr = sh.nr;
+    const bool changed = (na | nr) != 0;
+    bool arriver = plan_wave && lane == 0;
+    int next_epoch = ep;
+    if (nr <= na) {
+        n = sh.n;
+        if (changed) {
+            // the remembered mask: 8-byte words dealt to the blocks round-robin (the reference keeps the old
+            // mask when the update leaves nothing active)
+            uint8_t *mask_out = cur_mask2 + (size_t)(ep ^ 1) * I;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const int bi = tid * nw_rt + w;
+                if (w < nw_rt && bi * 8 < I && (bi % G) == blk)
+                    *reinterpret_cast<uint64_t *>(mask_out + (size_t)bi * 8) = n > 0 ? w_new[w] : w_cur[w];
+            }
+            if (blk == 0 && arriver) {
+                state[ST_STATE_N_BUF0 + (ep ^ 1)] = n;
+                state[ST_STATE_N_ACTIVE] = n;
+                state[ST_STATE_N_CHANGED] = na;
+                state[ST_STATE_N_ADDED] = na;
+                state[ST_STATE_N_REMOVED] = nr;
+                state[ST_STATE_SERIAL] = serial_old + 1;
+                state[ST_STATE_EPOCH] = ep ^ 1;
+                if (n > 0) {
+                    state[ST_STATE_STATUS] = 0;
+                    state[ST_STATE_VALID] = 1;
+                } else {
+                    state[ST_STATE_STATUS] = ST_ERR_NO_ACTIVE;
+                }
+            }
+            next_epoch = ep ^ 1;
+        } else if (blk == 0 && arriver) {
+            state[ST_STATE_N_CHANGED] = 0;
+            state[ST_STATE_N_ADDED] = 0;
+            state[ST_STATE_N_REMOVED] = 0;
+        }
+        if (arriver) arrival = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
+    } else {
+        // ---- removals outnumber additions: the sequential part of the reference decides the order
+        PlanView pv;
+        cache_plan<true, TPB, true, false>(pv, smem, &plan_shared, new_mask, cur_mask2, indices2, state, I, I, tid,
+                                           [] {}, [] {});
+        n = pv.n_new;
+        if (plan_wave) {
+            int s = -1;
+            if (lane < Q && my_p < n) {
+                const bool moved = my_p >= pv.n_old || ((pv.dirty[my_p >> 5] >> (my_p & 31)) & 1u);
+                s = moved ? ((int)pv.idx_l[my_p] | kSrcPool) : my_p;
+            }
+            sh.src[lane] = s;
+        }
+        arriver = pv.arriver; arrival = pv.arrival; next_epoch = pv.next_epoch;
+        // (requested again so that the first request's registers are free while the plan above runs)
+        speculate(std::integral_constant<int, 0>{}, std::integral_constant<int, SPEC>{});
+        lds_barrier();
+    }
+    ST_TL(4);
+
+    float acc[NB][VEC];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[b][e] = 0.f;
+
+    const int jcount = n > blk ? (n - blk + G - 1) / G : 0;      // rows of this block
+    const int nbat = ((jcount + ngrp - 1) / ngrp + RB - 1) / RB;  // uniform over the block
+    for (int bat = 0; bat < nbat; ++bat) {
+        unsigned fresh = 0u;   // bit k: row of slot k comes from the pool and has to be written back
+        auto request = [&](int k, bool speculated) __attribute__((always_inline)) {
+            const int q = grp + ngrp * (bat * RB + k);
+            const int p = blk + G * q;
+            const int s = sh.src[q < kSparseMaxQ ? q : kSparseMaxQ - 1];
+            const bool ok = q < Q && s >= 0;
+            const bool pooled = ok && (s & kSrcPool) != 0;
+            if (pooled) fresh |= 1u << k;
+            if (speculated && !pooled && p < n_spec) return;
+            const size_t ro = ok ? (size_t)(s & (kSrcPool - 1)) * row_bytes + coff : 0;   // no row: one piece for the whole wave
+            wu[k] = ld16_stream((pooled ? pool_u : act_u) + ro);
+            wd[k] = ld16_stream((pooled ? pool_d : act_d) + ro);
+            wg[k] = has_gate ? ld16_stream((pooled ? pool_g : act_g) + ro) : zero4;
+        };
+        if (wave_live) {
+            const bool spec = bat == 0 && n_spec > 0;
+#pragma unroll
+            for (int k = SPEC; k < RB; ++k) request(k, false);
+#pragma unroll
+            for (int k = 0; k < SPEC; ++k) request(k, spec);
+            if (spec && !has_gate) {
+#pragma unroll
+                for (int k = 0; k < SPEC; ++k) wg[k] = zero4;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < RB; ++k) wg[k] = wu[k] = wd[k] = zero4;
+        }
+        ST_TL(6);
+
+        // ---- phase 1: partial dot products on this thread's chunk
+        uint4 xq[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) xq[b] = (valid && b < B) ? xr[b] : zero4;
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                float pg = 0.f, pu = 0.f;
+                dot_chunk<T>(wg[k], wu[k], xq[b], pg, pu);
+                const float sg = wave_sum_dpp(pg), su = wave_sum_dpp(pu);
+                if (lane == 0) {
+                    red[wave][k][b][0] = sg;
+                    red[wave][k][b][1] = su;
+                }
+            }
+        }
+        // write the fresh rows back while the reductions settle
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+            if (((fresh >> k) & 1u) && valid) {
+                const size_t ro = (size_t)row_of(bat, k) * row_bytes + coff;
+                st16(act_u + ro, wu[k]);
+                st16(act_d + ro, wd[k]);
+                if (has_gate) st16(act_g + ro, wg[k]);
+            }
+        }
+        __syncthreads();
+        if (tid < ngrp * RB * NB) {
+            const int g_ = tid / (RB * NB), rem = tid - g_ * (RB * NB);
+            const int k_ = rem / NB, b_ = rem - k_ * NB;
+            const int row = blk + G * (g_ + ngrp * (bat * RB + k_));
+            float sg = 0.f, su = 0.f;
+            for (int wv = g_ * wpg; wv < (g_ + 1) * wpg; ++wv) {
+                sg += red[wv][k_][b_][0];
+                su += red[wv][k_][b_][1];
+            }
+            const float hv = has_gate ? activate(sg, act) * su : activate(su, act);
+            const bool ok = row < n;
+            hs[g_][k_][b_] = ok ? hv : 0.f;
+            if (ok && combined && b_ < B) {
+                combined[(size_t)b_ * ldc + row] = from_float<T>(hv);
+                if (has_gate) combined[(size_t)b_ * ldc + n + row] = from_float<T>(su);
+            }
+        }
+        __syncthreads();
+        // ---- phase 2: down projection from the rows already in registers
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+            const bool row_ok = row_of(bat, k) < n;
+            const uint4 rd = row_ok ? wd[k] : zero4;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) axpy_chunk<T>(hs[grp][k][b], rd, acc[b]);
+        }
+    }
+
+    // ---- combine the thread groups through LDS (behind the plan arrays), one fp32 partial row per block
+    if (ngrp > 1) {
+        float *redc = reinterpret_cast<float *>(smem + plan_bytes);  // [ngrp-1][NB][H]
+        if (grp > 0 && valid) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int e = 0; e < VEC; e += 4)
+                    *reinterpret_cast<float4 *>(redc + ((size_t)(grp - 1) * NB + b) * H + (size_t)cc * VEC + e) =
+                        make_float4(acc[b][e], acc[b][e + 1], acc[b][e + 2], acc[b][e + 3]);
+        }
+        __syncthreads();
+        if (grp == 0 && valid) {
+            for (int gq = 1; gq < ngrp; ++gq)
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+#pragma unroll
+                    for (int e = 0; e < VEC; e += 4) {
+                        const float4 v = *reinterpret_cast<const float4 *>(redc + ((size_t)(gq - 1) * NB + b) * H +
+                                                                            (size_t)cc * VEC + e);
+                        acc[b][e] += v.x; acc[b][e + 1] += v.y; acc[b][e + 2] += v.z; acc[b][e + 3] += v.w;
+                    }
+        }
+    }
+    if (grp == 0 && valid) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int e = 0; e < VEC; e += 4)
+                *reinterpret_cast<float4 *>(partials + ((size_t)blk * NB + b) * H + (size_t)cc * VEC + e) =
+                    make_float4(acc[b][e], acc[b][e + 1], acc[b][e + 2], acc[b][e + 3]);
+    }
+    // the block that arrived last resets the arrivals and sets the epoch (the atomic's result is first looked at here)
+    if (arriver) {
+        asm volatile("" : "+v"(arrival));
+        if ((arrival & 0xffffu) == gridDim.x - 1)
+            atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)next_epoch << 16);
+    }
+    ST_TL(7);
+}
+
 // in [R,C] -> out [C,R], 64x64 tiles through LDS.
 template <typename E>
 __global__ __launch_bounds__(256) void transpose_kernel(const E *__restrict__ in, E *__restrict__ out, int R, int C)
@@ -975,7 +1434,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
                          ((uintptr_t)c->b.indices % 16 == 0);
     static const bool fused_off = [] { const char *v = getenv("ST_CACHE_FUSED"); return v && atoi(v) == 0; }();
     const bool fused = !fused_off && B <= 2 && aligned && I <= 8 * TPB * kPlanMaxWords && chunks <= TPB &&
-                       row_bytes % 16 == 0 && lds <= (size_t)(156 * 1024);
+                       row_bytes % 16 == 0 && lds <= (size_t)(148 * 1024);
     if (!fused) {   // two launches: update, then the forward that reads the count on the device
         const int rc = st_cache_update_async(c, mask, stream);
         if (rc != ST_OK) return rc;
@@ -1013,6 +1472,47 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
             return ST_OK;
         };
         int rc;
+        // The per-position plan (cache_sparse_decode_kernel): a block owns at most kSparseMaxQ positions and the
+        // masks fit its bitmaps.  ST_FUSED_SPARSE=0 keeps the per-index plan below.
+        static const bool sparse_off = [] { const char *v = getenv("ST_FUSED_SPARSE"); return v && atoi(v) == 0; }();
+        const bool sparse = !sparse_off && (I + G - 1) / G <= kSparseMaxQ && I <= 32 * kSparseMaxW32 &&
+                            I <= 8 * TPB * kSparseWords;
+        if (sparse) {
+            auto launch_sparse = [&](auto kern, auto *xt, auto *ct) -> int {
+                static bool attr_set = false;
+                if (!attr_set) {
+                    ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 148 * 1024));
+                    attr_set = true;
+                }
+                ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, fr, mask, c->b.cur_mask, c->b.indices, c->b.state, I, xt,
+                          (int)B, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint);
+                return ST_OK;
+            };
+            const int rpg = ((hint + G - 1) / G + ngrp - 1) / ngrp;   // rows per thread group on the caller's guess
+            const bool seven = c->dtype != ST_F32 && B == 1 && (rpg + 6) / 7 < (rpg + 5) / 6;   // 7, 13, 14, ...
+#define ST_SPARSE_NW(TYPE, ROWS, NBX)                                                                               \
+    rc = I <= 8 * TPB ? launch_sparse(cache_sparse_decode_kernel<TYPE, ROWS, TPB, NBX, 1>, xt, ct)                  \
+                      : launch_sparse(cache_sparse_decode_kernel<TYPE, ROWS, TPB, NBX, 2>, xt, ct)
+#define ST_SPARSE_LAUNCH(TYPE)                                                                                      \
+    do {                                                                                                            \
+        const TYPE *xt = static_cast<const TYPE *>(x);                                                              \
+        TYPE *ct = static_cast<TYPE *>(combined);                                                                   \
+        if (B == 2 && rpg <= 6) ST_SPARSE_NW(TYPE, 6, 2);                                                           \
+        else if (B == 2) ST_SPARSE_NW(TYPE, 5, 2);                                                                  \
+        else if (seven) ST_SPARSE_NW(TYPE, 7, 1);                                                                   \
+        else if (rpg >= 1 && rpg <= 3) ST_SPARSE_NW(TYPE, 3, 1);                                                    \
+        else ST_SPARSE_NW(TYPE, DecodeRows<TYPE>::value, 1);                                                        \
+    } while (0)
+            if (c->dtype == ST_F32) ST_SPARSE_LAUNCH(float);
+            else if (c->dtype == ST_BF16) ST_SPARSE_LAUNCH(bf16_t);
+            else ST_SPARSE_LAUNCH(f16_t);
+#undef ST_SPARSE_LAUNCH
+#undef ST_SPARSE_NW
+            if (rc != ST_OK) return rc;
+            ST_HIP(hipGetLastError());
+            return launch_mlp_reduce(c->dtype, partials, G, NBF, (int)B, H, out, s);
+        }
         // split roles need whole row groups for each half and the plan done by half the threads
         static const bool split_off = [] { const char *v = getenv("ST_FUSED_SPLIT"); return v && atoi(v) == 0; }();
         // (only the fp16 instantiation of the split kernel fits the register file without spilling)
