@@ -23,6 +23,8 @@
 // the old buffer, because nobody writes it during this launch.
 #include "st_common.h"
 
+#include <atomic>
+
 #include <cstdlib>
 #include <new>
 #include <type_traits>
@@ -92,28 +94,6 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t *wave_t
     return prefix + incl - v;
 }
 
-// Barrier among a subset of the block's waves (all of which are resident together), through a counter in
-// LDS that only grows: each wave adds one and waits until all `waves` have.  The wait is bounded, so a
-// wave can never hang the GPU; running out of spins would mean a broken launch, not a slow one.
-__device__ __forceinline__ void sub_barrier(uint32_t *counter, uint32_t &target, int waves, int tid,
-                                            int32_t *fault)
-{
-    target += (uint32_t)waves;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    if ((tid & (kWave - 1)) == 0) atomicAdd(counter, 1u);
-    for (uint32_t spins = 0;; ++spins) {
-        if (spins == (1u << 22)) {   // leave a mark the host will see; the results of this launch are void
-            if ((tid & (kWave - 1)) == 0) *fault = 1;
-            break;
-        }
-        // (an atomic load rather than a volatile one: the latter is emitted as a flat load, which queues
-        // behind the block's global memory traffic)
-        if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= target) break;
-        __builtin_amdgcn_s_sleep(1);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
 struct CopyPlan {
     const unsigned char *pool[3];
     unsigned char *active[3];
@@ -165,14 +145,11 @@ constexpr size_t plan_lds_bytes(int I)
 struct PlanShared {
     uint32_t wave_tot[kPlanWaves];
     int n_new_s;   // count after the sequential removals (slow path)
-    uint32_t sub_count;          // sub_barrier counter
-    int out_n_old, out_n_new, out_changed;   // the finished plan, for waves that did not take part
 };
 
 // Replays the bookkeeping of one update in LDS and publishes it (block 0 writes the other bookkeeping
-// buffer, the last block to arrive flips the epoch).  Called by PT threads of the block (tid = 0..PT-1)
-// that are exactly the threads executing block barriers at that time, or by all of them together with
-// the rest of the block waiting at a block barrier (SUB); contains barriers.  VEC: I % 8 == 0 and the mask is
+// buffer, the last block to arrive flips the epoch).  Called by all PT threads of the block (tid = 0..PT-1);
+// contains block barriers.  VEC: I % 8 == 0 and the mask is
 // 8-byte aligned, so masks are read as 8-byte words and indices as 16-byte vectors; both bookkeeping
 // buffers are requested together with the ticket, so the front costs one memory round trip.  MARK: the
 // dirty bitmap is kept on the fast path too.  `after_issue()` runs right after the front loads have
@@ -183,7 +160,7 @@ struct PlanShared {
 // Barrier sequence: 1 after the LDS fill; 2 in the diff scan;
 // [unchanged mask: done]; 1 after the lists; 1 after phases 1 and 2; [surplus removals: 1 after phase 3,
 // 2 in the compaction scan, 1 after the compaction].
-template <bool VEC, int PT, bool MARK, bool SUB, typename F, typename F2>
+template <bool VEC, int PT, bool MARK, typename F, typename F2>
 __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, PlanShared *ps,
                                            const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2,
                                            int32_t *__restrict__ indices2, int32_t *__restrict__ state, int I,
@@ -201,12 +178,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
     uint8_t *flag_l = reinterpret_cast<uint8_t *>(dirty + ((dirty_words + 1) & ~1));  // bit0 new, bit1 old; 8-byte aligned
     uint32_t *wave_tot = ps->wave_tot;
     int &n_new_s = ps->n_new_s;
-    // SUB: the PT threads are only part of the block and synchronise among themselves
-    uint32_t sub_target = 0;
-    auto sync = [&]() __attribute__((always_inline)) {
-        if constexpr (SUB) sub_barrier(&ps->sub_count, sub_target, PT / kWave, tid, &state[ST_STATE_FAULT]);
-        else lds_barrier();
-    };
+    auto sync = [&]() __attribute__((always_inline)) { lds_barrier(); };
     pv.pos_l = pos_l; pv.idx_l = idx_l; pv.lists = lists; pv.dirty = dirty;
     pv.arriver = tid == 0;
 
@@ -287,11 +259,7 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
         }
     }
     ST_TL(1);
-    // SUB: this one barrier is a block barrier -- the rest of the block holds its memory requests back
-    // until the plan's own loads have arrived (under a saturated memory system they would take several
-    // times longer, and the whole plan hangs on them)
-    if constexpr (SUB) lds_barrier();
-    else sync();
+    sync();
     after_fill();
     ST_TL(2);
     if (VEC && n > idx_cap) {   // more positions in use than the caller expected: fetch the rest (one more round trip)
@@ -473,26 +441,6 @@ __device__ __forceinline__ void cache_plan(PlanView &pv, unsigned char *smem, Pl
 }
 
 
-// The finished plan as seen by waves that did not take part in it (after the block barrier that follows
-// plan_publish).
-__device__ __forceinline__ void plan_publish(const PlanView &pv, PlanShared *ps)
-{
-    if (pv.arriver) {
-        ps->out_n_old = pv.n_old;
-        ps->out_n_new = pv.n_new;
-        ps->out_changed = pv.changed ? 1 : 0;
-    }
-}
-__device__ __forceinline__ void plan_adopt(PlanView &pv, unsigned char *smem, const PlanShared *ps, int I)
-{
-    uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);
-    pv.pos_l = pos_l; pv.idx_l = pos_l + I; pv.lists = pos_l + 2 * I;
-    pv.dirty = reinterpret_cast<uint32_t *>(pv.lists + I + (I & 1));
-    pv.arriver = false; pv.writer = false; pv.arrival = 0; pv.next_epoch = 0; pv.ep = 0; pv.n_changed = 0;
-    pv.na = pv.nr = 0;
-    pv.n_old = ps->out_n_old; pv.n_new = ps->out_n_new; pv.changed = ps->out_changed != 0;
-}
-
 // Last step of a kernel that ran cache_plan: the block that arrived last resets the arrivals and sets the
 // epoch.  Looking at the atomic's result only here keeps its round trip off the critical path.
 __device__ __forceinline__ void plan_finish(const PlanView &pv, int32_t *__restrict__ state)
@@ -517,7 +465,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
     __shared__ PlanShared ps;
     const int tid = threadIdx.x;
     PlanView pv;
-    cache_plan<VEC, TPB, false, false>(pv, smem, &ps, new_mask, cur_mask2, indices2, state, I, idx_cap, tid, [] {}, [] {});
+    cache_plan<VEC, TPB, false>(pv, smem, &ps, new_mask, cur_mask2, indices2, state, I, idx_cap, tid, [] {}, [] {});
     if (!pv.changed) {
         plan_finish(pv, state);
         return;
@@ -564,239 +512,6 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
 
     plan_finish(pv, state);
     ST_TL(6);
-}
-
-// ---------------------------------------------------------------------------
-// update + sparse MLP for one row of x in ONE kernel.
-//
-// Every block replays the plan (as above) and then streams its share of the
-// active rows exactly like mlp_decode_kernel does -- except that a position
-// whose index changed is read from the POOL row of its new index instead of
-// the active buffer, and written back to the active buffer from the registers
-// it already sits in.  The separate copy pass, its launch and its memory round
-// trips disappear; the cache ends in the same state as after
-// cache_update_kernel, and the arithmetic (row -> block dealing, summation
-// order) is that of mlp_decode_kernel, so the result is bit-identical to
-// update followed by forward.
-// Rows are dealt to blocks round-robin: row(bat, k) = blk + G * (grp + ngrp * (bat * RB + k)).
-// ---------------------------------------------------------------------------
-template <typename T, int RB, int PLANW, int TPB, bool AHEAD = false, int NB = 1>
-__global__ __launch_bounds__(TPB) void cache_update_decode_kernel(
-    FusedRows fr, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
-    int32_t *__restrict__ state, int I, const T *__restrict__ x, int B, int H, T *__restrict__ combined, long ldc,
-    float *__restrict__ partials, int act, int gs_log2, int plan_bytes, int n_hint, int idx_cap)
-{
-    // NB rows of x per pass (B <= NB; rows past B are zeros): [G][NB][H] partial rows
-    constexpr int VEC = Elem<T>::kVec;
-    extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ float red[TPB / kWave][RB][NB][2];  // per-wave partial (g,u)
-    __shared__ float hs[TPB / kWave][RB][NB];      // h of the rows being computed
-
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const int G = gridDim.x, blk = blockIdx.x;
-    const int chunks = H / VEC;
-    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
-    const int GS = 1 << gs_log2, ngrp = TPB >> gs_log2, wpg = GS >> 6;
-    const int grp = tid >> gs_log2, cc = tid & (GS - 1);
-    const bool valid = cc < chunks;
-    const size_t coff = valid ? (size_t)cc * 16 : 0;   // byte offset of this thread's chunk (clamped)
-    const bool wave_live = __builtin_amdgcn_readfirstlane(cc & ~(kWave - 1)) < chunks;
-    const bool has_gate = fr.has_gate != 0;
-    const int row_bytes = fr.row_bytes;
-    const unsigned char *const pool_g = fr.pool_g, *const pool_u = fr.pool_u, *const pool_d = fr.pool_d;
-    unsigned char *const act_g = fr.act_g, *const act_u = fr.act_u, *const act_d = fr.act_d;
-
-    // x is requested behind the loads the plan hangs on (planning waves) or while waiting for them (the
-    // others), and looked at only in phase 1
-    uint4 xr[NB];
-    auto load_x = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int b = 0; b < NB; ++b)
-            xr[b] = ld16(reinterpret_cast<const unsigned char *>(x) + (size_t)(b < B ? b : 0) * row_bytes + coff);
-    };
-
-    auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
-
-    // PLANW > 0: only the last PLANW waves work out the plan while the others already stream their share of
-    // the first batch of rows from the active buffers, on the host's guess of the count (most rows are
-    // unchanged; the others are requested again from the right place once the plan is known).  A wave
-    // owns a range of columns of its row group's rows, so whatever the planning waves own arrives late:
-    // the fewer they are, the less.
-    uint4 wg[RB], wu[RB], wd[RB];
-    constexpr bool SPLIT = PLANW > 0;
-    constexpr int PT = SPLIT ? PLANW * kWave : TPB;
-    const bool streams_ahead = SPLIT && tid < TPB - PT;
-    // AHEAD (all waves plan): every wave requests its first batch on the host's guess as soon as the plan's
-    // own loads are in, and goes on planning with those requests in flight.  Wherever the plan code makes
-    // a wave wait for its outstanding loads it waits for the rows too, so this pays when a block's rows
-    // arrive in less time than the plan takes (few active rows per block).
-    static_assert(!(AHEAD && SPLIT), "the two ways of streaming ahead exclude each other");
-    const int n_spec = (SPLIT || AHEAD) ? (n_hint < I ? n_hint : I) : 0;
-    __shared__ PlanShared plan_shared;
-    PlanView pv;
-    if (SPLIT && tid == 0) plan_shared.sub_count = 0;
-    auto speculate = [&]() __attribute__((always_inline)) {
-        if (wave_live && n_spec > 0) {
-#pragma unroll
-            for (int k = 0; k < RB; ++k) {
-                const int p = row_of(0, k);
-                const size_t ro = (size_t)(p < n_spec ? p : n_spec - 1) * row_bytes + coff;
-                wu[k] = ld16_stream(act_u + ro);
-                wd[k] = ld16_stream(act_d + ro);
-                if (has_gate) wg[k] = ld16_stream(act_g + ro);
-            }
-        }
-    };
-    if (streams_ahead) {
-        load_x();
-        lds_barrier();   // (A) the plan's own loads have arrived (inside cache_plan, after the LDS fill)
-        speculate();
-        lds_barrier();   // (B) the plan is finished
-        plan_adopt(pv, smem, &plan_shared, I);
-    } else {
-        // block barrier (A) sits inside the plan, where its loads have arrived; after it the planning
-        // waves synchronise among themselves, so the streaming waves are free to stall on their own
-        // memory requests
-        cache_plan<true, PT, true, SPLIT>(pv, smem, &plan_shared, new_mask, cur_mask2, indices2, state, I,
-                                          idx_cap, SPLIT ? tid - (TPB - PT) : tid,
-                                          [&] { load_x(); },
-                                          [&] { if constexpr (AHEAD) speculate(); });
-        if (SPLIT) {
-            plan_publish(pv, &plan_shared);
-            lds_barrier();   // (B)
-        }
-    }
-    const int n = pv.n_new, n_old = pv.n_old;
-
-    float acc[NB][VEC];
-#pragma unroll
-    for (int b = 0; b < NB; ++b)
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[b][e] = 0.f;
-
-    const int jcount = n > blk ? (n - blk + G - 1) / G : 0;      // rows of this block
-    const int nbat = ((jcount + ngrp - 1) / ngrp + RB - 1) / RB;  // uniform over the block
-    for (int bat = 0; bat < nbat; ++bat) {
-        unsigned fresh = 0u;   // bit k: row of slot k comes from the pool and has to be written back
-        // (rows, source) of slot k; issues the loads unless the speculative request already covers them
-        auto request = [&](int k, bool speculated) __attribute__((always_inline)) {
-            const int p = row_of(bat, k);
-            const bool ok = p < n;
-            const int pc = ok ? p : n - 1;   // clamped; rows past the count are neutralised below
-            const bool moved = pc >= n_old || ((pv.dirty[pc >> 5] >> (pc & 31)) & 1u);
-            const bool pooled = ok && moved && pv.changed;
-            if (pooled) fresh |= 1u << k;
-            if (speculated && !pooled && p < n_spec) return;
-            const int pooled_row = (int)pv.idx_l[pc];   // read whether needed or not: no branch, plain selects below
-            const size_t ro = (size_t)(pooled ? pooled_row : pc) * row_bytes + coff;
-            wu[k] = ld16_stream((pooled ? pool_u : act_u) + ro);
-            wd[k] = ld16_stream((pooled ? pool_d : act_d) + ro);
-            wg[k] = has_gate ? ld16_stream((pooled ? pool_g : act_g) + ro) : zero4;
-        };
-        if (wave_live) {
-            const bool spec = (streams_ahead || AHEAD) && bat == 0 && n_spec > 0;   // uniform over the wave
-#pragma unroll
-            for (int k = 0; k < RB; ++k) request(k, spec);   // static slot numbers keep the rows in registers
-            if (spec && !has_gate) {
-#pragma unroll
-                for (int k = 0; k < RB; ++k) wg[k] = zero4;
-            }
-        } else {
-#pragma unroll
-            for (int k = 0; k < RB; ++k) wg[k] = wu[k] = wd[k] = zero4;
-        }
-        ST_TL(6);
-
-        // ---- phase 1: partial dot products on this thread's chunk
-        uint4 xq[NB];
-#pragma unroll
-        for (int b = 0; b < NB; ++b) xq[b] = (valid && b < B) ? xr[b] : zero4;
-#pragma unroll
-        for (int k = 0; k < RB; ++k) {
-#pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                float pg = 0.f, pu = 0.f;
-                dot_chunk<T>(wg[k], wu[k], xq[b], pg, pu);
-                const float sg = wave_sum_dpp(pg), su = wave_sum_dpp(pu);
-                if (lane == 0) {
-                    red[wave][k][b][0] = sg;
-                    red[wave][k][b][1] = su;
-                }
-            }
-        }
-        // write the fresh rows back while the reductions settle
-#pragma unroll
-        for (int k = 0; k < RB; ++k) {
-            if (((fresh >> k) & 1u) && valid) {
-                const size_t ro = (size_t)row_of(bat, k) * row_bytes + coff;
-                st16(act_u + ro, wu[k]);
-                st16(act_d + ro, wd[k]);
-                if (has_gate) st16(act_g + ro, wg[k]);
-            }
-        }
-        __syncthreads();
-        if (tid < ngrp * RB * NB) {
-            const int g_ = tid / (RB * NB), rem = tid - g_ * (RB * NB);
-            const int k_ = rem / NB, b_ = rem - k_ * NB;
-            const int row = blk + G * (g_ + ngrp * (bat * RB + k_));
-            float sg = 0.f, su = 0.f;
-            for (int wv = g_ * wpg; wv < (g_ + 1) * wpg; ++wv) {
-                sg += red[wv][k_][b_][0];
-                su += red[wv][k_][b_][1];
-            }
-            const float hv = has_gate ? activate(sg, act) * su : activate(su, act);
-            const bool ok = row < n;
-            hs[g_][k_][b_] = ok ? hv : 0.f;
-            if (ok && combined && b_ < B) {
-                combined[(size_t)b_ * ldc + row] = from_float<T>(hv);
-                if (has_gate) combined[(size_t)b_ * ldc + n + row] = from_float<T>(su);
-            }
-        }
-        __syncthreads();
-        // ---- phase 2: down projection from the rows already in registers
-#pragma unroll
-        for (int k = 0; k < RB; ++k) {
-            const bool row_ok = row_of(bat, k) < n;
-            const uint4 rd = row_ok ? wd[k] : zero4;
-#pragma unroll
-            for (int b = 0; b < NB; ++b) axpy_chunk<T>(hs[grp][k][b], rd, acc[b]);
-        }
-    }
-
-    // ---- combine the thread groups through LDS (behind the plan arrays), one fp32 partial row per block
-    if (ngrp > 1) {
-        float *redc = reinterpret_cast<float *>(smem + plan_bytes);  // [ngrp-1][NB][H]
-        if (grp > 0 && valid) {
-#pragma unroll
-            for (int b = 0; b < NB; ++b)
-#pragma unroll
-                for (int e = 0; e < VEC; e += 4)
-                    *reinterpret_cast<float4 *>(redc + ((size_t)(grp - 1) * NB + b) * H + (size_t)cc * VEC + e) =
-                        make_float4(acc[b][e], acc[b][e + 1], acc[b][e + 2], acc[b][e + 3]);
-        }
-        __syncthreads();
-        if (grp == 0 && valid) {
-            for (int gq = 1; gq < ngrp; ++gq)
-#pragma unroll
-                for (int b = 0; b < NB; ++b)
-#pragma unroll
-                    for (int e = 0; e < VEC; e += 4) {
-                        const float4 v = *reinterpret_cast<const float4 *>(redc + ((size_t)(gq - 1) * NB + b) * H +
-                                                                            (size_t)cc * VEC + e);
-                        acc[b][e] += v.x; acc[b][e + 1] += v.y; acc[b][e + 2] += v.z; acc[b][e + 3] += v.w;
-                    }
-        }
-    }
-    if (grp == 0 && valid) {
-#pragma unroll
-        for (int b = 0; b < NB; ++b)
-#pragma unroll
-            for (int e = 0; e < VEC; e += 4)
-                *reinterpret_cast<float4 *>(partials + ((size_t)blk * NB + b) * H + (size_t)cc * VEC + e) =
-                    make_float4(acc[b][e], acc[b][e + 1], acc[b][e + 2], acc[b][e + 3]);
-    }
-    plan_finish(pv, state);
-    ST_TL(7);
 }
 
 // ---------------------------------------------------------------------------
@@ -1085,7 +800,7 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     } else {
         // ---- removals outnumber additions: the sequential part of the reference decides the order
         PlanView pv;
-        cache_plan<true, TPB, true, false>(pv, smem, &plan_shared, new_mask, cur_mask2, indices2, state, I, I, tid,
+        cache_plan<true, TPB, true>(pv, smem, &plan_shared, new_mask, cur_mask2, indices2, state, I, I, tid,
                                            [] {}, [] {});
         n = pv.n_new;
         if (plan_wave) {
@@ -1385,11 +1100,11 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     {
         ProfScope ps(ST_K_CACHE_UPDATE, s);
         auto launch = [&](auto kern) -> int {
-            static bool attr_set = false;
-            if (!attr_set) {
+            static std::atomic<bool> attr_set{false};   // (setting the attribute twice from two threads is harmless)
+            if (!attr_set.load(std::memory_order_acquire)) {
                 ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
-                attr_set = true;
+                attr_set.store(true, std::memory_order_release);
             }
             ST_LAUNCH(ps, kern, dim3(grid), dim3(tpb), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state,
                                I, gs_log2, idx_cap);
@@ -1430,11 +1145,15 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
     const size_t plan_bytes = (plan_lds_bytes(I) + 15) & ~(size_t)15;
     const int NBF = B == 2 ? 2 : 1;   // rows of x the fused kernel takes in one pass
     const size_t lds = plan_bytes + (size_t)(ngrp - 1) * NBF * H * 4;
+    const int G = mlp_grid();
     const bool aligned = (I % 8 == 0) && ((uintptr_t)mask % 8 == 0) && ((uintptr_t)c->b.cur_mask % 8 == 0) &&
                          ((uintptr_t)c->b.indices % 16 == 0);
     static const bool fused_off = [] { const char *v = getenv("ST_CACHE_FUSED"); return v && atoi(v) == 0; }();
-    const bool fused = !fused_off && B <= 2 && aligned && I <= 8 * TPB * kPlanMaxWords && chunks <= TPB &&
-                       row_bytes % 16 == 0 && lds <= (size_t)(148 * 1024);
+    // One kernel for one or two rows of x when a block owns at most kSparseMaxQ positions, the masks fit the
+    // kernel's bitmaps and a row fits one pass of a thread group; everything else runs as two calls.
+    const bool fused = !fused_off && B <= 2 && aligned && I >= 8 && (I + G - 1) / G <= kSparseMaxQ &&
+                       I <= 32 * kSparseMaxW32 && I <= 8 * TPB * kSparseWords && chunks <= TPB && row_bytes % 16 == 0 &&
+                       lds <= (size_t)(148 * 1024);
     if (!fused) {   // two launches: update, then the forward that reads the count on the device
         const int rc = st_cache_update_async(c, mask, stream);
         if (rc != ST_OK) return rc;
@@ -1451,49 +1170,30 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
     fr.act_g = c->has_gate ? static_cast<unsigned char *>(c->b.gate_active) : fr.act_u;
     fr.row_bytes = row_bytes;
     fr.has_gate = c->has_gate ? 1 : 0;
-    const int G = mlp_grid();
     float *partials = static_cast<float *>(workspace);
     const int hint = (int)(n_hint < 0 ? 0 : (n_hint > c->I ? c->I : n_hint));
-    // The plan needs the index list only up to the count in use, which lives on the device: blocks fetch the
-    // first `idx_cap` positions with their other bookkeeping loads (a quarter more than the caller's guess)
-    // and the rest, if the guess was too low, in a second round trip.
-    const int idx_cap = hint > 0 && hint + hint / 4 + 64 < I ? (hint + hint / 4 + 64 + 7) & ~7 : I;
     {
         ProfScope ps(ST_K_CACHE_UPDATE_DECODE, s);
         auto launch = [&](auto kern, auto *xt, auto *ct) -> int {
-            static bool attr_set = false;
-            if (!attr_set) {
+            static std::atomic<bool> attr_set{false};   // (setting the attribute twice from two threads is harmless)
+            if (!attr_set.load(std::memory_order_acquire)) {
                 ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
-                attr_set = true;
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 148 * 1024));
+                attr_set.store(true, std::memory_order_release);
             }
-            ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, fr, mask, c->b.cur_mask, c->b.indices, c->b.state, I,
-                               xt, (int)B, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint, idx_cap);
+            ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, fr, mask, c->b.cur_mask, c->b.indices, c->b.state, I, xt,
+                      (int)B, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint);
             return ST_OK;
         };
         int rc;
-        // The per-position plan (cache_sparse_decode_kernel): a block owns at most kSparseMaxQ positions and the
-        // masks fit its bitmaps.  ST_FUSED_SPARSE=0 keeps the per-index plan below.
-        static const bool sparse_off = [] { const char *v = getenv("ST_FUSED_SPARSE"); return v && atoi(v) == 0; }();
-        const bool sparse = !sparse_off && (I + G - 1) / G <= kSparseMaxQ && I <= 32 * kSparseMaxW32 &&
-                            I <= 8 * TPB * kSparseWords;
-        if (sparse) {
-            auto launch_sparse = [&](auto kern, auto *xt, auto *ct) -> int {
-                static bool attr_set = false;
-                if (!attr_set) {
-                    ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 148 * 1024));
-                    attr_set = true;
-                }
-                ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, fr, mask, c->b.cur_mask, c->b.indices, c->b.state, I, xt,
-                          (int)B, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint);
-                return ST_OK;
-            };
-            const int rpg = ((hint + G - 1) / G + ngrp - 1) / ngrp;   // rows per thread group on the caller's guess
-            const bool seven = c->dtype != ST_F32 && B == 1 && (rpg + 6) / 7 < (rpg + 5) / 6;   // 7, 13, 14, ...
+        // Rows a thread group keeps in flight (it does not change which rows a group sums, or in which order): six;
+        // seven where the caller's guess of the count gives a group 7, 13 or 14 rows (one batch less); three when
+        // a group has at most three rows; two rows of x: six when that is one batch, else five.
+        const int rpg = ((hint + G - 1) / G + ngrp - 1) / ngrp;   // rows per thread group on the caller's guess
+        const bool seven = c->dtype != ST_F32 && B == 1 && (rpg + 6) / 7 < (rpg + 5) / 6;
 #define ST_SPARSE_NW(TYPE, ROWS, NBX)                                                                               \
-    rc = I <= 8 * TPB ? launch_sparse(cache_sparse_decode_kernel<TYPE, ROWS, TPB, NBX, 1>, xt, ct)                  \
-                      : launch_sparse(cache_sparse_decode_kernel<TYPE, ROWS, TPB, NBX, 2>, xt, ct)
+    rc = I <= 8 * TPB ? launch(cache_sparse_decode_kernel<TYPE, ROWS, TPB, NBX, 1>, xt, ct)                         \
+                      : launch(cache_sparse_decode_kernel<TYPE, ROWS, TPB, NBX, 2>, xt, ct)
 #define ST_SPARSE_LAUNCH(TYPE)                                                                                      \
     do {                                                                                                            \
         const TYPE *xt = static_cast<const TYPE *>(x);                                                              \
@@ -1504,63 +1204,11 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
         else if (rpg >= 1 && rpg <= 3) ST_SPARSE_NW(TYPE, 3, 1);                                                    \
         else ST_SPARSE_NW(TYPE, DecodeRows<TYPE>::value, 1);                                                        \
     } while (0)
-            if (c->dtype == ST_F32) ST_SPARSE_LAUNCH(float);
-            else if (c->dtype == ST_BF16) ST_SPARSE_LAUNCH(bf16_t);
-            else ST_SPARSE_LAUNCH(f16_t);
+        if (c->dtype == ST_F32) ST_SPARSE_LAUNCH(float);
+        else if (c->dtype == ST_BF16) ST_SPARSE_LAUNCH(bf16_t);
+        else ST_SPARSE_LAUNCH(f16_t);
 #undef ST_SPARSE_LAUNCH
 #undef ST_SPARSE_NW
-            if (rc != ST_OK) return rc;
-            ST_HIP(hipGetLastError());
-            return launch_mlp_reduce(c->dtype, partials, G, NBF, (int)B, H, out, s);
-        }
-        // split roles need whole row groups for each half and the plan done by half the threads
-        static const bool split_off = [] { const char *v = getenv("ST_FUSED_SPLIT"); return v && atoi(v) == 0; }();
-        // (only the fp16 instantiation of the split kernel fits the register file without spilling)
-        // and it pays only when a block has enough rows to stream while the plan is worked out
-        const bool split = !split_off && ngrp >= 2 && (ngrp & 1) == 0 && hint >= 6 * G &&
-                           I <= 8 * (TPB / 2) * kPlanMaxWords;
-        // (four planning waves instead of eight leave less to arrive late, but take so much longer over the
-        // plan that the kernel measures 21.1 us instead of 18.9 us)
-        // few rows per block: all waves plan, with their rows requested ahead
-        static const int ahead_env = [] { const char *v = getenv("ST_FUSED_AHEAD"); return v ? atoi(v) : -1; }();
-        const bool ahead = !split && hint > 0 && (ahead_env < 0 ? hint < 6 * G : ahead_env != 0);
-        // (the rows in flight per group do not change which rows a group sums or in which order, so the
-        // ahead variant is free to keep three: enough for fewer than 6 rows per block, and it leaves the
-        // registers the plan needs beside them)
-        // seven rows per group: one batch of seven (all 16 waves plan: the split form has no registers left for
-        // a seventh row) beats a batch of six and a second one of one -- 26.9 against 30.1 us at n = 3584, H = 4096
-        const int rows_per_group = ((hint + G - 1) / G + ngrp - 1) / ngrp;
-        const bool rows7 = c->dtype != ST_F32 && (rows_per_group + 6) / 7 < (rows_per_group + 5) / 6;   // 7, 13, 14, ...
-#define ST_FUSED_LAUNCH(TYPE, PLANW, AHEAD)                                                            \
-    rc = launch(cache_update_decode_kernel<TYPE, (AHEAD) ? 3 : DecodeRows<TYPE>::value, PLANW, TPB, AHEAD>, \
-                static_cast<const TYPE *>(x), static_cast<TYPE *>(combined))
-        // two rows of x: all waves plan (the second row of x costs the registers the split form would need); six
-        // rows per group in flight when that is one batch, else five (measured faster than six at seven rows)
-        if (B == 2) {
-#define ST_FUSED_LAUNCH2(TYPE, ROWS)                                                                             \
-    rc = launch(cache_update_decode_kernel<TYPE, ROWS, 0, TPB, false, 2>, static_cast<const TYPE *>(x),          \
-                static_cast<TYPE *>(combined))
-            const bool one_batch = ((hint + G - 1) / G + ngrp - 1) / ngrp <= 6;
-            if (c->dtype == ST_F32) { if (one_batch) ST_FUSED_LAUNCH2(float, 6); else ST_FUSED_LAUNCH2(float, 5); }
-            else if (c->dtype == ST_BF16) { if (one_batch) ST_FUSED_LAUNCH2(bf16_t, 6); else ST_FUSED_LAUNCH2(bf16_t, 5); }
-            else { if (one_batch) ST_FUSED_LAUNCH2(f16_t, 6); else ST_FUSED_LAUNCH2(f16_t, 5); }
-#undef ST_FUSED_LAUNCH2
-        } else if (c->dtype == ST_F32 && split) ST_FUSED_LAUNCH(float, 8, false);
-        else if (c->dtype == ST_F32 && ahead) ST_FUSED_LAUNCH(float, 0, true);
-        else if (c->dtype == ST_F32) ST_FUSED_LAUNCH(float, 0, false);
-        else if (c->dtype == ST_BF16 && rows7)
-            rc = launch(cache_update_decode_kernel<bf16_t, 7, 0, TPB, false>, static_cast<const bf16_t *>(x),
-                        static_cast<bf16_t *>(combined));
-        else if (c->dtype == ST_F16 && rows7)
-            rc = launch(cache_update_decode_kernel<f16_t, 7, 0, TPB, false>, static_cast<const f16_t *>(x),
-                        static_cast<f16_t *>(combined));
-        else if (c->dtype == ST_BF16 && split) ST_FUSED_LAUNCH(bf16_t, 8, false);
-        else if (c->dtype == ST_BF16 && ahead) ST_FUSED_LAUNCH(bf16_t, 0, true);
-        else if (c->dtype == ST_BF16) ST_FUSED_LAUNCH(bf16_t, 0, false);
-        else if (split) ST_FUSED_LAUNCH(f16_t, 8, false);
-        else if (ahead) ST_FUSED_LAUNCH(f16_t, 0, true);
-        else ST_FUSED_LAUNCH(f16_t, 0, false);
-#undef ST_FUSED_LAUNCH
         if (rc != ST_OK) return rc;
     }
     ST_HIP(hipGetLastError());

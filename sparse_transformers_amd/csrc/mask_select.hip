@@ -15,6 +15,8 @@
 // change the result.
 #include "st_common.h"
 
+#include <atomic>
+
 namespace st {
 
 constexpr int kSelThreads = 1024;
@@ -376,11 +378,11 @@ extern "C" int st_mask_select(const float *scores, int64_t B, int64_t I, int met
         rowmask = static_cast<uint8_t *>(workspace) + 16;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<bool> attr_set{false};   // (setting the attribute twice from two threads is harmless)
+    if (!attr_set.load(std::memory_order_acquire)) {
         ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(mask_select_kernel<0>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, kSelMaxLdsKeys * 4));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     ProfScope ps(ST_K_MASK_SELECT, s);
     const dim3 grid((unsigned)B), block(kSelThreads);

@@ -29,6 +29,8 @@
 // SkipMLP._forward_sparse_weight_cache (src/modeling_skip.py:114-117).
 #include "st_mfma.h"
 
+#include <atomic>
+
 namespace st {
 
 constexpr int kBtThreads = 512;
@@ -385,11 +387,11 @@ static int launch_gateup(const T *x, int B, const T *gate, const T *up, int n, c
 {
     auto kern = batch_gateup_kernel<T, KSW, HG, NT>;
     const size_t lds = (NT == 1 ? (size_t)kBtRows * (KSW * 256 + kBtXPad) * 2 : 0) + (size_t)NT * kBtRedFloats * 4;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<bool> attr_set{false};   // (setting the attribute twice from two threads is harmless)
+    if (!attr_set.load(std::memory_order_acquire)) {
         ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)lds));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     ProfScope ps(ST_K_MLP_BATCH_GATEUP, stream);
     ST_LAUNCH(ps, kern, dim3(device_cu_count()), dim3(kBtThreads), lds, stream, x, B, gate, up, n, n_dev, hbuf,
@@ -404,11 +406,11 @@ static int launch_down(const T *hbuf, int ldh, int B, const T *down, int H, int 
     auto kern = batch_down_kernel<T, NP, NX>;
     const size_t red = (size_t)kBtWaves * NP * 4 * 256 * 4, stage = (size_t)kBtWaves * kBtStageBytes;
     const size_t lds = red > stage ? red : stage;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<bool> attr_set{false};   // (setting the attribute twice from two threads is harmless)
+    if (!attr_set.load(std::memory_order_acquire)) {
         ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)lds));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     ProfScope ps(ST_K_MLP_BATCH_DOWN, stream);
     ST_LAUNCH(ps, kern, dim3(cg * rs), dim3(kBtThreads), lds, stream, hbuf, ldh, B, down, H, n, n_dev, partial, cg, rs);

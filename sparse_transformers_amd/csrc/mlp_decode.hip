@@ -20,6 +20,8 @@
 // and SkipMLP._forward_sparse_weight_cache (src/modeling_skip.py:114-117).
 #include "st_common.h"
 
+#include <atomic>
+
 #include <cstdlib>
 #include <mutex>
 
@@ -327,11 +329,11 @@ static int launch_inst(const MlpLaunch &a, int b0, int bcount)
     const size_t lds = (size_t)(ngrp - 1) * NB * a.H * 4;
     ST_REQUIRE(lds <= (size_t)kMaxLds - 8192, "st_mlp_forward: H=%d needs %zu bytes of LDS", a.H, lds);
     auto kern = mlp_decode_kernel<T, NB, RB, CPT, TPB, DB>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static std::atomic<bool> attr_set{false};   // (setting the attribute twice from two threads is harmless)
+    if (!attr_set.load(std::memory_order_acquire)) {
         ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    kMaxLds - 8192));
-        attr_set = true;
+        attr_set.store(true, std::memory_order_release);
     }
     const T *x = static_cast<const T *>(a.x) + (size_t)b0 * a.H;
     T *comb = a.combined ? static_cast<T *>(a.combined) + (size_t)b0 * a.ldc : nullptr;
