@@ -146,6 +146,10 @@ int st_mask_select(const float *scores, int64_t B, int64_t I, int method, int64_
  * in sparse_mlp_op.cpp:208) for float scores: threshold[b] = 0.9 * the
  * max(1, k*cells/F)-th largest sketch cell of row b.  F >= 4, 0 < k <= F. */
 int st_approx_topk_threshold(const float *scores, int64_t B, int64_t F, int64_t k, float *threshold, void *stream);
+/* The same for double scores and thresholds (the reference dispatches on every floating type, approx_topk.h:33;
+ * its adjustment factor is then the double 0.9). */
+int st_approx_topk_threshold_f64(const double *scores, int64_t B, int64_t F, int64_t k, double *threshold,
+                                 void *stream);
 
 /* ------------------------------------------------------------------------
  * Differential weight cache, resident in HBM.

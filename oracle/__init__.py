@@ -60,6 +60,7 @@ def lib() -> C.CDLL:
         L.orc_mask_topk.argtypes = [vp, i64, i64, i64, vp]
         L.orc_mask_statistical.argtypes = [vp, i64, i64, C.c_float, vp, vp]
         L.orc_approx_topk_threshold.argtypes = [vp, i64, i64, i64, vp]
+        L.orc_approx_topk_threshold_f64.argtypes = [vp, i64, i64, i64, vp]
         _lib = L
     return _lib
 
@@ -186,8 +187,10 @@ def mask_statistical(scores, z):
 
 
 def approx_topk_threshold(scores, k) -> np.ndarray:
-    """Per-row sketch threshold [B] (sparse_transformers/csrc/approx_topk.h:10-88)."""
-    s = _f32(scores)
+    """Per-row sketch threshold [B] (sparse_transformers/csrc/approx_topk.h:10-88).  float64 scores give a float64
+    threshold (the reference dispatches on the scores' type), anything else is evaluated in float32."""
+    f64 = isinstance(scores, np.ndarray) and scores.dtype == np.float64
+    s = np.ascontiguousarray(scores, dtype=np.float64) if f64 else _f32(scores)
     if s.ndim != 2:
         raise ValueError("Input scores must be 2D tensor [batch_size, features]")
     if k <= 0:
@@ -196,8 +199,9 @@ def approx_topk_threshold(scores, k) -> np.ndarray:
         raise ValueError("k cannot be larger than feature size")
     if s.shape[1] < 4:
         raise ValueError("feature size below 4: the reference divides by a sketch width of zero")
-    thr = np.empty(s.shape[0], dtype=np.float32)
-    lib().orc_approx_topk_threshold(_p(s), s.shape[0], s.shape[1], int(k), _p(thr))
+    thr = np.empty(s.shape[0], dtype=s.dtype)
+    fn = lib().orc_approx_topk_threshold_f64 if f64 else lib().orc_approx_topk_threshold
+    fn(_p(s), s.shape[0], s.shape[1], int(k), _p(thr))
     return thr
 
 

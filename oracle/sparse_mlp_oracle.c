@@ -396,3 +396,36 @@ void orc_approx_topk_threshold(const float *scores, int64_t B, int64_t F, int64_
     }
     free(cell);
 }
+
+/* The same for double scores (the reference dispatches on every floating type, approx_topk.h:33); its
+ * adjustment factor is then the double 0.9. */
+static int cmp_double_desc(const void *a, const void *b)
+{
+    const double x = *(const double *)a, y = *(const double *)b;
+    return (x < y) - (x > y);
+}
+
+void orc_approx_topk_threshold_f64(const double *scores, int64_t B, int64_t F, int64_t k, double *threshold)
+{
+    const int64_t W = F / 4 < 1024 ? F / 4 : 1024;
+    double *cell = (double *)malloc((size_t)(4 * W) * sizeof(double));
+    for (int64_t b = 0; b < B; ++b) {
+        const double *s = scores + b * F;
+        for (int64_t i = 0; i < 4 * W; ++i) cell[i] = -INFINITY;
+        for (int64_t t = 0; t < 4; ++t)
+            for (int64_t f = 0; f < F; ++f) {
+                double *c = cell + t * W + (t * F + f) % W;
+                if (s[f] > *c) *c = s[f];
+            }
+        int64_t cells = 0;
+        for (int64_t i = 0; i < 4 * W; ++i)
+            if (cell[i] != -INFINITY) cell[cells++] = cell[i];
+        if (cells == 0) { threshold[b] = 0.0; continue; }
+        int64_t sk = k * cells / F;
+        if (sk < 1) sk = 1;
+        if (sk > cells) sk = cells;
+        qsort(cell, (size_t)cells, sizeof(double), cmp_double_desc);
+        threshold[b] = cell[sk - 1] * 0.9;
+    }
+    free(cell);
+}

@@ -46,6 +46,7 @@ SIGNATURES = {
     "st_mask_select_workspace_bytes": (_i64, [_i64, _i64]),
     "st_mask_select": (_ci, [_vp, _i64, _i64, _ci, _i64, _f, _vp, _vp, _vp, _i64, _vp]),
     "st_approx_topk_threshold": (_ci, [_vp, _i64, _i64, _i64, _vp, _vp]),
+    "st_approx_topk_threshold_f64": (_ci, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "st_cache_max_intermediate": (_i64, []),
     "st_cache_create": (_vp, [C.POINTER(CacheBuffers), _i64, _i64, _ci, _ci]),
     "st_cache_destroy": (None, [_vp]),

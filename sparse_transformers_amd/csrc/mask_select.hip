@@ -350,6 +350,74 @@ __global__ __launch_bounds__(kSelThreads) void approx_topk_kernel(const float *_
     if (tid == 0) threshold[b] = key_value(kth) * 0.9f;
 }
 
+// The same for double scores (the reference dispatches on every floating type, approx_topk.h:33).  Cells are 64-bit
+// order-preserving keys; the k-th largest is found by the 32-bit radix select twice: on the upper halves, then --
+// among the keys that share the winning upper half -- on the lower halves.
+__device__ __forceinline__ unsigned long long order_key64(double v)
+{
+    unsigned long long u = (unsigned long long)__double_as_longlong(v);
+    if (u == 0x8000000000000000ull) u = 0ull;
+    return (u >> 63) ? ~u : (u | 0x8000000000000000ull);
+}
+__device__ __forceinline__ double key_value64(unsigned long long k)
+{
+    return __longlong_as_double((long long)((k >> 63) ? (k & 0x7fffffffffffffffull) : ~k));
+}
+
+__global__ __launch_bounds__(kSelThreads) void approx_topk_f64_kernel(const double *__restrict__ scores, int F, long k,
+                                                                     int W, double *__restrict__ threshold)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ SelShared sh;
+    unsigned long long *cell = reinterpret_cast<unsigned long long *>(smem);  // [4][W], W <= 1024
+    const int tid = threadIdx.x, b = blockIdx.x;
+    const double *row = scores + (size_t)b * F;
+    const unsigned long long kNegInf = order_key64(-__builtin_inf());
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (tid + u * kSelThreads < 4 * W) cell[tid + u * kSelThreads] = kNegInf;
+    __syncthreads();
+    for (int f = tid; f < F; f += kSelThreads) {
+        const unsigned long long kv = order_key64(row[f]);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) atomicMax(&cell[s * W + (int)(((long)s * F + f) % W)], kv);
+    }
+    __syncthreads();
+    unsigned long long kr[4];
+    int filled = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int i = tid + u * kSelThreads;
+        kr[u] = i < 4 * W ? cell[i] : kNegInf;
+        filled += kr[u] != kNegInf;
+    }
+    const long cells = (long)(block_sum((double)filled, sh, tid) + 0.5);
+    if (cells == 0) {
+        if (tid == 0) threshold[b] = 0.0;
+        return;
+    }
+    long sk = k * cells / F;
+    if (sk < 1) sk = 1;
+    if (sk > cells) sk = cells;
+    // (empty cells hold the key of -inf, the smallest there is: they never reach the sk <= cells largest)
+    uint32_t rem, cnt;
+    auto sweep_hi = [&](auto &&fn) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (tid + u * kSelThreads < 4 * W) fn((uint32_t)(kr[u] >> 32));
+    };
+    const uint32_t hi = radix_select_desc(sweep_hi, (uint32_t)sk, sh, tid, rem, cnt);
+    const uint32_t want = rem;   // the rem-th largest lower half among the keys whose upper half is `hi`
+    __syncthreads();
+    auto sweep_lo = [&](auto &&fn) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (tid + u * kSelThreads < 4 * W && (uint32_t)(kr[u] >> 32) == hi) fn((uint32_t)kr[u]);
+    };
+    const uint32_t lo = radix_select_desc(sweep_lo, want, sh, tid, rem, cnt);
+    if (tid == 0) threshold[b] = key_value64(((unsigned long long)hi << 32) | lo) * 0.9;
+}
+
 }  // namespace st
 
 extern "C" int64_t st_mask_select_workspace_bytes(int64_t B, int64_t I)
@@ -415,6 +483,25 @@ extern "C" int st_approx_topk_threshold(const float *scores, int64_t B, int64_t 
     ProfScope ps(ST_K_MASK_SELECT, s);
     ST_LAUNCH(ps, approx_topk_kernel, dim3((unsigned)B), dim3(kSelThreads), (size_t)4 * W * 4, s, scores, (int)F, (long)k,
               W, threshold);
+    ST_HIP(hipGetLastError());
+    return ST_OK;
+}
+
+extern "C" int st_approx_topk_threshold_f64(const double *scores, int64_t B, int64_t F, int64_t k, double *threshold,
+                                            void *stream)
+{
+    using namespace st;
+    ST_REQUIRE(scores && threshold, "st_approx_topk_threshold_f64: null pointer");
+    ST_REQUIRE(B >= 1 && B <= 65535, "st_approx_topk_threshold_f64: B=%lld out of range", (long long)B);
+    ST_REQUIRE(F >= 4 && F <= (1 << 24), "st_approx_topk_threshold_f64: feature size %lld out of range [4, 2^24]",
+               (long long)F);
+    ST_REQUIRE(k > 0, "st_approx_topk_threshold_f64: k must be positive");
+    ST_REQUIRE(k <= F, "st_approx_topk_threshold_f64: k cannot be larger than feature size");
+    const int W = (int)(F / 4 < 1024 ? F / 4 : 1024);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    ProfScope ps(ST_K_MASK_SELECT, s);
+    ST_LAUNCH(ps, approx_topk_f64_kernel, dim3((unsigned)B), dim3(kSelThreads), (size_t)4 * W * 8, s, scores, (int)F,
+              (long)k, W, threshold);
     ST_HIP(hipGetLastError());
     return ST_OK;
 }

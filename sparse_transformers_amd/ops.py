@@ -327,19 +327,21 @@ def mask_select(scores: torch.Tensor, method: str, k: int = 0, std_multiplier: f
 
 def approx_topk_threshold(scores: torch.Tensor, k: int) -> torch.Tensor:
     """Per-row approximate top-k threshold [B, 1] from four max-sketches
-    (sparse_transformers/csrc/approx_topk.h:10-88).  ``scores`` is a float32 [B, F] GPU tensor."""
+    (sparse_transformers/csrc/approx_topk.h:10-88).  ``scores`` is a float32 or float64 [B, F] GPU tensor; the
+    threshold has its dtype (the reference dispatches on the scores' type, :33)."""
     dev = require_gpu(scores)
     if scores.dim() != 2:
         raise RuntimeError("Input scores must be 2D tensor [batch_size, features]")
-    if scores.dtype != torch.float32:
-        raise TypeError("approx_topk_threshold: scores must be float32")
+    if scores.dtype not in (torch.float32, torch.float64):
+        raise TypeError("approx_topk_threshold: scores must be float32 or float64")
     if k <= 0:
         raise RuntimeError("k must be positive")
     if k > scores.size(1):
         raise RuntimeError("k cannot be larger than feature size")
     scores = scores if scores.is_contiguous() else scores.contiguous()
     B, F = scores.shape
-    thr = torch.empty(B, 1, dtype=torch.float32, device=dev)
-    rc = _lib.lib().st_approx_topk_threshold(scores.data_ptr(), B, F, int(k), thr.data_ptr(), current_stream_ptr(dev))
+    thr = torch.empty(B, 1, dtype=scores.dtype, device=dev)
+    fn = _lib.lib().st_approx_topk_threshold if scores.dtype == torch.float32 else _lib.lib().st_approx_topk_threshold_f64
+    rc = fn(scores.data_ptr(), B, F, int(k), thr.data_ptr(), current_stream_ptr(dev))
     _lib.check(rc, "st_approx_topk_threshold")
     return thr

@@ -13,6 +13,8 @@ produced by compiling its sources (sparse_transformers/csrc/sparse_mlp_op.cpp + 
   approx_topk.json    fp32 score rows and the thresholds torch.ops.sparse_mlp.approx_topk_threshold
                       returns for them (approx_topk.h:10-88), incl. feature sizes that are not
                       multiples of the sketch width, repeated values and -inf scores
+  approx_topk_f64.json the same operator on float64 scores (it dispatches on the scores' type), incl. values that
+                      agree in the upper half of their bits
 
 Run from the repository root in a container that has /root/reference:  python tests/golden/make_golden.py
 """
@@ -142,6 +144,27 @@ def main():
     with open(os.path.join(HERE, "approx_topk.json"), "w") as f:
         json.dump({"source": "torch.ops.sparse_mlp.approx_topk_threshold compiled from sparse_transformers/csrc",
                    "cases": acases}, f, separators=(",", ":"))
+    # the same operator on double scores (it dispatches on the scores' type, approx_topk.h:33)
+    dcases = []
+    g = torch.Generator().manual_seed(10)
+    for (B, F, k, kind) in [(2, 16, 4, "normal"), (3, 37, 5, "normal"), (1, 257, 30, "coarse"), (2, 96, 20, "neginf"),
+                            (1, 1500, 200, "close"), (1, 2051, 513, "coarse")]:
+        sc = torch.randn(B, F, generator=g, dtype=torch.float64)
+        if kind == "coarse":
+            sc = (sc * 4).round() / 4
+        elif kind == "neginf":
+            sc[:, ::2] = float("-inf")
+            sc[1] = float("-inf")
+        elif kind == "close":      # values that differ only far down the mantissa: equal upper key halves
+            sc = 1.0 + sc * 1e-12
+        thr = approx(sc, k)
+        assert thr.dtype == torch.float64
+        dcases.append({"B": B, "F": F, "k": k,
+                       "scores_f64_b64": base64.b64encode(sc.numpy().astype("<f8").tobytes()).decode("ascii"),
+                       "threshold_f64_b64": base64.b64encode(thr.numpy().astype("<f8").tobytes()).decode("ascii")})
+    with open(os.path.join(HERE, "approx_topk_f64.json"), "w") as f:
+        json.dump({"source": "torch.ops.sparse_mlp.approx_topk_threshold on float64 scores, compiled from "
+                             "sparse_transformers/csrc", "cases": dcases}, f, separators=(",", ":"))
     print("wrote", os.listdir(HERE))
 
 

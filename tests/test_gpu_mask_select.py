@@ -146,6 +146,32 @@ def test_approx_topk_bit_exact(B, F, kind):
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), k
 
 
+def test_approx_topk_f64_reference_vectors_and_oracle():
+    """Double scores (the reference dispatches on the type, approx_topk.h:33): bit-equal to the vectors written from
+    the compiled reference and to the oracle, incl. values whose bit patterns agree in their upper halves."""
+    import base64
+    with open(os.path.join(os.path.dirname(__file__), "golden", "approx_topk_f64.json")) as f:
+        cases = json.load(f)["cases"]
+    for c in cases:
+        sc = np.frombuffer(base64.b64decode(c["scores_f64_b64"]), dtype="<f8").copy().reshape(c["B"], c["F"])
+        want = np.frombuffer(base64.b64decode(c["threshold_f64_b64"]), dtype="<f8")
+        got = st.approx_topk_threshold(torch.from_numpy(sc).to(DEV), c["k"])
+        assert got.dtype == torch.float64 and tuple(got.shape) == (c["B"], 1)
+        assert np.array_equal(got.cpu().numpy().reshape(-1), want), (c["B"], c["F"], c["k"])
+    rng = np.random.default_rng(8)
+    for F in (4, 100, 4096, 14336):
+        for kind in ("normal", "close", "ties"):
+            s = rng.standard_normal((3, F))
+            if kind == "close":
+                s = -3.0 + s * 1e-13
+            elif kind == "ties":
+                s = np.round(s * 2) / 2
+            for k in sorted({1, max(1, F // 9), F}):
+                want = oracle.approx_topk_threshold(s, k)
+                got = st.approx_topk_threshold(torch.from_numpy(s).to(DEV), k).cpu().numpy().reshape(-1)
+                assert np.array_equal(got, want), (F, kind, k)
+
+
 def test_approx_topk_errors():
     s = torch.zeros(2, 64, device=DEV)
     for bad in (lambda: st.approx_topk_threshold(s, 0), lambda: st.approx_topk_threshold(s, 65),

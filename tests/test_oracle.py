@@ -272,6 +272,36 @@ def test_approx_topk_against_compiled_reference_random():
                 assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (F, B, k)
 
 
+def test_approx_topk_f64_matches_reference_vectors_and_live_reference():
+    """The reference dispatches approx_topk_threshold on the scores' floating type (approx_topk.h:33): double scores
+    against the vectors written from the compiled reference, and against that build itself where it is present."""
+    import base64
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(__file__), "golden", "approx_topk_f64.json")) as f:
+        cases = json.load(f)["cases"]
+    assert len(cases) >= 6
+    for c in cases:
+        sc = np.frombuffer(base64.b64decode(c["scores_f64_b64"]), dtype="<f8").copy().reshape(c["B"], c["F"])
+        want = np.frombuffer(base64.b64decode(c["threshold_f64_b64"]), dtype="<f8")
+        got = oracle.approx_topk_threshold(sc, c["k"])
+        assert got.dtype == np.float64 and np.array_equal(got, want), (c["B"], c["F"], c["k"])
+    if oracle.load_reference() is None:
+        return
+    import torch
+
+    op = torch.ops.sparse_mlp.approx_topk_threshold
+    rng = np.random.default_rng(22)
+    for F in (4, 63, 1000, 4097, 11008):
+        sc = rng.standard_normal((2, F))
+        if F % 2:
+            sc = 1.0 + sc * 1e-13              # equal upper halves of the bit patterns
+        for k in sorted({1, max(1, F // 7), F}):
+            want = op(torch.from_numpy(sc), k).numpy().reshape(-1)
+            assert np.array_equal(oracle.approx_topk_threshold(sc, k), want), (F, k)
+
+
 def test_approx_topk_special_cases():
     # F a multiple of the sketch width: all four sketches equal the per-residue maxima, so with k = F the
     # threshold is 0.9 * the smallest of those maxima
