@@ -27,10 +27,51 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each scaled by
-# what the same counter reads for a 256 MiB copy; see profiles/decode_traffic_llama3b_stack_fp16.md
-MEASURED_TRAFFIC_BYTES = {("llama3b_stack_fp16", "mlp_decode"): 53_169_357 + 3_145_728,
-                          ("llama3b_stack_fp16", "cache_update_decode"): 56_787_558 + 8_574_259}
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic.md")
+
+
+def csrc_hash() -> str:
+    """sha256 over the HIP sources the library is built from (first 16 hex digits), or "" when they are not there."""
+    import glob
+    import hashlib
+    files = sorted(glob.glob(os.path.join(ROOT, "sparse_transformers_amd", "csrc", "*")))
+    if not files:
+        return ""
+    h = hashlib.sha256()
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload: str, kernel_kind: str, batch: int):
+    """HBM bytes per launch of a workload's dominant kernel as rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE counted them,
+    from the table rows of profiles/hbm_traffic.md:
+        | workload | batch | kernel kind | kernel | csrc hash | fetched bytes | written bytes |
+    A row only counts while the sources it was measured on are the ones in this tree (same hash): otherwise the
+    figure would silently describe another kernel.  Returns (bytes or None, where the figure comes from / why not)."""
+    have = csrc_hash()
+    if not os.path.exists(TRAFFIC_TABLE):
+        return None, "profiles/hbm_traffic.md not found"
+    stale = None
+    with open(TRAFFIC_TABLE) as f:
+        for line in f:
+            cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
+            if len(cells) != 7 or cells[0] != workload or cells[2] != kernel_kind:
+                continue
+            try:
+                b, fetched, written = int(cells[1]), int(cells[5].replace(" ", "")), int(cells[6].replace(" ", ""))
+            except ValueError:
+                continue
+            if b != batch:
+                continue
+            if cells[4] == have and have:
+                return fetched + written, f"profiles/hbm_traffic.md ({cells[3]}, csrc {have}): FETCH_SIZE {fetched} + WRITE_SIZE {written}"
+            stale = cells[4]
+    if stale is not None:
+        return None, f"profiles/hbm_traffic.md was measured on csrc {stale}, this tree is {have or 'without sources'}"
+    return None, f"no row for {workload} batch {batch} {kernel_kind} in profiles/hbm_traffic.md"
 
 
 def parse_args():
@@ -47,6 +88,8 @@ def parse_args():
     ap.add_argument("--no-fused", action="store_true",
                     help="cache update and MLP as two kernels per layer instead of the fused update+decode kernel")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-prefill-probe", action="store_true",
+                    help="skip the short 512-row MFMA pass whose figures the decode line carries as `prefill_512`")
     ap.add_argument("--cpu-layers", type=int, default=4)
     ap.add_argument("--cpu-steps", type=int, default=300)
     ap.add_argument("--profile-steps", type=int, default=32)
@@ -65,22 +108,20 @@ def parse_args():
 MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 / bf16
 
 
-def prefill_bench(args, wl, torch, st, _lib, syn):
-    """One step = `--prefill` rows of x through the sparse MLP of every layer, the caches holding the union of the
-    rows' masks (per-row masks of the workload's active fraction that share 60 % of their indices)."""
+def prefill_measure(stack, wl, T, layers, K, W, profile_steps, seed, torch, _lib, syn):
+    """`T` rows of x through the sparse MLP of the first `layers` layers of `stack`, each cache at the union of the
+    rows' masks (per-row masks of the workload's active fraction that share 60 % of their indices): tok/s, the kernels'
+    event times and the gate/up kernel against the dense MFMA peak."""
     import ctypes as C
     dev = torch.device("cuda:0")
     dt = getattr(torch, wl.dtype)
-    if wl.dtype == "float32":
-        print("bench.py: --prefill needs an fp16 / bf16 workload (the MFMA kernels)", file=sys.stderr)
-        sys.exit(2)
-    T, H, I = args.prefill, wl.hidden, wl.intermediate
-    layers = args.layers or min(wl.layers, 8)
-    K, W = args.steps, args.warmup
-    stack, g = build_stack(wl, layers, 1, args.seed, torch, st)
+    H, I = wl.hidden, wl.intermediate
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed + 101)
+    sub = stack.layers[:layers]
     ns = []
-    for l, layer in enumerate(stack.layers):
-        union = syn.overlapping_token_masks(args.seed + 11 + l, I, T, wl.n_active, 0.6).any(axis=0)
+    for l, layer in enumerate(sub):
+        union = syn.overlapping_token_masks(seed + 11 + l, I, T, wl.n_active, 0.6).any(axis=0)
         layer.cache.update_active_weights(torch.from_numpy(union).to(dev))
         ns.append(int(union.sum()))
     x0 = torch.randn(T, H, generator=g, device=dev, dtype=torch.float32).to(dt)
@@ -88,7 +129,7 @@ def prefill_bench(args, wl, torch, st, _lib, syn):
 
     def step():
         x = x0
-        for l, layer in enumerate(stack.layers):
+        for l, layer in enumerate(sub):
             x = layer.cache.forward(x, wl.act, out=bufs[l & 1])
         return x
 
@@ -106,7 +147,7 @@ def prefill_bench(args, wl, torch, st, _lib, syn):
     cap = 8 * layers
     kinds, ms = (C.c_int * cap)(), (C.c_float * cap)()
     per = {}
-    for _ in range(max(4, args.profile_steps // 4)):
+    for _ in range(max(4, profile_steps // 4)):
         _lib.check(L.st_profile_enable(cap), "st_profile_enable")
         step()
         torch.cuda.synchronize()
@@ -122,18 +163,33 @@ def prefill_bench(args, wl, torch, st, _lib, syn):
     gu_flops = 2.0 * (c - 1) * T * n_mean * H
     gu_us = kern["mlp_prefill_gateup"]["mean_us"]
     achieved = gu_flops / (gu_us * 1e-6) / 1e12
+    return {"ms_per_step": ms_per_step, "kernels_us": kern, "n_mean": n_mean, "flops_layer": flops_layer,
+            "gu_flops": gu_flops, "gu_us": gu_us, "achieved_tflops": achieved, "layers": layers,
+            "stack_tflops": layers * flops_layer / (ms_per_step * 1e-3) / 1e12}
+
+
+def prefill_bench(args, wl, torch, st, _lib, syn):
+    """One step = `--prefill` rows of x through the sparse MLP of every layer (see prefill_measure)."""
+    if wl.dtype == "float32":
+        print("bench.py: --prefill needs an fp16 / bf16 workload (the MFMA kernels)", file=sys.stderr)
+        sys.exit(2)
+    T, H, I = args.prefill, wl.hidden, wl.intermediate
+    layers = args.layers or min(wl.layers, 8)
+    K, W = args.steps, args.warmup
+    stack, _ = build_stack(wl, layers, 1, args.seed, torch, st)
+    m = prefill_measure(stack, wl, T, layers, K, W, args.profile_steps, args.seed, torch, _lib, syn)
     out = {
-        "metric": "sparse_mlp_prefill_tokens_per_s", "value": round(T / (ms_per_step * 1e-3), 1), "unit": "tok/s",
-        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "metric": "sparse_mlp_prefill_tokens_per_s", "value": round(T / (m["ms_per_step"] * 1e-3), 1), "unit": "tok/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(m["ms_per_step"], 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": {"float16": "f16", "bfloat16": "bf16"}[wl.dtype],
         "data": "synthetic (seeded weights, inputs and per-row masks; caches at the union of the rows' masks)",
         "config": {"workload": wl.name + "_prefill", "layers": layers, "hidden": H, "intermediate": I, "rows": T,
-                   "active_rows_mean": n_mean, "act": wl.act, "has_gate": wl.has_gate},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": None, "kernel": "prefill_gateup_kernel",
-                     "flops_per_launch": gu_flops, "mean_us": gu_us},
-        "stack_tflops": round(layers * flops_layer / (ms_per_step * 1e-3) / 1e12, 1),
-        "kernels_us": kern,
+                   "active_rows_mean": m["n_mean"], "act": wl.act, "has_gate": wl.has_gate},
+        "roofline": {"bound": "mfma", "achieved": round(m["achieved_tflops"], 1), "peak": MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(m["achieved_tflops"] / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "prefill_gateup_kernel", "flops_per_launch": m["gu_flops"], "mean_us": m["gu_us"]},
+        "stack_tflops": round(m["stack_tflops"], 1),
+        "kernels_us": m["kernels_us"],
     }
     print(json.dumps(out))
 
@@ -166,39 +222,42 @@ def build_stack(wl, layers, batch, seed, torch, st):
     return st.SparseMLPStack(stack_layers), g
 
 
-def cpu_baseline(wl, layers, steps, seed, torch):
-    """The same path on the host: the reference's own C++ WeightCache (compiled into oracle/_ref) when
-    it loads, else the C oracle; predictor and MLP as the torch-CPU calls of src/modeling_skip.py
-    (fp32, as the reference cache is fp32 only).  Returns tok/s scaled to the full stack depth."""
+def cpu_baseline(wl, stack, trace, x_in, x_pred, layers, steps, torch):
+    """The same path on the host, on the GPU run's own inputs: the first `layers` layers' weights are read back from
+    the GPU caches and predictors, the masks are the first steps of the GPU run's trace and x / the predictor inputs
+    are the ones the GPU steps saw.  Cache = the reference's own C++ WeightCache (compiled into oracle/_ref) when it
+    loads, else the C oracle; predictor and MLP as the torch-CPU calls of src/modeling_skip.py (fp32, as the
+    reference cache is fp32 only).  Returns tok/s scaled to the full stack depth."""
     import oracle
-    from sparse_transformers_amd import synthetic as syn
 
     ref = oracle.load_reference()
     kind = "reference" if ref else "port"
-    H, I, r = wl.hidden, wl.intermediate, wl.rank
-    rng = np.random.default_rng(seed)
-    trace = syn.mask_trace(seed + 1, layers, I, wl.n_active, steps + 4, wl.churn_lo, wl.churn_hi)
+    H = wl.hidden
+    steps = min(steps, trace.shape[0] - 1)
+    tr = trace[:steps + 1, :layers].cpu().numpy()
+    xs = x_in[:steps + 1].float().cpu()
+    xps = x_pred[:steps + 1, :layers].float().cpu()
     act = {"silu": torch.nn.functional.silu, "relu": torch.relu}[wl.act]
     built = []
     for l in range(layers):
-        w = syn.layer_weights(rng, H, I, r, has_gate=wl.has_gate)
-        up, down = torch.from_numpy(w["up"]), torch.from_numpy(w["down"])
-        gate = torch.from_numpy(w["gate"]) if wl.has_gate else None
-        A, Bm = torch.from_numpy(w["A"]), torch.from_numpy(w["Bm"])
-        m0 = torch.from_numpy(trace[0, l])
+        c, p = stack.layers[l].cache, stack.layers[l].predictor
+        up, down = c.up_pool.float().cpu(), c.downT_pool.float().cpu().t().contiguous()
+        gate = c.gate_pool.float().cpu() if wl.has_gate else None
+        A, Bm = p.down_weight.float().cpu(), p.up_weight.float().cpu()
         if ref:
-            cache = ref[0](m0, H, gate, up, down, wl.has_gate)
+            cache = ref[0](torch.from_numpy(tr[0, l]), H, gate, up, down, wl.has_gate)
         else:
-            cache = oracle.OracleWeightCache(trace[0, l], H, w["gate"], w["up"], w["down"], wl.has_gate)
+            cache = oracle.OracleWeightCache(tr[0, l], H, gate.numpy() if wl.has_gate else None, up.numpy(), down.numpy(),
+                                             wl.has_gate)
         built.append((cache, A, Bm))
-    x = torch.randn(wl.batch, H)
     times = []
-    for t in range(1, steps + 4):
+    for t in range(1, steps + 1):
+        x = xs[t]
         t0 = time.perf_counter()
         for l, (cache, A, Bm) in enumerate(built):
-            scores = (x @ A.t()) @ Bm.t()
+            scores = (xps[t, l] @ A.t()) @ Bm.t()
             _ = (scores >= 0).any(dim=0)                    # predictor + naive mask + union
-            m = trace[t, l]
+            m = tr[t, l]
             if ref:
                 cache.update_active_weights(torch.from_numpy(m))
                 cw, dw = cache.get_concat_weight(), cache.get_active_down_weight()
@@ -207,16 +266,16 @@ def cpu_baseline(wl, layers, steps, seed, torch):
                 cw, dw = torch.from_numpy(cache.get_concat_weight()), torch.from_numpy(cache.get_active_down_weight())
             if wl.has_gate:
                 gt, u = x.matmul(cw.t()).chunk(2, dim=-1)
-                y = (act(gt) * u).matmul(dw.t())
+                x = (act(gt) * u).matmul(dw.t())
             else:
-                y = act(x.matmul(cw.t())).matmul(dw.t())
+                x = act(x.matmul(cw.t())).matmul(dw.t())
         times.append(time.perf_counter() - t0)
-    per_layer_step = float(np.median(times[4:])) / layers
-    tok_s = wl.batch / (per_layer_step * wl.layers)
+    per_layer_step = float(np.median(times[min(4, len(times) - 1):])) / layers
+    tok_s = xs.shape[1] / (per_layer_step * wl.layers)
     return {
         "value": round(tok_s, 3), "unit": "tok/s", "cores": int(torch.get_num_threads()), "kind": kind,
-        "sample": f"{layers} of {wl.layers} layers x {steps} steps, fp32, median per-layer time scaled to "
-                  f"{wl.layers} layers; cache update = "
+        "sample": f"the first {layers} of {wl.layers} layers x the first {steps} steps of the GPU run's own weights, "
+                  f"mask trace and inputs, fp32, median per-layer time scaled to {wl.layers} layers; cache update = "
                   + ("reference WeightCache compiled from its own sources" if ref else "C restatement")
                   + ", predictor/MLP = torch CPU matmul path",
         "ms_per_layer_step": round(per_layer_step * 1e3, 3),
@@ -411,6 +470,7 @@ def main():
     achieved = launch_bytes / (mlp_us * 1e-6) / 1e9
     upd_us = (unfused or per_kernel).get("cache_update", {}).get("mean_us")
 
+    traffic, traffic_src = measured_traffic(wl.name, dom, B)
     churn_mean = 0.5 * (wl.churn_lo + wl.churn_hi)
     result = {
         "metric": "sparse-MLP decode tok/s", "value": round(tok_s, 2), "unit": "tok/s",
@@ -425,8 +485,10 @@ def main():
                    "kernel_timing": "hip events stamped at kernel begin/end (hipExtLaunchKernelGGL), eager second pass"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((wl.name, dom)) if B == wl.batch else None,
-                     "kernel": dom + "_kernel", "bytes_per_launch": launch_bytes, "mean_us": mlp_us,
+                     "traffic": traffic, "traffic_source": traffic_src,
+                     "kernel": {"cache_update_decode": "cache_sparse_decode_kernel", "mlp_decode": "mlp_decode_kernel",
+                                "mlp_batch_gateup": "batch_gateup_kernel + batch_down_kernel"}[dom],
+                     "bytes_per_launch": launch_bytes, "mean_us": mlp_us,
                      "bytes_mlp": alg_bytes, "bytes_cache_update": upd_bytes if dom == "cache_update_decode" else 0,
                      "frac_mlp_bytes_only": round(alg_bytes / (mlp_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)},
         "cache_update_us_per_layer": upd_us,
@@ -440,10 +502,25 @@ def main():
         "kernels_us_unfused": unfused,
         "churn_mean": churn_mean,
     }
+    if not args.no_prefill_probe and wl.dtype != "float32" and B == 1:
+        # the MFMA path in the same line: 512 rows of x through the first layers' sparse MLPs (caches at the union of
+        # the rows' masks).  Runs last: it moves those caches away from the decode trace.
+        try:
+            pl = max(1, min(8, layers))
+            m = prefill_measure(stack, wl, 512, pl, 6, 2, 8, args.seed, torch, _lib, syn)
+            result["prefill_512"] = {
+                "layers": pl, "rows": 512, "active_rows_mean": m["n_mean"], "tok_s": round(512 / (m["ms_per_step"] * 1e-3), 1),
+                "us_per_layer": round(m["ms_per_step"] * 1e3 / pl, 2), "stack_tflops": round(m["stack_tflops"], 1),
+                "roofline": {"bound": "mfma", "kernel": "prefill_gateup_kernel", "achieved": round(m["achieved_tflops"], 1),
+                             "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                             "frac": round(m["achieved_tflops"] / MFMA_PEAK_TFLOPS, 4), "mean_us": m["gu_us"]},
+                "kernels_us": m["kernels_us"]}
+        except Exception as exc:
+            result["prefill_512"] = {"error": repr(exc)}
     if not args.no_cpu_baseline:
         try:
-            result["cpu_baseline"] = cpu_baseline(wl, max(1, min(args.cpu_layers, layers)), args.cpu_steps,
-                                                  args.seed, torch)
+            result["cpu_baseline"] = cpu_baseline(wl, stack, trace, x_in, x_pred, max(1, min(args.cpu_layers, layers)),
+                                                  args.cpu_steps, torch)
         except Exception as exc:  # the baseline is reported, never required for the GPU numbers
             result["cpu_baseline"] = {"value": None, "unit": "tok/s", "cores": 0, "kind": "port",
                                       "sample": f"failed: {exc!r}"}
