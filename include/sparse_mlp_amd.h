@@ -118,6 +118,14 @@ int st_mlp_forward_static(const void *x, int64_t B, int64_t H, const void *gate_
  * ------------------------------------------------------------------------ */
 int st_predictor_mask(const void *x, int64_t B, int64_t H, const void *A, int64_t r, const void *Bm, int64_t I,
                       int dtype, float thr, int cmp_ge, float *t_ws, float *scores, uint8_t *mask, void *stream);
+/* The same with flags.  ST_PRED_ROUND_STORAGE: the rank-r intermediate and the scores are rounded to `dtype` before
+ * they are used, which is what FastLoRAProjection computes when the model runs in fp16 / bf16 (up(down(x)) as two
+ * modules in the model's type, src/modeling_skip.py:52-53): scores close to the cut then fall on the side the
+ * reference's own arithmetic puts them.  Without it both stay in fp32 (st_predictor_mask).  No effect for ST_F32. */
+enum st_predictor_flags { ST_PRED_ROUND_STORAGE = 1 };
+int st_predictor_mask_ex(const void *x, int64_t B, int64_t H, const void *A, int64_t r, const void *Bm, int64_t I,
+                         int dtype, float thr, int cmp_ge, int flags, float *t_ws, float *scores, uint8_t *mask,
+                         void *stream);
 
 /* ------------------------------------------------------------------------
  * Mask methods that need a statistic of the whole score row, then the union

@@ -153,7 +153,28 @@ def mlp_forward(x, concat_weight, active_down_weight, act="silu", has_gate=True)
     return out.reshape(np.asarray(x).shape), comb
 
 
-def predictor_scores(x, A, Bm) -> np.ndarray:
+def _round_storage(a: np.ndarray, storage: str) -> np.ndarray:
+    """float32 -> nearest value of the storage type (round to nearest even) -> float32."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    if storage == "float16":
+        return a.astype(np.float16).astype(np.float32)
+    if storage == "bfloat16":
+        u = a.view(np.uint32).astype(np.uint64)
+        r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+        out = (r & 0xFFFFFFFF).astype(np.uint32).view(np.float32).copy()
+        out[np.isnan(a)] = np.nan
+        return out
+    raise ValueError(f"unknown storage type {storage!r}")
+
+
+def predictor_scores(x, A, Bm, storage=None) -> np.ndarray:
+    """scores = (x @ A^T) @ Bm^T (src/modeling_skip.py:52-53).  ``storage`` ("float16" / "bfloat16"): the two maps as
+    modules of a half-precision model compute them -- each output rounded to the storage type (products summed in
+    higher precision first, as the BLAS kernels do)."""
+    if storage in ("float16", "bfloat16"):
+        x2 = np.asarray(x, dtype=np.float64).reshape(-1, np.asarray(x).shape[-1])
+        t = _round_storage((x2 @ np.asarray(A, dtype=np.float64).T).astype(np.float32), storage)
+        return _round_storage((t.astype(np.float64) @ np.asarray(Bm, dtype=np.float64).T).astype(np.float32), storage)
     x2 = _f32(x).reshape(-1, np.asarray(x).shape[-1])
     A, Bm = _f32(A), _f32(Bm)
     B, H = x2.shape

@@ -43,6 +43,7 @@ SIGNATURES = {
     "st_mlp_static_scratch_bytes": (_i64, []),
     "st_mlp_forward_static": (_ci, [_vp, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _ci, _ci, _ci, _vp]),
     "st_predictor_mask": (_ci, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _ci, _f, _ci, _vp, _vp, _vp, _vp]),
+    "st_predictor_mask_ex": (_ci, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _ci, _f, _ci, _ci, _vp, _vp, _vp, _vp]),
     "st_mask_select_workspace_bytes": (_i64, [_i64, _i64]),
     "st_mask_select": (_ci, [_vp, _i64, _i64, _ci, _i64, _f, _vp, _vp, _vp, _i64, _vp]),
     "st_approx_topk_threshold": (_ci, [_vp, _i64, _i64, _i64, _vp, _vp]),

@@ -21,7 +21,7 @@ constexpr int kPredDownUnroll = 2;  // chunks per thread issued together
 template <typename T, int BT>
 __global__ __launch_bounds__(kPredDownThreads) void predictor_down_kernel(const T *__restrict__ x, int B, int H,
                                                                           const T *__restrict__ A, int r,
-                                                                          float *__restrict__ t)
+                                                                          float *__restrict__ t, int round_storage)
 {
     constexpr int VEC = Elem<T>::kVec;
     __shared__ float red[kPredDownThreads / kWave][BT];
@@ -74,7 +74,8 @@ __global__ __launch_bounds__(kPredDownThreads) void predictor_down_kernel(const 
             float s = 0.f;
 #pragma unroll
             for (int w2 = 0; w2 < kPredDownThreads / kWave; ++w2) s += red[w2][tid];
-            t[(size_t)(b0 + tid) * r + k] = s;
+            // (round_storage: the rank-r intermediate as a module in the storage type would hand it on)
+            t[(size_t)(b0 + tid) * r + k] = round_storage ? to_float<T>(from_float<T>(s)) : s;
         }
         __syncthreads();
     }
@@ -94,7 +95,7 @@ template <typename T, int LPR, int RPW>
 __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_kernel(const float *__restrict__ t, int B, int r,
                                                                   const T *__restrict__ Bm, int I, float thr,
                                                                   int cmp_ge, float *__restrict__ scores,
-                                                                  uint8_t *__restrict__ mask)
+                                                                  uint8_t *__restrict__ mask, int round_storage)
 {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int RPI = kWave / LPR;                                          // rows per iteration
@@ -170,7 +171,8 @@ __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_kernel(const
 #pragma unroll
             for (int b = 0; b < kPredUpBTile; ++b) {
                 if (b0 + b < B) {  // uniform across the wave
-                    const float v = group_sum_dpp<LPR>(s[it][b]);
+                    float v = group_sum_dpp<LPR>(s[it][b]);
+                    if (round_storage) v = to_float<T>(from_float<T>(v));
                     any[it] = any[it] || (cmp_ge ? (v >= thr) : (v > thr));
                     if (scores && cl == 0 && row_ok) scores[(size_t)(b0 + b) * I + row] = v;
                 }
@@ -195,7 +197,7 @@ template <typename T, int LPR, int NITER>
 __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_rows_kernel(const float *__restrict__ t, int B, int r,
                                                                        const T *__restrict__ Bm, int I, float thr,
                                                                        int cmp_ge, float *__restrict__ scores,
-                                                                       uint8_t *__restrict__ mask)
+                                                                       uint8_t *__restrict__ mask, int round_storage)
 {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int RPI = kWave / LPR;   // rows per iteration
@@ -254,7 +256,8 @@ __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_rows_kernel(
                     float acc = 0.f;
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) acc = fmaf(fw[e], tr[b][e], acc);
-                    const float v = group_sum_dpp<LPR>(acc);
+                    float v = group_sum_dpp<LPR>(acc);
+                    if (round_storage) v = to_float<T>(from_float<T>(v));
                     if (cmp_ge ? (v >= thr) : (v > thr)) any |= 1u << it;
                     if (scores && cl == 0 && row < I) scores[(size_t)(b0 + b) * I + row] = v;
                 }
@@ -270,18 +273,18 @@ __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_rows_kernel(
 
 template <typename T, int LPR, int RPW>
 static void launch_up_rpw(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
-                          float *scores, uint8_t *mask, hipStream_t stream)
+                          float *scores, uint8_t *mask, int round_storage, hipStream_t stream)
 {
     constexpr size_t batch = (size_t)kPredUpThreads * 2 * 16;   // the staging buffer is padded to whole batches
     const size_t lds = ((size_t)B * r * sizeof(float) + batch - 1) / batch * batch;
     constexpr int rows = RPW * (kPredUpThreads / kWave);
     ST_LAUNCH(ps, (predictor_up_mask_kernel<T, LPR, RPW>), dim3((I + rows - 1) / rows), dim3(kPredUpThreads), lds,
-              stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask);
+              stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask, round_storage);
 }
 
 template <typename T, int LPR>
 static void launch_up(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
-                      float *scores, uint8_t *mask, hipStream_t stream)
+                      float *scores, uint8_t *mask, int round_storage, hipStream_t stream)
 {
     constexpr int NITER = LPR >= 16 ? LPR / 16 : 1;   // about four rows of Bm per wave (measured against 1, 2 and 8 per lane)
     if (B > 1 && r / Elem<T>::kVec <= LPR) {
@@ -289,38 +292,38 @@ static void launch_up(ProfScope &ps, const float *t_ws, int B, int r, const void
         const size_t lds = ((size_t)B * r * sizeof(float) + batch - 1) / batch * batch;
         constexpr int rows = (kWave / LPR) * NITER * (kPredUpThreads / kWave);
         ST_LAUNCH(ps, (predictor_up_mask_rows_kernel<T, LPR, NITER>), dim3((I + rows - 1) / rows), dim3(kPredUpThreads),
-                  lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask);
+                  lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask, round_storage);
         return;
     }
-    launch_up_rpw<T, LPR, pred_rows_per_wave(LPR)>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+    launch_up_rpw<T, LPR, pred_rows_per_wave(LPR)>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
 }
 
 template <typename T>
 static int launch_predictor(const void *x, int B, int H, const void *A, int r, const void *Bm, int I, float thr,
-                            int cmp_ge, float *t_ws, float *scores, uint8_t *mask, hipStream_t stream)
+                            int cmp_ge, float *t_ws, float *scores, uint8_t *mask, int round_storage, hipStream_t stream)
 {
     constexpr int VEC = Elem<T>::kVec;
     {
         ProfScope ps(ST_K_PRED_DOWN, stream);
         if (B == 1)
             ST_LAUNCH(ps, (predictor_down_kernel<T, 1>), dim3(r), dim3(kPredDownThreads), 0, stream,
-                      static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
+                      static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws, round_storage);
         else if (B <= kPredBTile)
             ST_LAUNCH(ps, (predictor_down_kernel<T, kPredBTile>), dim3(r), dim3(kPredDownThreads), 0, stream,
-                      static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
+                      static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws, round_storage);
         else   // 9 to 16 rows of x in one pass (one memory round trip instead of two)
             ST_LAUNCH(ps, (predictor_down_kernel<T, 2 * kPredBTile>), dim3(r), dim3(kPredDownThreads), 0, stream,
-                      static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws);
+                      static_cast<const T *>(x), B, H, static_cast<const T *>(A), r, t_ws, round_storage);
     }
     ST_HIP(hipGetLastError());
     const int chunks = r / VEC;
     {
         ProfScope ps(ST_K_PRED_UP_MASK, stream);
-        if (chunks <= 4) launch_up<T, 4>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
-        else if (chunks <= 8) launch_up<T, 8>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
-        else if (chunks <= 16) launch_up<T, 16>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
-        else if (chunks <= 32) launch_up<T, 32>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
-        else launch_up<T, 64>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, stream);
+        if (chunks <= 4) launch_up<T, 4>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
+        else if (chunks <= 8) launch_up<T, 8>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
+        else if (chunks <= 16) launch_up<T, 16>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
+        else if (chunks <= 32) launch_up<T, 32>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
+        else launch_up<T, 64>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
     }
     ST_HIP(hipGetLastError());
     return ST_OK;
@@ -328,28 +331,37 @@ static int launch_predictor(const void *x, int B, int H, const void *A, int r, c
 
 }  // namespace st
 
+extern "C" int st_predictor_mask_ex(const void *x, int64_t B, int64_t H, const void *A, int64_t r, const void *Bm,
+                                    int64_t I, int dtype, float thr, int cmp_ge, int flags, float *t_ws, float *scores,
+                                    uint8_t *mask, void *stream)
+{
+    using namespace st;
+    ST_REQUIRE(x && A && Bm && t_ws && mask, "st_predictor_mask_ex: null pointer");
+    ST_REQUIRE(dtype >= ST_F32 && dtype <= ST_BF16, "st_predictor_mask_ex: unknown dtype %d", dtype);
+    const int esz = dtype == ST_F32 ? 4 : 2;
+    ST_REQUIRE(B >= 1 && B <= 64, "st_predictor_mask_ex: B=%lld out of range [1,64]", (long long)B);
+    ST_REQUIRE(H >= 1 && (H * esz) % 16 == 0, "st_predictor_mask_ex: H=%lld rows are not 16-byte multiples",
+               (long long)H);
+    ST_REQUIRE(r >= 1 && (r * esz) % 16 == 0, "st_predictor_mask_ex: rank %lld rows are not 16-byte multiples",
+               (long long)r);
+    ST_REQUIRE(I >= 1 && I <= (1 << 24), "st_predictor_mask_ex: I=%lld out of range", (long long)I);
+    ST_REQUIRE(B * r * 4 <= 56 * 1024, "st_predictor_mask_ex: B*r=%lld too large for the LDS staging buffer",
+               (long long)(B * r));
+    const uintptr_t align = (uintptr_t)x | (uintptr_t)A | (uintptr_t)Bm;
+    ST_REQUIRE((align & 15) == 0, "st_predictor_mask_ex: pointers must be 16-byte aligned");
+    ST_REQUIRE((flags & ~ST_PRED_ROUND_STORAGE) == 0, "st_predictor_mask_ex: unknown flags %d", flags);
+    const int round_storage = (flags & ST_PRED_ROUND_STORAGE) && dtype != ST_F32 ? 1 : 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+    case ST_F32: return launch_predictor<float>(x, (int)B, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, scores, mask, round_storage, s);
+    case ST_F16: return launch_predictor<f16_t>(x, (int)B, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, scores, mask, round_storage, s);
+    default: return launch_predictor<bf16_t>(x, (int)B, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, scores, mask, round_storage, s);
+    }
+}
+
 extern "C" int st_predictor_mask(const void *x, int64_t B, int64_t H, const void *A, int64_t r, const void *Bm,
                                  int64_t I, int dtype, float thr, int cmp_ge, float *t_ws, float *scores,
                                  uint8_t *mask, void *stream)
 {
-    using namespace st;
-    ST_REQUIRE(x && A && Bm && t_ws && mask, "st_predictor_mask: null pointer");
-    ST_REQUIRE(dtype >= ST_F32 && dtype <= ST_BF16, "st_predictor_mask: unknown dtype %d", dtype);
-    const int esz = dtype == ST_F32 ? 4 : 2;
-    ST_REQUIRE(B >= 1 && B <= 64, "st_predictor_mask: B=%lld out of range [1,64]", (long long)B);
-    ST_REQUIRE(H >= 1 && (H * esz) % 16 == 0, "st_predictor_mask: H=%lld rows are not 16-byte multiples",
-               (long long)H);
-    ST_REQUIRE(r >= 1 && (r * esz) % 16 == 0, "st_predictor_mask: rank %lld rows are not 16-byte multiples",
-               (long long)r);
-    ST_REQUIRE(I >= 1 && I <= (1 << 24), "st_predictor_mask: I=%lld out of range", (long long)I);
-    ST_REQUIRE(B * r * 4 <= 56 * 1024, "st_predictor_mask: B*r=%lld too large for the LDS staging buffer",
-               (long long)(B * r));
-    const uintptr_t align = (uintptr_t)x | (uintptr_t)A | (uintptr_t)Bm;
-    ST_REQUIRE((align & 15) == 0, "st_predictor_mask: pointers must be 16-byte aligned");
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    switch (dtype) {
-    case ST_F32: return launch_predictor<float>(x, (int)B, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, scores, mask, s);
-    case ST_F16: return launch_predictor<f16_t>(x, (int)B, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, scores, mask, s);
-    default: return launch_predictor<bf16_t>(x, (int)B, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, scores, mask, s);
-    }
+    return st_predictor_mask_ex(x, B, H, A, r, Bm, I, dtype, thr, cmp_ge, 0, t_ws, scores, mask, stream);
 }

@@ -219,13 +219,16 @@ def sparse_mlp_forward(x: torch.Tensor, concat_weight: torch.Tensor, active_down
 
 def predictor_mask(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.Tensor, thr: float = 0.0,
                    ge: bool = True, return_scores: bool = False, out: Optional[torch.Tensor] = None,
-                   t_ws: Optional[torch.Tensor] = None, scores_out: Optional[torch.Tensor] = None):
+                   t_ws: Optional[torch.Tensor] = None, scores_out: Optional[torch.Tensor] = None,
+                   round_to_storage: bool = False):
     """mask[i] = any over rows b of ((x @ down^T) @ up^T)[b, i] >= thr  (``>`` when ``ge`` is False).
 
     x: [..., H]; down_weight: [r, H] (FastLoRAProjection.down.weight); up_weight: [I, r].
     Returns a bool[I] tensor (and the fp32 scores [B, I] when ``return_scores`` or ``scores_out`` is given;
     ``scores_out`` is a caller-owned buffer, for loops that must not allocate).
     thr = 0, ge = True is the reference's "naive" method (src/modeling_skip.py:206-207).
+    ``round_to_storage``: round the rank-r intermediate and the scores to x's dtype before they are used, as the
+    reference's two half-precision modules do (by default both stay in fp32).
     """
     dev = require_gpu(x, down_weight, up_weight, out)
     H = x.shape[-1]
@@ -256,16 +259,20 @@ def predictor_mask(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.
     mask = out if out is not None else torch.empty(I, dtype=torch.bool, device=dev)
     if mask.dtype != torch.bool or mask.numel() != I or not mask.is_contiguous():
         raise ValueError("out must be a contiguous bool[I] tensor")
-    rc = _lib.lib().st_predictor_mask(
+    rc = _lib.lib().st_predictor_mask_ex(
         x2.data_ptr(), B, H, down_weight.data_ptr(), r, up_weight.data_ptr(), I, dtype_code(x2), float(thr), int(ge),
-        t_ws.data_ptr(), scores.data_ptr() if scores is not None else None, mask.data_ptr(), current_stream_ptr(dev))
-    _lib.check(rc, "st_predictor_mask")
+        1 if round_to_storage else 0, t_ws.data_ptr(), scores.data_ptr() if scores is not None else None,
+        mask.data_ptr(), current_stream_ptr(dev))
+    _lib.check(rc, "st_predictor_mask_ex")
     return (mask, scores) if (return_scores or scores_out is not None) else mask
 
 
-def predictor_scores(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.Tensor) -> torch.Tensor:
-    """fp32 scores [B, I] of the LoRA predictor (FastLoRAProjection.forward)."""
-    return predictor_mask(x, down_weight, up_weight, 0.0, True, return_scores=True)[1]
+def predictor_scores(x: torch.Tensor, down_weight: torch.Tensor, up_weight: torch.Tensor,
+                     round_to_storage: bool = False) -> torch.Tensor:
+    """fp32 scores [B, I] of the LoRA predictor (FastLoRAProjection.forward); with ``round_to_storage`` they hold
+    values of x's dtype (see predictor_mask)."""
+    return predictor_mask(x, down_weight, up_weight, 0.0, True, return_scores=True,
+                          round_to_storage=round_to_storage)[1]
 
 
 MASK_METHODS = {"topk": 0, "statistical_topk": 1}

@@ -23,9 +23,12 @@ from .weight_cache import WeightCache
 class FastLoRAProjection:
     """scores = (x @ down.weight^T) @ up.weight^T with down.weight [r,H], up.weight [I,r]."""
 
-    def __init__(self, down_weight: torch.Tensor, up_weight: torch.Tensor):
+    def __init__(self, down_weight: torch.Tensor, up_weight: torch.Tensor, round_to_storage: bool = False):
+        """``round_to_storage``: round the rank-r intermediate and the scores to the weights' dtype, as the reference's
+        ``up(down(x))`` does when the model runs in fp16 / bf16 (default: both stay in fp32)."""
         self.down_weight = down_weight.contiguous()
         self.up_weight = up_weight.contiguous()
+        self.round_to_storage = bool(round_to_storage)
         self.lora_size, self.hidden_size = self.down_weight.shape
         self.intermediate_size = self.up_weight.size(0)
 
@@ -49,7 +52,7 @@ class FastLoRAProjection:
         return f"final_predictor_layer_{layer_idx}_lora_{lora_pct:.1f}pct.pt"
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return predictor_scores(x, self.down_weight, self.up_weight)
+        return predictor_scores(x, self.down_weight, self.up_weight, self.round_to_storage)
 
     __call__ = forward
 
@@ -66,16 +69,18 @@ class FastLoRAProjection:
         allocation-free.
         """
         if method == "naive":
-            return predictor_mask(x, self.down_weight, self.up_weight, 0.0, True, out=out, t_ws=t_ws)
+            return predictor_mask(x, self.down_weight, self.up_weight, 0.0, True, out=out, t_ws=t_ws,
+                                  round_to_storage=self.round_to_storage)
         if method == "threshold":
-            return predictor_mask(x, self.down_weight, self.up_weight, thr, ge, out=out, t_ws=t_ws)
+            return predictor_mask(x, self.down_weight, self.up_weight, thr, ge, out=out, t_ws=t_ws,
+                                  round_to_storage=self.round_to_storage)
         if method not in ("topk", "statistical_topk"):
             raise ValueError(f"unknown sparsity method {method!r}")
         if scores_ws is None:
             scores = self.forward(x)
         else:   # caller-owned buffers: nothing is allocated (what a captured decode loop needs)
             scores = predictor_mask(x, self.down_weight, self.up_weight, 0.0, True, out=out, t_ws=t_ws,
-                                    scores_out=scores_ws)[1]
+                                    scores_out=scores_ws, round_to_storage=self.round_to_storage)[1]
         return mask_select(scores, method, k=k, std_multiplier=std_multiplier, out=out, workspace=select_ws)
 
 

@@ -133,3 +133,38 @@ def test_loaded_checkpoints_drive_the_hip_predictor(tmp_path):
         got_naive = p.mask(x.to(DEV), "naive").cpu().numpy()
         safe = np.abs(s_ref).min(0) > 8e-6 * scale
         assert np.array_equal(got_naive[safe], oracle.mask_threshold(s_ref, 0.0, True)[safe]) and safe.mean() > 0.999
+
+
+@pytest.mark.parametrize("dtype,B,H,r,I", [("float16", 1, 3072, 128, 8192), ("bfloat16", 4, 4096, 256, 14336)])
+def test_scores_rounded_to_the_storage_type(dtype, B, H, r, I):
+    """round_to_storage: the rank-r intermediate and the scores as two half-precision modules hand them on
+    (FastLoRAProjection in an fp16 / bf16 model, src/modeling_skip.py:52-53) against the oracle's restatement of that;
+    and how many mask bits that moves against the fp32 scores at the benchmark's active fraction."""
+    x, A, Bm = _weights(5, B, H, r, I, dtype)
+    xs, As, Bs = x.float().numpy(), A.float().numpy(), Bm.float().numpy()
+    want = oracle.predictor_scores(xs, As, Bs, storage=dtype)
+    got = st.predictor_scores(x.to(DEV), A.to(DEV), Bm.to(DEV), round_to_storage=True).cpu().numpy()
+    # every score is a value of the storage type
+    tdt = getattr(torch, dtype)
+    assert np.array_equal(torch.from_numpy(got).to(tdt).float().numpy(), got)
+    # equal to the oracle's except where an fp32 sum sat within rounding distance of a tie between two storage values:
+    # a score is then one step of the storage type off, or -- when it was an entry of the intermediate -- a few
+    ulp = np.abs(want) * (2.0 ** -10 if dtype == "float16" else 2.0 ** -7) + 1e-30
+    diff = np.abs(got - want)
+    assert (diff <= 8 * ulp + 1e-3 * np.abs(want).max()).all() and (diff > 0).mean() < 0.02, \
+        ((diff > 0).mean(), (diff / ulp).max())
+    # masks: exact wherever the two implementations' scores agree; and the count of bits the rounding itself moves
+    s32 = oracle.predictor_scores(xs, As, Bs)
+    thr = syn.threshold_for_fraction(s32.max(0), 0.35)
+    m_round = st.predictor_mask(x.to(DEV), A.to(DEV), Bm.to(DEV), thr, True, round_to_storage=True).cpu().numpy()
+    agree = (diff == 0).all(0)
+    assert np.array_equal(m_round[agree], oracle.mask_threshold(want, thr, True)[agree])
+    m_fp32 = st.predictor_mask(x.to(DEV), A.to(DEV), Bm.to(DEV), thr, True).cpu().numpy()
+    moved = int((m_round != m_fp32).sum())
+    print(f"{dtype}: {moved} of {I} mask bits differ between scores kept in fp32 and scores rounded to {dtype}")
+    assert moved <= (40 if dtype == "float16" else 300)
+    # fp32 storage: the flag changes nothing
+    x32, A32, B32 = _weights(6, 1, 256, 16, 512, "float32")
+    a = st.predictor_scores(x32.to(DEV), A32.to(DEV), B32.to(DEV), round_to_storage=True)
+    b = st.predictor_scores(x32.to(DEV), A32.to(DEV), B32.to(DEV))
+    assert torch.equal(a, b)
