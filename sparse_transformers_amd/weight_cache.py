@@ -157,8 +157,18 @@ class WeightCache:
 
     def update_active_weights(self, mask: torch.Tensor) -> None:
         """weight_cache.h:229: raises RuntimeError("No active weights") when the mask empties the cache."""
+        known = not self._dirty
+        serial = int(self._host_state[_lib.STATE_SERIAL])
         self.update_active_weights_async(mask)
-        self.sync_state()
+        try:
+            self.sync_state()
+        except RuntimeError as exc:
+            # The "emptied" status stays in the state words until an update changes something.  An update with an
+            # unchanged mask touches nothing and returns silently in the reference (weight_cache.h:237-240), also
+            # right after the update that emptied the cache: only an update that did something may raise.
+            if str(exc) == "No active weights" and known and int(self._host_state[_lib.STATE_SERIAL]) == serial:
+                return
+            raise
 
     def sync_state(self) -> dict:
         """Read the state words back (waits for the current stream)."""

@@ -126,6 +126,12 @@ def test_noop_and_error_semantics():
     assert s1["serial"] == s0["serial"] and s1["n_changed"] == 0 and s1["n_active"] == 3
     with pytest.raises(RuntimeError, match="No active weights"):
         wc.update_active_weights(torch.zeros(I, dtype=torch.bool, device=DEV))
+    # the remembered mask is still m0 (the reference stores the new mask only after a successful rebuild), so m0 is
+    # an unchanged mask now: the reference returns before touching anything, and so does this -- no second error
+    wc.update_active_weights(_t(m0, torch.bool))
+    assert wc.get_num_active() == 0
+    with pytest.raises(RuntimeError, match="No active weights"):      # all-false again differs from m0: it raises again
+        wc.update_active_weights(torch.zeros(I, dtype=torch.bool, device=DEV))
     # an all-false init mask is an unchanged mask for the constructor's update (weight_cache.h:223-226,237-240):
     # nothing is built, and the getters then refuse like the reference's TORCH_CHECK(cache_valid)
     empty = st.WeightCache(torch.zeros(I, dtype=torch.bool, device=DEV), H, _t(gate), _t(up), _t(down), True)
