@@ -954,6 +954,248 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     ST_TL(7);
 }
 
+// ---------------------------------------------------------------------------
+// update for intermediate sizes the kernels above cannot hold in LDS (kPlanMaxI < I <= kBigMaxI).
+// The same replay of WeightCache::update_active_weights (weight_cache.h:229-359) in every block, with the
+// masks as bitmaps and no added / removed lists: the i-th removed or added index is found through per-word
+// prefix counts (rank of a set bit; i-th set bit by bisection), which leaves 4.5 bytes of LDS per element --
+// the two index maps the sequential surplus removals (:310-353) need.  Blocks then copy the rows of the
+// positions they own (position p belongs to block p mod (blocks - 1); block 0 publishes the bookkeeping).
+// ---------------------------------------------------------------------------
+constexpr int64_t kBigMaxI = 32768;
+constexpr int kBigThreads = 1024;
+constexpr int kBigWords = 4;   // 8-byte mask words per thread: I <= 8 * 1024 * 4
+
+constexpr size_t big_lds_bytes(int I)
+{
+    const size_t w32 = (size_t)((I + 31) >> 5);
+    return (size_t)I * 4 + w32 * 4 * 3 + w32 * 2 * 2 + 64;
+}
+
+struct BigShared {
+    uint32_t wave_tot[kBigThreads / kWave];
+    int n_new, na, nr;
+};
+
+// index of the i-th (from 0) set bit of bits[w] & ~mask_out[w] over all words, given the exclusive prefix counts
+__device__ __forceinline__ int big_select(const uint32_t *bits, const uint32_t *notbits, const uint16_t *prefix, int W32, int i)
+{
+    int lo = 0;
+    for (int step = 1024; step >= 1; step >>= 1) {
+        const int c = lo + step;
+        if (c < W32 && (int)prefix[c] <= i) lo = c;
+    }
+    uint32_t w = bits[lo] & ~notbits[lo];
+    int j = i - (int)prefix[lo], pos = 0;
+#pragma unroll
+    for (int half = 16; half >= 1; half >>= 1) {
+        const uint32_t lowmask = (1u << half) - 1u;
+        const int c = __popc(w & lowmask);
+        if (j >= c) { j -= c; pos += half; w >>= half; }
+        w &= lowmask;
+    }
+    return lo * 32 + pos;
+}
+
+__global__ __launch_bounds__(kBigThreads) void cache_update_big_kernel(FusedRows fr, const uint8_t *__restrict__ new_mask,
+                                                                      uint8_t *__restrict__ cur_mask2,
+                                                                      int32_t *__restrict__ indices2,
+                                                                      int32_t *__restrict__ state, int I)
+{
+    constexpr int TPB = kBigThreads;
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ BigShared bs;
+    const int tid = threadIdx.x;
+    const int W32 = (I + 31) >> 5;
+    uint16_t *pos_l = reinterpret_cast<uint16_t *>(smem);   // index -> position (kNone when absent)
+    uint16_t *idx_l = pos_l + I;                            // position -> index
+    uint32_t *newbits = reinterpret_cast<uint32_t *>(idx_l + I + (I & 1));
+    uint32_t *oldbits = newbits + W32, *dirty = oldbits + W32;
+    uint16_t *pa = reinterpret_cast<uint16_t *>(dirty + W32), *pr = pa + W32 + (W32 & 1);
+    auto sync = [&]() __attribute__((always_inline)) { lds_barrier(); };
+
+    const uint32_t tword = __hip_atomic_load(reinterpret_cast<const uint32_t *>(&state[ST_STATE_TICKET]), __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+    const int ep = (int)((tword >> 16) & 1u);
+    const int n = state[ST_STATE_N_BUF0 + ep];
+    const int serial_old = state[ST_STATE_SERIAL];
+    const uint8_t *cur_mask = cur_mask2 + (size_t)ep * I;
+    const int32_t *indices = indices2 + (size_t)ep * I;
+    // masks -> bitmaps (8 elements per byte of the bitmaps), kept as 0x01 bytes in registers for publishing
+    uint64_t w_new[kBigWords], w_cur[kBigWords];
+#pragma unroll
+    for (int w = 0; w < kBigWords; ++w) {
+        const int bi = tid * kBigWords + w;
+        const bool in = bi * 8 < I;
+        const int ec = in ? bi * 8 : 0;
+        w_new[w] = in ? nonzero_bytes(*reinterpret_cast<const uint64_t *>(new_mask + ec)) : 0ull;
+        w_cur[w] = in ? nonzero_bytes(*reinterpret_cast<const uint64_t *>(cur_mask + ec)) : 0ull;
+        if (bi < W32 * 4) {
+            reinterpret_cast<uint8_t *>(newbits)[bi] = (uint8_t)pack_bits8(w_new[w]);
+            reinterpret_cast<uint8_t *>(oldbits)[bi] = (uint8_t)pack_bits8(w_cur[w]);
+        }
+    }
+    for (int i = tid; i < I; i += TPB) pos_l[i] = kNone;
+    for (int w = tid; w < W32; w += TPB) dirty[w] = 0u;
+    for (int p = tid; p < n; p += TPB) idx_l[p] = (uint16_t)indices[p];
+    sync();
+    for (int p = tid; p < n; p += TPB) pos_l[idx_l[p]] = (uint16_t)p;
+    // per-word prefix counts of added / removed indices (one word per thread: W32 <= 1024)
+    uint32_t addw = 0u, remw = 0u;
+    if (tid < W32) { addw = newbits[tid] & ~oldbits[tid]; remw = oldbits[tid] & ~newbits[tid]; }
+    uint32_t total;
+    const uint32_t off = block_excl_scan<TPB / kWave>((uint32_t)__popc(addw) | ((uint32_t)__popc(remw) << 16), bs.wave_tot,
+                                                      &total, tid, sync);
+    if (tid < W32) { pa[tid] = (uint16_t)(off & 0xffffu); pr[tid] = (uint16_t)(off >> 16); }
+    const int na = (int)(total & 0xffffu), nr = (int)(total >> 16);
+    const bool writer = blockIdx.x == 0;
+    uint32_t arrival = 0;
+    if (na == 0 && nr == 0) {   // unchanged mask: nothing is touched (weight_cache.h:237-240)
+        if (tid == 0 && writer) {
+            state[ST_STATE_N_CHANGED] = 0;
+            state[ST_STATE_N_ADDED] = 0;
+            state[ST_STATE_N_REMOVED] = 0;
+        }
+        if (tid == 0) {
+            arrival = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
+            if ((arrival & 0xffffu) == gridDim.x - 1)
+                atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)ep << 16);
+        }
+        return;
+    }
+    sync();   // pos_l, pa, pr complete
+    const int pairs = na < nr ? na : nr;
+    // ---- phase 1: the i-th removed index hands its position to the i-th added one; phase 2: surplus additions appended
+    if (tid < W32) {
+        uint32_t r = remw;
+        int rank = (int)pr[tid];
+        while (r && rank < pairs) {
+            const int e = tid * 32 + __ffs((int)r) - 1;
+            r &= r - 1u;
+            const uint16_t p = pos_l[e];
+            if (p != kNone) {
+                const int a = big_select(newbits, oldbits, pa, W32, rank);
+                idx_l[p] = (uint16_t)a;
+                pos_l[a] = p;
+                pos_l[e] = kNone;
+                atomicOr(&dirty[p >> 5], 1u << (p & 31));
+            }
+            ++rank;
+        }
+        uint32_t a_bits = addw;
+        int arank = (int)pa[tid];
+        while (a_bits) {
+            const int a = tid * 32 + __ffs((int)a_bits) - 1;
+            a_bits &= a_bits - 1u;
+            if (arank >= pairs) {
+                const int p = n + (arank - pairs);
+                if (p < I) {
+                    idx_l[p] = (uint16_t)a;
+                    pos_l[a] = (uint16_t)p;
+                    atomicOr(&dirty[p >> 5], 1u << (p & 31));
+                }
+            }
+            ++arank;
+        }
+    }
+    sync();
+    int n_new;
+    if (nr <= na) {
+        n_new = n + (na - pairs);
+        if (n_new > I) n_new = I;
+    } else {
+        // ---- phase 3: surplus removals in ascending index order, sequential by construction
+        if (tid == 0) {
+            int m = n, k = 0;
+            for (int w = 0; w < W32; ++w) {
+                uint32_t r = oldbits[w] & ~newbits[w];
+                while (r) {
+                    const int e = w * 32 + __ffs((int)r) - 1;
+                    r &= r - 1u;
+                    if (k++ < pairs) continue;
+                    const uint16_t p = pos_l[e];
+                    if (p == kNone) continue;
+                    if (m <= 0) { w = W32; break; }
+                    const int last = m - 1;
+                    if ((int)p != last) {
+                        const uint16_t li = idx_l[last];
+                        idx_l[p] = li;
+                        pos_l[li] = p;
+                        dirty[p >> 5] |= 1u << (p & 31);
+                    }
+                    --m;
+                    pos_l[e] = kNone;
+                }
+            }
+            bs.n_new = m;
+        }
+        sync();
+        n_new = bs.n_new;
+    }
+    // rows rewritten: positions below the new count whose index changed
+    uint32_t dcount = 0;
+    for (int w = tid; w < W32; w += TPB) {
+        uint32_t d = dirty[w];
+        const int lo = w << 5;
+        if (lo >= n_new) d = 0u;
+        else if (lo + 32 > n_new) d &= (1u << (n_new - lo)) - 1u;
+        dcount += (uint32_t)__popc(d);
+    }
+    uint32_t n_changed;
+    (void)block_excl_scan<TPB / kWave>(dcount, bs.wave_tot, &n_changed, tid, sync);
+    // ---- publish: block 0 writes the other bookkeeping buffer, the last arrival flips the epoch
+    if (writer) {
+        int32_t *idx_out = indices2 + (size_t)(ep ^ 1) * I;
+        uint8_t *mask_out = cur_mask2 + (size_t)(ep ^ 1) * I;
+        for (int p = tid; p < n_new; p += TPB) idx_out[p] = idx_l[p];
+#pragma unroll
+        for (int w = 0; w < kBigWords; ++w) {
+            const int bi = tid * kBigWords + w;
+            if (bi * 8 < I) *reinterpret_cast<uint64_t *>(mask_out + (size_t)bi * 8) = n_new > 0 ? w_new[w] : w_cur[w];
+        }
+        if (tid == 0) {
+            state[ST_STATE_N_BUF0 + (ep ^ 1)] = n_new;
+            state[ST_STATE_N_ACTIVE] = n_new;
+            state[ST_STATE_N_CHANGED] = (int)n_changed;
+            state[ST_STATE_N_ADDED] = na;
+            state[ST_STATE_N_REMOVED] = nr;
+            state[ST_STATE_SERIAL] = serial_old + 1;
+            state[ST_STATE_EPOCH] = ep ^ 1;
+            if (n_new > 0) {
+                state[ST_STATE_STATUS] = 0;
+                state[ST_STATE_VALID] = 1;
+            } else {
+                state[ST_STATE_STATUS] = ST_ERR_NO_ACTIVE;
+            }
+        }
+    }
+    if (tid == 0) arrival = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
+    // ---- copies: active[p] <- pool[index at p] for the dirty positions this block owns
+    {
+        const int row_bytes = fr.row_bytes, chunks = row_bytes >> 4;
+        const bool has_gate = fr.has_gate != 0;
+        const bool solo = gridDim.x == 1;
+        const int owners = solo ? 1 : (int)gridDim.x - 1, me = solo ? 0 : (int)blockIdx.x - 1;
+        if (solo || !writer) {
+            for (int p = me; p < n_new; p += owners) {
+                if (!((dirty[p >> 5] >> (p & 31)) & 1u)) continue;   // uniform over the block
+                const size_t from = (size_t)idx_l[p] * row_bytes, to = (size_t)p * row_bytes;
+                for (int c = tid; c < chunks; c += TPB) {
+                    const size_t o = (size_t)c << 4;
+                    const uint4 vu = ld16(fr.pool_u + from + o), vd = ld16(fr.pool_d + from + o);
+                    uint4 vg = make_uint4(0u, 0u, 0u, 0u);
+                    if (has_gate) vg = ld16(fr.pool_g + from + o);
+                    st16(fr.act_u + to + o, vu);
+                    st16(fr.act_d + to + o, vd);
+                    if (has_gate) st16(fr.act_g + to + o, vg);
+                }
+            }
+        }
+    }
+    if (tid == 0 && (arrival & 0xffffu) == gridDim.x - 1)
+        atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)(ep ^ 1) << 16);
+}
+
 // in [R,C] -> out [C,R], 64x64 tiles through LDS.
 template <typename E>
 __global__ __launch_bounds__(256) void transpose_kernel(const E *__restrict__ in, E *__restrict__ out, int R, int C)
@@ -992,7 +1234,7 @@ struct st_cache {
     int32_t *host_state;  // pinned
 };
 
-extern "C" int64_t st_cache_max_intermediate(void) { return st::kPlanMaxI; }
+extern "C" int64_t st_cache_max_intermediate(void) { return st::kBigMaxI; }
 
 extern "C" st_cache *st_cache_create(const st_cache_buffers *bufs, int64_t I, int64_t H, int dtype, int has_gate)
 {
@@ -1001,7 +1243,8 @@ extern "C" st_cache *st_cache_create(const st_cache_buffers *bufs, int64_t I, in
     if (!bufs) return fail("null buffers");
     if (dtype < ST_F32 || dtype > ST_BF16) return fail("unknown dtype");
     const int esz = dtype == ST_F32 ? 4 : 2;
-    if (I < 1 || I > kPlanMaxI) return fail("intermediate size out of range (see st_cache_max_intermediate)");
+    if (I < 1 || I > kBigMaxI) return fail("intermediate size out of range (see st_cache_max_intermediate)");
+    if (I > kPlanMaxI && I % 8 != 0) return fail("intermediate sizes above 22000 must be multiples of 8");
     if (H < 1 || (H * esz) % 16 != 0) return fail("rows are not 16-byte multiples");
     if (!bufs->up_pool || !bufs->downT_pool || !bufs->up_active || !bufs->down_active || !bufs->indices ||
         !bufs->cur_mask || !bufs->state)
@@ -1060,6 +1303,31 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     ST_REQUIRE(c && mask, "st_cache_update_async: null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int I = (int)c->I;
+    if (I > kPlanMaxI) {   // index maps of the other kernels do not fit the LDS: bitmap plan, rows by position
+        ST_REQUIRE(I % 8 == 0 && (uintptr_t)mask % 8 == 0 && (uintptr_t)c->b.cur_mask % 8 == 0,
+                   "st_cache_update_async: for I > %lld the masks must be 8-byte aligned", (long long)kPlanMaxI);
+        FusedRows fr;
+        fr.pool_u = static_cast<const unsigned char *>(c->b.up_pool);
+        fr.act_u = static_cast<unsigned char *>(c->b.up_active);
+        fr.pool_d = static_cast<const unsigned char *>(c->b.downT_pool);
+        fr.act_d = static_cast<unsigned char *>(c->b.down_active);
+        fr.pool_g = c->has_gate ? static_cast<const unsigned char *>(c->b.gate_pool) : fr.pool_u;
+        fr.act_g = c->has_gate ? static_cast<unsigned char *>(c->b.gate_active) : fr.act_u;
+        fr.row_bytes = (int)(c->H * c->esz);
+        fr.has_gate = c->has_gate ? 1 : 0;
+        const size_t lds_big = big_lds_bytes(I);
+        static std::atomic<bool> big_attr{false};
+        if (!big_attr.load(std::memory_order_acquire)) {
+            ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(cache_update_big_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+            big_attr.store(true, std::memory_order_release);
+        }
+        ProfScope ps(ST_K_CACHE_UPDATE, s);
+        ST_LAUNCH(ps, cache_update_big_kernel, dim3(device_cu_count()), dim3(kBigThreads), lds_big, s, fr, mask,
+                  c->b.cur_mask, c->b.indices, c->b.state, I);
+        ST_HIP(hipGetLastError());
+        return ST_OK;
+    }
     const size_t lds = plan_lds_bytes(I);
     CopyPlan cp;
     cp.nmat = 0;

@@ -93,6 +93,53 @@ def test_full_size_index_order(I, n, lo, hi):
     assert st_["n_active"] == n and st_["n_added"] == st_["n_removed"] > 0
 
 
+@pytest.mark.parametrize("I,has_gate", [(28672, True), (32768, False), (22016, True)])
+def test_large_intermediate_sizes(I, has_gate):
+    """Intermediate sizes of the 70B-class models (28672), above what the index lists of the smaller kernels allow:
+    index order and layout against the oracle over a trace that starts with every row active, shrinks to a quarter
+    (thousands of sequential removals), then churns with the active count drifting both ways, with a no-op update,
+    the error of an emptying mask and the state after it."""
+    H = 16
+    rng = np.random.default_rng(I)
+    g = rng.standard_normal((I, H)).astype(np.float32)
+    u = rng.standard_normal((I, H)).astype(np.float32)
+    d = rng.standard_normal((H, I)).astype(np.float32)
+    oc = oracle.OracleWeightCache(np.ones(I, bool), H, g if has_gate else None, u, d, has_gate)
+    wc = st.WeightCache(torch.ones(I, dtype=torch.bool, device=DEV), H, _t(g) if has_gate else None, _t(u), _t(d), has_gate)
+    assert wc.get_active_indices().cpu().tolist() == list(range(I))
+    m = rng.random(I) < 0.25
+    masks = [m.copy()]
+    for t in range(24):
+        m = m ^ (rng.random(I) < rng.choice([0.003, 0.02, 0.1]))
+        masks.append(m.copy())
+        if t == 9:
+            masks.append(m.copy())           # unchanged mask
+    for t, mk in enumerate(masks):
+        oc.update_active_weights(mk)
+        wc.update_active_weights(_t(mk, torch.bool))
+        assert wc.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist(), (I, t)
+        if t in (0, 5, len(masks) - 1):
+            _check_layout(wc, oc.get_active_indices().tolist(), g, u, d, has_gate)
+    with pytest.raises(RuntimeError, match="No active weights"):
+        wc.update_active_weights(torch.zeros(I, dtype=torch.bool, device=DEV))
+    with pytest.raises(RuntimeError):
+        oc.update_active_weights(np.zeros(I, bool))
+    # (the remembered mask is still the last good one: only indices outside it are added now)
+    oc.update_active_weights(np.ones(I, bool))
+    wc.update_active_weights(torch.ones(I, dtype=torch.bool, device=DEV))
+    assert wc.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist()
+    assert 0 < wc.get_num_active() < I
+    # update + MLP in one call at this size (two launches underneath) against the oracle
+    x = rng.standard_normal((1, H)).astype(np.float32)
+    oc.update_active_weights(masks[7])
+    y = wc.update_and_forward(_t(masks[7], torch.bool), _t(x), "silu" if has_gate else "relu")
+    want, _ = oracle.mlp_forward(x, oc.get_concat_weight(), oc.get_active_down_weight(), "silu" if has_gate else "relu",
+                                 has_gate)
+    assert wc.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist()
+    scale = np.abs(want).max()
+    assert np.abs(y.cpu().numpy() - want).max() <= 1e-5 * scale + 1e-6
+
+
 def test_full_size_layout_invariants_fp16():
     """cfg-2 shapes: every active row is a bit-copy of its pool row; set(indices) == nonzero(mask)."""
     I, H, n = 8192, 3072, 2867
