@@ -538,6 +538,7 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
 constexpr int kSparseMaxQ = 64;       // positions a block can own
 constexpr int kSparseMaxW32 = 512;    // mask words: I <= 16384
 constexpr int kSparseWords = 2;       // 8-byte mask words per thread, at most
+constexpr int kSparseScan = 4;         // positions per thread whose old index is fetched up front for that replay
 constexpr int kSrcPool = 0x40000000;  // src[]: bit 30 = read the pool row (low bits) and write it back; else active row
 
 struct SparseShared {
@@ -545,6 +546,7 @@ struct SparseShared {
     uint16_t pr[kSparseMaxW32];   // removed indices below each word
     int na, nr, n;
     int src[kSparseMaxQ];
+    int found, paired_tail, replay_ok, nchg;   // surplus removals (removed > added)
 };
 
 // 0x01-per-element bytes -> 8 bits (element k -> bit k)
@@ -619,6 +621,18 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     const int my_p = blk + G * lane;
     const int my_pc = my_p < I ? my_p : I - 1;
     const int i_old0 = indices2[my_pc], i_old1 = indices2[(size_t)I + my_pc];
+    // The ordered list itself, four positions per thread, for the case that removals outnumber additions (the
+    // surplus ones can sit at any position); only as far as the caller's guess of the count plus a quarter.
+    const int n_spec = n_hint < I ? n_hint : I;
+    int scan_cap = (n_spec + (n_spec >> 2) + 64) & ~3;
+    if (scan_cap > kSparseScan * TPB) scan_cap = kSparseScan * TPB;
+    if (scan_cap > I) scan_cap = I & ~3;
+    const int scan_p = kSparseScan * tid;
+    const bool scan_in = scan_p + kSparseScan <= scan_cap;
+    const int scan_pc = scan_in ? scan_p : 0;
+    static_assert(kSparseScan == 4, "one 16-byte load per bookkeeping buffer");
+    const int4 sc0 = *reinterpret_cast<const int4 *>(indices2 + scan_pc);
+    const int4 sc1 = *reinterpret_cast<const int4 *>(indices2 + (size_t)I + scan_pc);
     uint4 xr[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b)
@@ -626,7 +640,6 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
 
     // ---- the first batch of rows, on the caller's guess of the count, from the active buffers
     auto row_of = [&](int bat, int k) { return blk + G * (grp + ngrp * (bat * RB + k)); };
-    const int n_spec = n_hint < I ? n_hint : I;
     uint4 wg[RB], wu[RB], wd[RB];
     // (every wave issues the same number of loads whatever its role: a wave without columns, and the gate loads
     // of an ungated cache, read one line of x instead -- with branches around the loads the compiler could no
@@ -675,6 +688,14 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
             reinterpret_cast<uint8_t *>(sh.newbits)[bi] = (uint8_t)pack_bits8(w_new[w]);
             reinterpret_cast<uint8_t *>(sh.oldbits)[bi] = (uint8_t)pack_bits8(w_cur[w]);
         }
+    }
+    // (behind the list of added indices, which holds I entries at most; the region of the per-index plan, six
+    // bytes per index, is unused on this path)
+    uint16_t *const scan_idx = reinterpret_cast<uint16_t *>(smem) + ((I + 7) & ~7);
+    if (scan_in) {
+        const int4 sc = ep ? sc1 : sc0;
+        *reinterpret_cast<uint2 *>(scan_idx + scan_p) =
+            make_uint2((uint32_t)(sc.x & 0xffff) | ((uint32_t)sc.y << 16), (uint32_t)(sc.z & 0xffff) | ((uint32_t)sc.w << 16));
     }
     lds_barrier();
     // ---- Rows are requested from here on, i.e. once every wave's bookkeeping loads have ARRIVED: loads issued into
@@ -753,7 +774,7 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
             if (lane == 0) sh.n = nn;
         }
         sh.src[lane] = s;
-        if (lane == 0) { sh.na = na_w; sh.nr = nr_w; }
+        if (lane == 0) { sh.na = na_w; sh.nr = nr_w; sh.found = 0; sh.paired_tail = 0; }
     }
     speculate(std::integral_constant<int, SPEC_A>{}, std::integral_constant<int, SPEC>{});
     __builtin_amdgcn_sched_barrier(0);
@@ -763,7 +784,113 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     const bool changed = (na | nr) != 0;
     bool arriver = plan_wave && lane == 0;
     int next_epoch = ep;
-    if (nr <= na) {
+    // Removals outnumber additions: the surplus ones are taken out one by one, in ascending index order, each by
+    // moving the last entry of the list into its place (weight_cache.h:310-353).  With S of them the list ends as
+    // its first n_old - S positions ("base"); the entries of the last S positions ("tail") that stay end up in the
+    // places of the surplus indices below the tail.  Step k takes the entry at tail slot S-1-k and puts it where
+    // the k-th surplus index sits at that time: its place in the list, unless that place is a tail slot whose own
+    // step came earlier (then it has travelled on with that step's move, possibly again).  So the places follow
+    // from the start positions by chasing through tail slots, which only surplus indices that START in the tail
+    // need (few: about S^2 / n_old); they are resolved one after the other, then every surviving tail entry finds
+    // its final place on its own.  Used when S <= min(1024, I/4) and the list was fetched far enough up front;
+    // else the per-index plan.
+    const int surplus = nr - na, tail_base = n_old - surplus;
+    const int smax = (I >> 2) < TPB ? (I >> 2) : TPB;
+    bool replay = surplus > 0 && surplus <= smax && tail_base >= 0 && n_old <= scan_cap;
+    constexpr uint16_t kGone = 0xffffu;   // hole[]: removed as the last entry, nothing moves; tailv[]: a surplus index
+    uint16_t *const hole = scan_idx + ((scan_cap + 7) & ~7);   // start position of the k-th surplus index, then its place at step k
+    uint16_t *const tailv = hole + ((smax + 7) & ~7);          // entry of tail slot j after the paired replacements
+    if (replay) {
+        const uint16_t *added_list = reinterpret_cast<const uint16_t *>(smem);
+        // ---- every thread, four positions: paired replacements in place; where the surplus indices sit; the tail
+        if (scan_in && scan_p < n_old) {
+            uint2 pk = *reinterpret_cast<const uint2 *>(scan_idx + scan_p);
+            uint32_t ent[kSparseScan] = {pk.x & 0xffffu, pk.x >> 16, pk.y & 0xffffu, pk.y >> 16};
+            int found = 0, paired_tail = 0;
+#pragma unroll
+            for (int j = 0; j < kSparseScan; ++j) {
+                const int p = scan_p + j;
+                const int e = (int)ent[j];
+                if (p < n_old) {
+                    const int word = (e >> 5) & (kSparseMaxW32 - 1), bit = e & 31;
+                    const uint32_t remw = sh.oldbits[word] & ~sh.newbits[word];
+                    const bool rem = (remw >> bit) & 1u;
+                    const int rank = rem ? (int)sh.pr[word] + __popc(remw & ((1u << bit) - 1u)) : 0;
+                    const bool extra = rem && rank >= na;
+                    if (rem && !extra) ent[j] = added_list[rank];
+                    if (extra) { hole[rank - na] = (uint16_t)p; ++found; }
+                    if (p >= tail_base) {
+                        tailv[p - tail_base] = extra ? kGone : (uint16_t)ent[j];
+                        if (rem && !extra) ++paired_tail;
+                    }
+                }
+            }
+            pk.x = ent[0] | (ent[1] << 16); pk.y = ent[2] | (ent[3] << 16);
+            *reinterpret_cast<uint2 *>(scan_idx + scan_p) = pk;
+            if (found) atomicAdd(&sh.found, found);
+            if (paired_tail) atomicAdd(&sh.paired_tail, paired_tail);
+        }
+        lds_barrier();
+        // ---- one wave: the places of the surplus indices that start in the tail, in ascending order
+        if (plan_wave) {
+            const int S = __builtin_amdgcn_readfirstlane(surplus), base = __builtin_amdgcn_readfirstlane(tail_base);
+            int in_tail = 0;
+            for (int c = 0; c < S; c += kWave) {
+                const int k = c + lane;
+                uint64_t todo = __builtin_amdgcn_ballot_w64(k < S && (int)hole[k < S ? k : 0] >= base);
+                in_tail += __popcll(todo);
+                while (todo) {
+                    const int kk = c + (int)__builtin_ctzll(todo);
+                    todo &= todo - 1;
+                    int pos = hole[kk];
+                    int i = S - 1 - (pos - base);   // the step that takes the entry of that tail slot
+                    for (int it = 0; it < S && pos >= base && i >= 0 && i < kk; ++it) {
+                        pos = hole[i];
+                        i = S - 1 - (pos - base);
+                    }
+                    if (pos >= base && i == kk) pos = kGone;
+                    if (lane == 0) hole[kk] = (uint16_t)pos;
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+                }
+            }
+            if (lane == 0) {
+                // (a surplus index missing from the list would make the counts disagree: per-index plan then)
+                sh.replay_ok = sh.found == S;
+                sh.n = base;
+                // rewritten positions: the pairs' below the tail, and the places of the surplus indices below it
+                sh.nchg = na - sh.paired_tail + (S - in_tail);
+            }
+        }
+        lds_barrier();
+        replay = sh.replay_ok != 0;
+        if (replay) {
+            // ---- every surviving tail entry to its final place
+            if (tid < surplus) {
+                const uint16_t v = tailv[tid];
+                if (v != kGone) {
+                    int pos = hole[surplus - 1 - tid];
+                    for (int it = 0; it < surplus && pos >= tail_base && pos < n_old; ++it)
+                        pos = hole[surplus - 1 - (pos - tail_base)];
+                    if (pos < tail_base) scan_idx[pos] = v;
+                }
+            }
+            lds_barrier();
+            if (plan_wave) {
+                int s = -1;
+                if (lane < Q && my_p < tail_base) {
+                    const int newidx = scan_idx[my_p];
+                    s = newidx != (ep ? i_old1 : i_old0) ? (newidx | kSrcPool) : my_p;
+                    indices2[(size_t)(ep ^ 1) * I + my_p] = newidx;
+                }
+                sh.src[lane] = s;
+            }
+            lds_barrier();
+        }
+    }
+    if (surplus <= 0 || replay) {
+        const int n_changed = replay ? sh.nchg : na;
         n = sh.n;
         if (changed) {
             // the remembered mask: 8-byte words dealt to the blocks round-robin (the reference keeps the old
@@ -778,7 +905,7 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
             if (blk == 0 && arriver) {
                 state[ST_STATE_N_BUF0 + (ep ^ 1)] = n;
                 state[ST_STATE_N_ACTIVE] = n;
-                state[ST_STATE_N_CHANGED] = na;
+                state[ST_STATE_N_CHANGED] = n_changed;
                 state[ST_STATE_N_ADDED] = na;
                 state[ST_STATE_N_REMOVED] = nr;
                 state[ST_STATE_SERIAL] = serial_old + 1;
@@ -798,7 +925,7 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
         }
         if (arriver) arrival = atomicAdd(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), 1u);
     } else {
-        // ---- removals outnumber additions: the sequential part of the reference decides the order
+        // ---- too many surplus removals for the replay above: the per-index plan
         PlanView pv;
         cache_plan<true, TPB, true>(pv, smem, &plan_shared, new_mask, cur_mask2, indices2, state, I, I, tid,
                                            [] {}, [] {});

@@ -190,3 +190,56 @@ def test_fused_two_rows_of_x(dtype, H, I, has_gate):
         if t % 6 == 0:
             _same_state(fused, plain, t)
     _same_state(fused, plain, "end")
+
+
+@pytest.mark.parametrize("I,n0,hint_slack", [(4096, 2000, 0), (8192, 2867, 0), (512, 300, 0), (4096, 2000, -600)])
+def test_fused_surplus_removals(I, n0, hint_slack):
+    """More indices removed than added (weight_cache.h:310-353, swap with the last entry, one by one): the
+    fused kernel places the entries of the list's end in one go.  Surpluses of 1 .. I/4 and beyond (the
+    per-index plan takes over), removed indices drawn from all over the list, mostly from its end (surplus
+    indices that sit in the last positions themselves travel with earlier moves), or ONLY from its end;
+    with and without additions; a hint too low to fetch the list up front.  Order, counts, rows and output
+    against update followed by forward, and the order against the oracle."""
+    H, dtype = 1024, "float16"
+    rng = np.random.default_rng(I + n0)
+    m = np.zeros(I, bool)
+    m[rng.permutation(I)[:n0]] = True
+    fused, plain, (gate, up, down), g = _pair(I, H, dtype, True, 9, torch.from_numpy(m))
+    oc = oracle.OracleWeightCache(m, H, gate.float().numpy(), up.float().numpy(), down.float().numpy(), True)
+    x = torch.randn(1, H, generator=g).half().to(DEV)
+    plans = [(1, 0, "any"), (5, 3, "end"), (40, 40, "end"), (64, 10, "only_end"), (65, 0, "any"), (300, 50, "end"),
+             (I // 4, 0, "end"), (I // 4 + 1, 7, "any"), (17, 200, "only_end"), (2, 0, "only_end"), (120, 0, "only_end")]
+    for step, (surplus, added, where) in enumerate(plans):
+        order = oc.get_active_indices()
+        n = order.size
+        if n < n0 // 2:                  # grow the set back (additions only), then go on
+            grow = rng.permutation(np.flatnonzero(~m))[: n0 - n]
+            m = m.copy(); m[grow] = True
+            md = torch.from_numpy(m).to(DEV)
+            fused.update_and_forward(md, x, "silu"); plain.update_active_weights_async(md); oc.update_active_weights(m)
+            order = oc.get_active_indices(); n = order.size
+        surplus, added = min(surplus, n // 3), min(added, n // 8, I - n0)
+        k = surplus + added
+        if where == "any":
+            out = rng.choice(order, k, replace=False)
+        elif where == "end":          # three quarters of them from the last 2k positions
+            end = order[max(0, n - 2 * k):]
+            take = rng.choice(end, min(end.size, (3 * k) // 4), replace=False)
+            rest = np.setdiff1d(order, take)
+            out = np.concatenate([take, rng.choice(rest, k - take.size, replace=False)])
+        else:                         # all of them among the last positions
+            out = rng.choice(order[n - min(n, k + k // 4 + 1):], k, replace=False)
+        m = m.copy()
+        m[out] = False
+        m[rng.permutation(np.flatnonzero(~m & ~np.isin(np.arange(I), out)))[:added]] = True
+        md = torch.from_numpy(m).to(DEV)
+        hint = max(0, n + hint_slack)
+        yf = fused.update_and_forward(md, x, "silu", n_hint=hint)
+        plain.update_active_weights_async(md)
+        yp = plain.forward(x, "silu")
+        oc.update_active_weights(m)
+        torch.cuda.synchronize()
+        assert torch.equal(yf, yp), (step, surplus, added, where)
+        _same_state(fused, plain, (step, surplus, added, where))
+        assert fused.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist(), (step, where)
+        assert fused.sync_state()["n_removed"] - fused.sync_state()["n_added"] == surplus
