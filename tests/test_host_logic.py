@@ -117,3 +117,70 @@ def test_bench_refuses_more_than_one_gpu():
     p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                        timeout=120, cwd=root)
     assert p.returncode != 0 and "ONE GPU" in p.stderr
+
+
+def test_surplus_removal_closed_form():
+    """The closed form the fused update + decode kernel uses when removals outnumber additions, against the
+    reference's sequential rule (weight_cache.h:310-353: each surplus index, ascending, is replaced by the then-last
+    entry of the list).  With S surplus indices the list ends as its first n - S positions; step k moves the entry
+    of tail slot S-1-k to where the k-th surplus index sits at that time, which differs from its start position
+    only when that start lies in the tail: then it sits where the step that took its slot's entry put it."""
+    import oracle
+
+    def closed_form(order, surplus_sorted):
+        n, S = len(order), len(surplus_sorted)
+        base = n - S
+        rank = {e: k for k, e in enumerate(surplus_sorted)}
+        place = [None] * S                       # place[k]: where step k puts the entry it moves (None: nothing moves)
+        for p, e in enumerate(order):
+            if e in rank:
+                place[rank[e]] = p
+        for k in range(S):                       # only indices that start in the tail need the chase
+            pos = place[k]
+            while pos >= base and S - 1 - (pos - base) < k:
+                pos = place[S - 1 - (pos - base)]
+            place[k] = None if pos >= base and S - 1 - (pos - base) == k else pos
+        out = list(order)
+        for s in range(S):                       # every surviving tail entry on its own
+            if order[base + s] in rank:
+                continue
+            pos = place[S - 1 - s]
+            while pos >= base:
+                pos = place[S - 1 - (pos - base)]
+            out[pos] = order[base + s]
+        return out[:base]
+
+    rng = np.random.default_rng(0)
+    for trial in range(20000):
+        n = int(rng.integers(2, 48))
+        S = int(rng.integers(1, n))               # at least one index stays
+        I = 64
+        order = rng.permutation(I)[:n]
+        mask = np.zeros(I, bool)
+        mask[order] = True
+        # (an arbitrary order cannot be put into the oracle's cache directly: the sequential rule is restated here,
+        # and the closed form is checked against the oracle itself further down)
+        surplus = np.sort(rng.choice(order, S, replace=False))
+        lst, m = list(order), n
+        pos = {e: i for i, e in enumerate(lst)}
+        for e in surplus:
+            p, last = pos[e], m - 1
+            if p != last:
+                lst[p] = lst[last]
+                pos[lst[p]] = p
+            m -= 1
+        assert closed_form(list(order), list(surplus)) == lst[:m], (trial, order, surplus)
+    # the sequential rule itself against the oracle: removals only, from the ascending initial order
+    for trial in range(200):
+        I = 40
+        mask = rng.random(I) < 0.7
+        if mask.sum() < 3:
+            continue
+        w = np.zeros((I, 8), np.float32)
+        oc = oracle.OracleWeightCache(mask, 8, w, w, np.zeros((8, I), np.float32), True)
+        order = oc.get_active_indices().tolist()
+        drop = np.sort(rng.choice(order, int(rng.integers(1, len(order))), replace=False))
+        m2 = mask.copy()
+        m2[drop] = False
+        oc.update_active_weights(m2)
+        assert closed_form(order, list(drop)) == oc.get_active_indices().tolist(), trial
