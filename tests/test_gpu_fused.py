@@ -16,12 +16,12 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _pair(I, H, dtype, has_gate, seed, init_mask):
+def _pair(I, H, dtype, has_gate, seed, init_mask, std=0.05):
     g = torch.Generator().manual_seed(seed)
     tdt = getattr(torch, dtype)
-    gate = (torch.randn(I, H, generator=g) * 0.05).to(tdt)
-    up = (torch.randn(I, H, generator=g) * 0.05).to(tdt)
-    down = (torch.randn(H, I, generator=g) * 0.05).to(tdt)
+    gate = (torch.randn(I, H, generator=g) * std).to(tdt)
+    up = (torch.randn(I, H, generator=g) * std).to(tdt)
+    down = (torch.randn(H, I, generator=g) * std).to(tdt)
     mk = lambda: st.WeightCache(init_mask.to(DEV), H, gate.to(DEV) if has_gate else None, up.to(DEV), down.to(DEV),
                                 has_gate)
     return mk(), mk(), (gate, up, down), g
@@ -117,20 +117,43 @@ def test_fused_full_size_trace_and_errors():
     assert fused.get_num_active() == 100
 
 
-def test_fused_call_with_several_rows_takes_the_two_kernel_path():
-    H, I = 2048, 1024
-    trace = syn.ragged_mask_trace(3, I, 6)
-    fused, plain, _, g = _pair(I, H, "bfloat16", True, 1, torch.from_numpy(trace[0]))
-    x = torch.randn(4, H, generator=g).bfloat16().to(DEV)
+@pytest.mark.parametrize("dtype,H,I,B,has_gate", [
+    ("bfloat16", 2048, 1024, 4, True), ("float16", 3072, 8192, 3, True), ("float16", 3072, 8192, 16, True),
+    ("bfloat16", 4096, 14336, 8, True), ("float16", 4096, 11008, 4, False), ("bfloat16", 3072, 4096, 20, True),
+    ("float16", 2048, 4096, 32, False), ("float32", 2048, 1024, 4, True), ("float16", 1024, 4096, 4, True)])
+def test_fused_several_rows_of_x(dtype, H, I, B, has_gate):
+    """3 <= B <= 32 rows of x through update_and_forward (one C call that enqueues the update and the MFMA batch
+    kernels, or the streaming kernels where those do not apply, with the count read on the device).  Result,
+    combined buffer and the cache state equal the two separate calls, bit for bit, over a ragged trace (growth,
+    shrinkage with surplus removals, no-ops, tiny sets); order and output against the oracle at the end."""
+    trace = syn.ragged_mask_trace(3 + H + B, I, 14)
+    # (weights small enough that the outputs are O(1): the absolute tolerance of the 16-bit types assumes that)
+    fused, plain, (gate, up, down), g = _pair(I, H, dtype, has_gate, 1, torch.from_numpy(trace[0]), std=0.012)
+    tdt = getattr(torch, dtype)
+    ncol = (2 if has_gate else 1) * I
     for t in range(1, len(trace)):
         if not trace[t].any():
             continue
         m = torch.from_numpy(trace[t]).to(DEV)
-        yf = fused.update_and_forward(m, x, "relu")
+        x = torch.randn(B, H, generator=g).to(tdt).to(DEV)
+        comb_f = torch.zeros(B, ncol, dtype=tdt, device=DEV)
+        comb_p = torch.zeros_like(comb_f)
+        yf = fused.update_and_forward(m, x, "silu", combined=comb_f)
         plain.update_active_weights_async(m)
-        yp = plain.forward(x, "relu")
-        assert torch.equal(yf, yp), t
-    _same_state(fused, plain, "end")
+        yp = plain.forward(x, "silu", combined=comb_p)
+        torch.cuda.synchronize()
+        assert torch.equal(yf, yp), (t, (yf.float() - yp.float()).abs().max().item())
+        assert torch.equal(comb_f, comb_p), t
+        _same_state(fused, plain, t)
+    oc = oracle.OracleWeightCache(trace[0], H, gate.float().numpy() if has_gate else None, up.float().numpy(),
+                                  down.float().numpy(), has_gate)
+    for t in range(1, len(trace)):
+        if trace[t].any():
+            oc.update_active_weights(trace[t])
+    assert fused.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist()
+    want, _ = oracle.mlp_forward(x.float().cpu().numpy(), oc.get_concat_weight(), oc.get_active_down_weight(), "silu",
+                                 has_gate)
+    assert_close(yf.float().cpu().numpy(), want, dtype, "fused batch output vs oracle")
 
 
 @pytest.mark.parametrize("dtype,H,I,n0", [("float16", 3072, 8192, 2867), ("bfloat16", 4096, 4096, 400),
