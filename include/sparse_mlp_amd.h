@@ -193,13 +193,14 @@ enum st_state_word {
     ST_STATE_TICKET = 8,    /* internal: (epoch << 16) | blocks arrived in the running update */
     ST_STATE_N_BUF0 = 9,    /* internal: active count of bookkeeping buffer 0 */
     ST_STATE_N_BUF1 = 10,   /* internal: active count of bookkeeping buffer 1 */
-    ST_STATE_FAULT = 11,    /* sticky: a bounded in-kernel wait ran out (never expected); reported as ST_ERR_HIP */
+    ST_STATE_FAULT = 11,    /* reserved (no kernel waits on another block any more); nonzero is reported as ST_ERR_HIP */
     ST_STATE_WORDS = 16
 };
 
 typedef struct st_cache st_cache;
 
-/* Largest intermediate size the update kernel supports (its index maps live in LDS). */
+/* Largest intermediate size the update kernels support (32768: their plan lives in LDS -- index maps up to
+ * 22000, bitmaps with two index maps beyond; the reference has no bound, weight_cache.h:167). */
 int64_t st_cache_max_intermediate(void);
 
 /* host only.  weight_cache.h:148-194 (allocation is the caller's). */
@@ -228,10 +229,11 @@ int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream);
  * updated cache -- weight_cache.h:229-359 then sparse_mlp_op.cpp:53-192 /
  * src/modeling_skip.py:114-117, i.e. what SkipDecoderLayer.forward does per
  * layer (src/modeling_skip.py:234-261) -- enqueued as one call.  For B <= 2
- * (16-byte aligned rows, 8-byte aligned mask, I % 8 == 0) this is ONE kernel
- * that replays the bookkeeping and streams the active rows, taking rows whose
- * index changed from the pool and writing them back on the way; otherwise it
- * is st_cache_update_async followed by st_mlp_forward.  Either way the cache
+ * (16-byte aligned rows, 8-byte aligned mask, I % 8 == 0, I <= 16384) this is
+ * ONE kernel in which every block works out where the rows of the positions
+ * it owns come from and streams them, taking rows whose index changed from
+ * the pool and writing them back on the way; otherwise it is
+ * st_cache_update_async followed by st_mlp_forward.  Either way the cache
  * ends in the same state and `out` holds the same bits as the two separate
  * calls.  x, out: [B,H] in the cache's dtype; combined: [B,ldc] or NULL;
  * workspace: st_mlp_workspace_bytes(B, H, I) bytes.  n_hint: the active count

@@ -532,8 +532,10 @@ __global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const ui
 // ordered list and a slice of the remembered mask into the other bookkeeping
 // buffer; block 0 writes the state words; the last block to arrive flips the
 // epoch (as in cache_plan).
-// When removals outnumber additions (:310-353 is sequential) the block falls
-// back to cache_plan above, for that launch only.
+// When removals outnumber additions, the surplus ones are taken out one by
+// one in the reference (:310-353); their outcome is worked out in closed form
+// (see the kernel), or, for very many of them, by cache_plan above for that
+// launch only.
 // ---------------------------------------------------------------------------
 constexpr int kSparseMaxQ = 64;       // positions a block can own
 constexpr int kSparseMaxW32 = 512;    // mask words: I <= 16384
@@ -1620,7 +1622,7 @@ extern "C" int st_cache_sync_state(st_cache *c, int32_t *state_out, void *stream
     if (state_out)
         for (int i = 0; i < ST_STATE_WORDS; ++i) state_out[i] = c->host_state[i];
     if (c->host_state[ST_STATE_FAULT] != 0) {
-        set_error("st_cache: an in-kernel wait ran out; the cache contents are undefined");
+        set_error("st_cache: the fault word of the state is set; the cache contents are undefined");
         return ST_ERR_HIP;
     }
     if (c->host_state[ST_STATE_STATUS] == ST_ERR_NO_ACTIVE) {
