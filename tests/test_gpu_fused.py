@@ -215,7 +215,9 @@ def test_fused_two_rows_of_x(dtype, H, I, has_gate):
     _same_state(fused, plain, "end")
 
 
-@pytest.mark.parametrize("I,n0,hint_slack", [(4096, 2000, 0), (8192, 2867, 0), (512, 300, 0), (4096, 2000, -600)])
+@pytest.mark.parametrize("I,n0,hint_slack", [(4096, 2000, 0), (8192, 2867, 0), (512, 300, 0), (4096, 2000, -600),
+                                             # the largest size the fused kernel takes: 64 positions per block
+                                             (16384, 5000, 0)])
 def test_fused_surplus_removals(I, n0, hint_slack):
     """More indices removed than added (weight_cache.h:310-353, swap with the last entry, one by one): the
     fused kernel places the entries of the list's end in one go.  Surpluses of 1 .. I/4 and beyond (the
