@@ -98,6 +98,10 @@ def parse_args():
     ap.add_argument("--active-frac", type=float, default=0.0,
                     help="override the active fraction (e.g. the union of several rows' masks)")
     ap.add_argument("--churn", type=float, default=-1.0, help="override the fraction of the active set swapped per step")
+    ap.add_argument("--count-wobble", type=float, default=0.0,
+                    help="let the active count of every layer-step vary by this fraction around the workload's value "
+                         "(as a predictor's threshold would: some updates add more than they remove, others remove "
+                         "more); 0 keeps the count fixed, which is what the headline is quoted on")
     ap.add_argument("--prefill", type=int, default=0,
                     help="time the MFMA path instead: this many rows of x per step through the stack's sparse MLPs, "
                          "each cache at the union of the rows' masks (roofline against the dense MFMA peak)")
@@ -316,7 +320,8 @@ def main():
 
     stack, g = build_stack(wl, layers, B, args.seed, torch, st)
     T = W + K + 1
-    trace = torch.from_numpy(syn.mask_trace(args.seed + 7, layers, I, n, T, wl.churn_lo, wl.churn_hi)).to(dev)
+    trace = torch.from_numpy(syn.mask_trace(args.seed + 7, layers, I, n, T, wl.churn_lo, wl.churn_hi,
+                                             args.count_wobble)).to(dev)
     # predictor inputs per layer and step, MLP input of the first layer per step
     x_pred = torch.randn(T, layers, B, H, generator=g, device=dev, dtype=torch.float32).to(dt)
     x_in = torch.randn(T, B, H, generator=g, device=dev, dtype=torch.float32).to(dt)
@@ -479,7 +484,7 @@ def main():
         "dtype": {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[wl.dtype], "data": "synthetic",
         "config": {"workload": wl.name, "layers": layers, "hidden": H, "intermediate": I, "predictor_rank": wl.rank,
                    "batch": B, "act": wl.act, "has_gate": wl.has_gate, "n_active": n,
-                   "churn": [wl.churn_lo, wl.churn_hi], "mask_source": "trace",
+                   "churn": [wl.churn_lo, wl.churn_hi], "count_wobble": args.count_wobble, "mask_source": "trace",
                    "launch": "hip_graph" if use_graph else "eager",
                    "streams": 2 if args.overlap else 1, "update_fused_into_decode": bool(stack.fused),
                    "kernel_timing": "hip events stamped at kernel begin/end (hipExtLaunchKernelGGL), eager second pass"},

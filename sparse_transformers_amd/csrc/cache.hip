@@ -798,7 +798,8 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     // else the per-index plan.
     const int surplus = nr - na, tail_base = n_old - surplus;
     const int smax = (I >> 2) < TPB ? (I >> 2) : TPB;
-    bool replay = surplus > 0 && surplus <= smax && tail_base >= 0 && n_old <= scan_cap;
+    // (LDS behind the list of added indices: the fetched list, then five arrays of smax entries: 6.5 bytes per index at most)
+    bool replay = surplus > 0 && surplus <= smax && tail_base >= 0 && n_old <= scan_cap && I >= 256;
     constexpr uint16_t kGone = 0xffffu;   // hole[]: removed as the last entry, nothing moves; tailv[]: a surplus index
     uint16_t *const hole = scan_idx + ((scan_cap + 7) & ~7);   // start position of the k-th surplus index, then its place at step k
     uint16_t *const tailv = hole + ((smax + 7) & ~7);          // entry of tail slot j after the paired replacements
@@ -833,29 +834,65 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
             if (paired_tail) atomicAdd(&sh.paired_tail, paired_tail);
         }
         lds_barrier();
-        // ---- one wave: the places of the surplus indices that start in the tail, in ascending order
+        // ---- one wave: the places of the surplus indices that start in the tail.  An index's place depends on those
+        // of smaller surplus indices only, and only on such that start in the tail themselves (the others stay where
+        // they are), so they are resolved 64 at a time, one lane each, in rounds: a lane whose chase runs into an
+        // index that is not resolved yet tries again in the next round (the smallest unresolved one always gets
+        // through; two or three rounds as a rule).
         if (plan_wave) {
             const int S = __builtin_amdgcn_readfirstlane(surplus), base = __builtin_amdgcn_readfirstlane(tail_base);
+            uint16_t *const jlist = tailv + ((smax + 7) & ~7);   // [S] the surplus indices (their rank k) that start in the tail
+            uint16_t *const jrank = jlist + ((smax + 7) & ~7);   // [S] k -> position in jlist
+            uint16_t *const jres = jrank + ((smax + 7) & ~7);    // [S] k -> resolved place
             int in_tail = 0;
             for (int c = 0; c < S; c += kWave) {
                 const int k = c + lane;
-                uint64_t todo = __builtin_amdgcn_ballot_w64(k < S && (int)hole[k < S ? k : 0] >= base);
-                in_tail += __popcll(todo);
-                while (todo) {
-                    const int kk = c + (int)__builtin_ctzll(todo);
-                    todo &= todo - 1;
-                    int pos = hole[kk];
-                    int i = S - 1 - (pos - base);   // the step that takes the entry of that tail slot
-                    for (int it = 0; it < S && pos >= base && i >= 0 && i < kk; ++it) {
-                        pos = hole[i];
-                        i = S - 1 - (pos - base);
+                const bool is = k < S && (int)hole[k < S ? k : 0] >= base;
+                const uint64_t m = __builtin_amdgcn_ballot_w64(is);
+                if (is) {
+                    const int j = in_tail + __popcll(m & ((1ull << lane) - 1ull));
+                    jlist[j] = (uint16_t)k;
+                    jrank[k] = (uint16_t)j;
+                }
+                in_tail += __popcll(m);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+            for (int j0 = 0; j0 < in_tail; j0 += kWave) {
+                const int kk = j0 + lane < in_tail ? (int)jlist[j0 + lane] : -1;
+                bool open = kk >= 0;
+                uint64_t resolved = 0;   // lanes of this group that are done (the same in every lane)
+                int place = 0;
+                for (int round = 0; round <= kWave && __builtin_amdgcn_ballot_w64(open) != 0; ++round) {
+                    bool done = false;
+                    if (open) {
+                        int pos = hole[kk];
+                        for (int it = 0; it <= S; ++it) {
+                            const int i = S - 1 - (pos - base);   // the step that takes the entry of that tail slot
+                            if (pos < base || pos == (int)kGone || i > kk || i < 0) { done = true; break; }   // stays there
+                            if (i == kk) { pos = kGone; done = true; break; }   // it is the last entry at its own step
+                            const int h = hole[i];
+                            if (h < base) { pos = h; done = true; break; }      // travelled with an index that never moves
+                            const int j = jrank[i];
+                            if (j >= j0 && !((resolved >> (j - j0)) & 1ull)) break;   // not known yet: next round
+                            pos = jres[i];
+                        }
+                        place = pos;
                     }
-                    if (pos >= base && i == kk) pos = kGone;
-                    if (lane == 0) hole[kk] = (uint16_t)pos;
+                    const uint64_t now = __builtin_amdgcn_ballot_w64(open && done);
+                    if (open && done) jres[kk] = (uint16_t)place;
+                    resolved |= now;
+                    open = open && !done;
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
                     __builtin_amdgcn_wave_barrier();
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
                 }
+            }
+            // (hole[] kept the start positions until here: the chase tells the two kinds of surplus index apart by them)
+            for (int j = lane; j < in_tail; j += kWave) {
+                const int kk = jlist[j];
+                hole[kk] = jres[kk];
             }
             if (lane == 0) {
                 // (a surplus index missing from the list would make the counts disagree: per-index plan then)

@@ -67,21 +67,29 @@ def initial_mask(rng: np.random.Generator, intermediate: int, n_active: int) -> 
     return m
 
 
-def churn_step(rng: np.random.Generator, mask: np.ndarray, frac: float) -> np.ndarray:
-    """Swap round(frac * n) active indices for as many inactive ones (n stays constant)."""
+def churn_step(rng: np.random.Generator, mask: np.ndarray, frac: float, target: int = -1) -> np.ndarray:
+    """Swap round(frac * n) active indices for as many inactive ones (n stays constant); with `target` >= 0 the
+    count moves to `target` as well (more additions than removals, or the other way round)."""
     act = np.flatnonzero(mask)
     ina = np.flatnonzero(~mask)
     c = min(int(round(frac * act.size)), act.size, ina.size)
+    delta = 0 if target < 0 else int(target) - act.size
+    rem = min(act.size, c + max(0, -delta))
+    add = min(ina.size, c + max(0, delta))
     out = mask.copy()
-    if c > 0:
-        out[rng.choice(act, size=c, replace=False)] = False
-        out[rng.choice(ina, size=c, replace=False)] = True
+    if rem > 0:
+        out[rng.choice(act, size=rem, replace=False)] = False
+    if add > 0:
+        out[rng.choice(ina, size=add, replace=False)] = True
     return out
 
 
 def mask_trace(seed: int, layers: int, intermediate: int, n_active: int, steps: int, churn_lo: float,
-               churn_hi: float) -> np.ndarray:
-    """bool [steps, layers, I]: per layer a correlated mask sequence; churn ~ U(lo, hi) per layer-step."""
+               churn_hi: float, wobble: float = 0.0) -> np.ndarray:
+    """bool [steps, layers, I]: per layer a correlated mask sequence; churn ~ U(lo, hi) per layer-step.  With
+    `wobble` > 0 the count of every step is drawn from n_active * (1 + U(-wobble, wobble)) instead of staying at
+    n_active, as it does when a predictor's threshold drives the mask: additions outnumber removals in some steps
+    and removals outnumber additions in others."""
     rng = np.random.default_rng(seed)
     out = np.empty((steps, layers, intermediate), dtype=bool)
     for l in range(layers):
@@ -89,7 +97,11 @@ def mask_trace(seed: int, layers: int, intermediate: int, n_active: int, steps: 
         out[0, l] = m
         for t in range(1, steps):
             frac = churn_lo if churn_hi <= churn_lo else rng.uniform(churn_lo, churn_hi)
-            m = churn_step(rng, m, frac)
+            target = -1
+            if wobble > 0.0:
+                target = int(round(n_active * (1.0 + rng.uniform(-wobble, wobble))))
+                target = max(1, min(intermediate, target))
+            m = churn_step(rng, m, frac, target)
             out[t, l] = m
     return out
 
