@@ -295,6 +295,262 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
 }
 
 // ---------------------------------------------------------------------------
+// kernel 1, wide form: 256 rows of x by 64 gate + 64 up rows per block, operands straight into LDS
+// ---------------------------------------------------------------------------
+// The form above reads 8 KB of fragments from LDS for every 16 MFMAs of a wave (64 x 64 wave tiles), which at
+// the LDS's ~110 bytes per clock takes as long as the MFMAs themselves.  Here a wave owns a 128 x (32 + 32)
+// tile (12 KB of fragments per 32 MFMAs) and the two waves of a SIMD share one tile: wave kh takes the
+// kh-th 32 of every 64-wide K stage into accumulators of its own, and the pair is summed through LDS once
+// at the end.  The operands do not pass through registers on their way in: every wave issues its share of a
+// stage as 1 KB global -> LDS loads (lane i's 16 bytes land at base + 16 i, so the lane asks for the chunk
+// that belongs at that place of the swizzled row), two stages ahead into the third of three LDS buffers,
+// and only waits -- on the count of its own outstanding loads -- before the stage's barrier.
+constexpr int kPwBM = 256, kPwWR = 64, kPwThreads = 512, kPwBufs = 3;
+
+// s_waitcnt immediate: vmcnt in bits 3:0 (and 15:14), expcnt 6:4 left at "no wait", lgkmcnt 11:8 = 0
+#define ST_WAIT_VM_LGKM0(vm) __builtin_amdgcn_s_waitcnt(((vm) & 15) | (7 << 4) | (0 << 8) | (((vm) >> 4) << 14))
+
+template <typename T, bool HG>
+__global__ __launch_bounds__(kPwThreads) void prefill_gateup_wide_kernel(const T *__restrict__ X, int M, int H,
+                                                                         const T *__restrict__ gate,
+                                                                         const T *__restrict__ up, int n_host,
+                                                                         const int *__restrict__ n_dev,
+                                                                         T *__restrict__ Hh, long ldh,
+                                                                         T *__restrict__ comb, long ldc, int act,
+                                                                         int jt, int mt)
+{
+    constexpr int kRows = kPwBM + (HG ? 2 : 1) * kPwWR;   // LDS rows of one buffer: x, gate, up
+    constexpr int kBuf = kRows * kPfLd1;                  // 16-byte units per buffer
+    constexpr int kDma = kRows / 64;                      // 1 KB loads per wave and stage
+    constexpr int kGRow = kPwBM, kURow = kPwBM + (HG ? kPwWR : 0);
+    __shared__ uint4 lds[kPwBufs * kBuf];
+
+    const int n = device_count(n_host, n_dev);
+    const int n_pad = (n + kPfBK - 1) / kPfBK * kPfBK;
+    const int tile = xcd_tile_id(blockIdx.x, jt * mt);
+    if (tile < 0) return;
+    const int j0 = (tile / mt) * kPwWR, m0 = (tile % mt) * kPwBM;
+    if (j0 >= n_pad) return;
+    ST_TL(0);
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kh = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
+    const int l16 = lane & 15, q = lane >> 4;
+    const int fsw = pf_swz(l16);
+
+    // the wave's loads of a stage: load j fills LDS rows 8 L .. 8 L + 7 (L = kDma wave + j), lane i the
+    // position i % 8 of row i / 8, which holds chunk (i % 8) ^ pf_swz(row)
+    const char *dbase[kDma];
+    unsigned doff[kDma];
+#pragma unroll
+    for (int j = 0; j < kDma; ++j) {
+        const int L = wave * kDma + j;
+        const int r = 8 * L + (lane >> 3), c = (lane & 7) ^ pf_swz(r);
+        int g;
+        if (8 * L < kPwBM) {
+            g = m0 + r;
+            g = g < M ? g : M - 1;
+            dbase[j] = reinterpret_cast<const char *>(X);
+        } else {
+            const bool isg = HG && 8 * L < kURow;
+            g = j0 + r - (isg ? kGRow : kURow);
+            g = g < n ? g : (n > 0 ? n - 1 : 0);
+            dbase[j] = reinterpret_cast<const char *>(isg ? gate : up);
+        }
+        doff[j] = ((unsigned)g * (unsigned)H + (unsigned)c * 8u) * (unsigned)sizeof(T);
+    }
+    const int nk = H / kPfBK1;
+    const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint4 *)lds;
+    // The load is written out as an instruction: the compiler treats the builtin form as a store to LDS that
+    // every later LDS read has to wait for (vmcnt(0) right behind the loads), which is exactly what the
+    // three buffers are there to avoid; the waits are placed by hand below.
+    auto dma = [&](int stage, int b) __attribute__((always_inline)) {
+        const size_t k0 = (size_t)stage * kPfBK1 * sizeof(T);
+#pragma unroll
+        for (int j = 0; j < kDma; ++j) {
+            const unsigned dst = (unsigned)(b * kBuf + (wave * kDma + j) * 64) * 16u + lds_base;
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :
+                         : "s"(dst), "v"(doff[j]), "s"(dbase[j] + k0)
+                         : "memory");
+        }
+    };
+
+    f32x4_t ag[8][2], au[8][2];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            ag[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            au[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+    // fragments: the wave's k step of a stage is the kh-th 32 of its 64.  The 128 rows of x go through the MFMAs
+    // as four pairs of 16-row fragments, each pair against the wave's two gate and two up fragments.
+    struct FragB { uint4 g[2], u[2]; };
+    uint4 A[3][2];
+    FragB Bc, Bn;
+    auto rdA = [&](uint4 (&F)[2], int b, int pair) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            F[i] = lds[b * kBuf + (128 * wm + 32 * pair + 16 * i + l16) * kPfLd1 + ((4 * kh + q) ^ fsw)];
+    };
+    auto rdB = [&](FragB &F, int b) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if (HG) F.g[j] = lds[b * kBuf + (kGRow + 32 * wn + 16 * j + l16) * kPfLd1 + ((4 * kh + q) ^ fsw)];
+            F.u[j] = lds[b * kBuf + (kURow + 32 * wn + 16 * j + l16) * kPfLd1 + ((4 * kh + q) ^ fsw)];
+        }
+    };
+    auto mm = [&](const uint4 (&F)[2], const FragB &W, int pair) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                au[2 * pair + i][j] = Mfma<T>::run(F[i], W.u[j], au[2 * pair + i][j]);
+                if (HG) ag[2 * pair + i][j] = Mfma<T>::run(F[i], W.g[j], ag[2 * pair + i][j]);
+            }
+    };
+    // Stage s = base + u (3 divides base) sits in LDS buffer u, its first pair of x fragments in slot u of the
+    // ring of three.  The loads of stage s + 2 go out first, into the buffer every wave finished reading before
+    // the previous stage's barrier.  Every pair of x fragments is requested before the MFMAs of the pair ahead of
+    // it; the next stage's weight fragments and first pair follow the barrier (which follows the wait for this
+    // wave's own loads of that stage) and run under the MFMAs of the last pair (past the last stage they read
+    // a stale buffer and are not used).  The barrier is the bare instruction: __syncthreads() would also wait
+    // for the loads that are meant to stay in flight.
+    auto stage = [&](int u, int s) __attribute__((always_inline)) {
+        const int x = u, y = (u + 1) % 3, z = (u + 2) % 3;
+        const bool load = s + 2 < nk;
+        if (load) dma(s + 2, z);
+        rdA(A[y], u, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(A[x], Bc, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        rdA(A[z], u, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(A[y], Bc, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        rdA(A[x], u, 3);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(A[z], Bc, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (load) ST_WAIT_VM_LGKM0(kDma); else ST_WAIT_VM_LGKM0(0);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        rdB(Bn, y);
+        rdA(A[y], y, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(A[x], Bc, 3);
+        __builtin_amdgcn_sched_barrier(0);
+        Bc = Bn;
+    };
+
+    dma(0, 0);
+    if (nk > 1) dma(1, 1);
+    if (nk > 1) ST_WAIT_VM_LGKM0(kDma); else ST_WAIT_VM_LGKM0(0);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    rdB(Bc, 0);
+    rdA(A[0], 0, 0);
+    ST_TL(1);
+    int base = 0;
+    for (; base + 3 <= nk; base += 3) {
+        stage(0, base);
+        stage(1, base + 1);
+        stage(2, base + 2);
+    }
+    if (base < nk) {
+        stage(0, base);
+        if (base + 1 < nk) stage(1, base + 1);
+    }
+
+    ST_TL(2);
+    // The pair's sums: the wave with kh = 0 finishes the first 64 rows of the tile, the other the last 64; each
+    // hands the other half of its accumulators over through LDS (all stage buffers are free: the last stage ends
+    // behind its barrier with no fragment read outstanding).
+    constexpr int kQuads = (HG ? 2 : 1) * 8;   // accumulator quads per lane handed over
+    f32x4_t *red = reinterpret_cast<f32x4_t *>(lds);
+    f32x4_t fg[4][2], fu[4][2];
+    {
+        f32x4_t *mine = red + (size_t)wave * kQuads * 64 + lane;
+        auto hand = [&](int h) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    mine[(i * 2 + j) * 64] = au[4 * h + i][j];
+                    if (HG) mine[(8 + i * 2 + j) * 64] = ag[4 * h + i][j];
+                    fu[i][j] = au[4 * (1 - h) + i][j];
+                    if (HG) fg[i][j] = ag[4 * (1 - h) + i][j];
+                }
+        };
+        if (kh == 0) hand(1); else hand(0);
+    }
+    __syncthreads();
+    {
+        const f32x4_t *other = red + (size_t)(wave ^ 4) * kQuads * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                fu[i][j] += other[(i * 2 + j) * 64];
+                if (HG) fg[i][j] += other[(8 + i * 2 + j) * 64];
+            }
+    }
+    __syncthreads();
+
+    ST_TL(3);
+    // the wave's 64 x 32 results leave through a tile of its own in LDS as whole 16-byte chunks (see above)
+    constexpr int kSP = 32 + 8;
+    T *stg = reinterpret_cast<T *>(lds) + (size_t)wave * 64 * kSP;
+    const bool comb16 = comb && ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(comb) & 15) == 0;
+    const int mrow0 = m0 + 128 * wm + 64 * kh, colw = j0 + 32 * wn;
+    auto store = [&](auto actc) __attribute__((always_inline)) {
+        constexpr int ACT = decltype(actc)::value;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int col = colw + 16 * j + l16;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float hv = 0.f;
+                    if (col < n) hv = HG ? activate_fast(fg[i][j][e], ACT) * fu[i][j][e] : activate_fast(fu[i][j][e], ACT);
+                    stg[(16 * i + 4 * q + e) * kSP + 16 * j + l16] = from_float<T>(hv);
+                }
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int idx = lane + 64 * c, row = idx / 4, ch = idx % 4;
+            const int m = mrow0 + row, col0 = colw + 8 * ch;
+            if (m < M && col0 < n_pad) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(stg + row * kSP + 8 * ch);
+                *reinterpret_cast<uint4 *>(Hh + (size_t)m * ldh + col0) = v;
+                if (comb16 && col0 + 8 <= n) {
+                    *reinterpret_cast<uint4 *>(comb + (size_t)m * ldc + col0) = v;
+                } else if (comb) {
+                    const T *sv = stg + row * kSP + 8 * ch;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        if (col0 + k < n) comb[(size_t)m * ldc + col0 + k] = sv[k];
+                }
+            }
+        }
+    };
+    switch (act) {
+    case ST_ACT_RELU: store(std::integral_constant<int, ST_ACT_RELU>{}); break;
+    case ST_ACT_SILU: store(std::integral_constant<int, ST_ACT_SILU>{}); break;
+    case ST_ACT_GELU_TANH: store(std::integral_constant<int, ST_ACT_GELU_TANH>{}); break;
+    case ST_ACT_SIGMOID: store(std::integral_constant<int, ST_ACT_SIGMOID>{}); break;
+    default: store(std::integral_constant<int, ST_ACT_IDENTITY>{}); break;
+    }
+    ST_TL(4);
+}
+
+// ---------------------------------------------------------------------------
 // kernel 2: down projection
 // ---------------------------------------------------------------------------
 // Out[M,H] = Hh[M,n] Wd[n,H].  Wd's rows run along K, so its tile goes to LDS as it is ([k][column], whole
@@ -534,8 +790,8 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         ProfScope ps(ST_K_MLP_PREFILL_GATEUP, stream);
         const int cus = device_cu_count();
         const int jt64 = (int)(ldh / 64), mt128 = (M + 127) / 128;
-        // 256-row blocks with 64 + 64 weight rows (one per CU, 25 % less operand traffic) once 128-row tiles
-        // outnumber the CUs.  Below that the K loop of a block, not the chip, is what takes the time: two thread
+        // 256-row blocks with 64 + 64 weight rows (one per CU, 25 % less operand traffic; the wide kernel) once
+        // 128-row tiles outnumber the CUs.  Below that the K loop of a block, not the chip, is what takes the time: two thread
         // groups per tile with half of K each, on 128 x (64 + 64) tiles while those number more than half the
         // CUs and on 128 x (32 + 32) tiles (twice the blocks) when there are fewer -- four groups with a quarter
         // of K each on 64 x (32 + 32) tiles while those fit one per CU.  What is left (one row tile and more
@@ -555,7 +811,7 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
             return ST_OK;
         };
         int rc;
-        if (big) rc = has_gate ? go(prefill_gateup_kernel<T, true, 256, 2, 1, 2>, 512) : go(prefill_gateup_kernel<T, false, 256, 2, 1, 2>, 512);
+        if (big) rc = has_gate ? go(prefill_gateup_wide_kernel<T, true>, kPwThreads) : go(prefill_gateup_wide_kernel<T, false>, kPwThreads);
         else if (quarters) rc = has_gate ? go(prefill_gateup_kernel<T, true, 64, 2, 4, 1>, 512) : go(prefill_gateup_kernel<T, false, 64, 2, 4, 1>, 512);
         else if (halves) rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 2, 1>, 512) : go(prefill_gateup_kernel<T, false, 128, 2, 2, 1>, 512);
         else if (wide_halves) rc = has_gate ? go(prefill_gateup_kernel<T, true, 128, 2, 2, 2>, 512) : go(prefill_gateup_kernel<T, false, 128, 2, 2, 2>, 512);
