@@ -77,7 +77,9 @@ const char *st_last_error(void);
  * cover) runs the streaming decode kernel; 3 <= B <= 32 in fp16 / bf16 with H in
  * {2048, 3072, 4096} runs the MFMA batch kernels (still HBM-bound, one pass over
  * the weights); otherwise B >= 32 in fp16 / bf16 with H % 128 == 0
- * runs the MFMA GEMM kernels (then only columns [0,n) of `combined` are written).
+ * runs the MFMA GEMM kernels (then only columns [0,n) of `combined` carry results; when its rows are 16-byte
+ * aligned and have room, the kernels keep their intermediate there and also zero the columns from n up to the next
+ * multiple of 128).
  * ------------------------------------------------------------------------ */
 int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n);
 int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,

@@ -733,6 +733,242 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__
     }
 }
 
+// ---------------------------------------------------------------------------
+// kernel 2, wide form: 256 rows of Hh by 128 output columns per block and K split, operands straight into LDS
+// ---------------------------------------------------------------------------
+// The same scheme as prefill_gateup_wide_kernel: waves own 128 x 64 tiles, the two waves of a SIMD share a
+// tile (wave kh takes the kh-th 32 of every 64-wide K stage), operands arrive by 1 KB global -> LDS loads
+// two stages ahead into three buffers.  Wd's rows run along K and cannot be padded when they are loaded this
+// way (a load fills 1 KB of LDS back to back: four rows of 256 bytes), so the 16-byte chunks of row k are
+// XORed with 2 (k % 4 + 4 (k / 8 % 2)): the 8 rows x 32 bytes that half a wave hands to the transposing read
+// then cover every bank once.
+__device__ __forceinline__ int pf_swz_b(int k) { return 2 * ((k & 3) | (((k >> 3) & 1) << 2)); }
+
+template <typename T>
+__global__ __launch_bounds__(kPwThreads) void prefill_down_wide_kernel(const T *__restrict__ Hh, long ldh, int M,
+                                                                       const T *__restrict__ Wd, int H, int n_host,
+                                                                       const int *__restrict__ n_dev,
+                                                                       T *__restrict__ Out,
+                                                                       float *__restrict__ partial, int split_k,
+                                                                       int ct, int mt)
+{
+    constexpr int kABuf = kPwBM * kPfLd1;             // 16-byte units of the Hh tile of a stage (32 KB)
+    constexpr int kBuf = kABuf + kPfBK2 * 16;         // + 64 rows of Wd x 256 bytes (16 KB)
+    constexpr int kDma = 6;                           // 1 KB loads per wave and stage
+    __shared__ uint4 lds[kPwBufs * kBuf];
+
+    const int n = device_count(n_host, n_dev);
+    const int tile = xcd_tile_id(blockIdx.x, ct * mt * split_k);   // row tiles fastest, then column tiles, then splits
+    if (tile < 0) return;
+    const int z = tile / (ct * mt), c0 = ((tile / mt) % ct) * kPfBN, m0 = (tile % mt) * kPwBM;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kh = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
+    const int l16 = lane & 15, q = lane >> 4;
+    const int fsw = pf_swz(l16);
+
+    // K range of this split, in stages of 64 (Hh is zero-padded to a multiple of 128 columns)
+    const int nst_all = (n + kPfBK - 1) / kPfBK * (kPfBK / kPfBK2);
+    const int per = (nst_all + split_k - 1) / split_k;
+    const int ks0 = z * per, ks1 = (ks0 + per < nst_all) ? ks0 + per : nst_all;
+    const int nst = ks1 - ks0;
+
+    // the wave's loads of a stage: loads L = 6 wave + j; L < 32 fills rows 8 L .. 8 L + 7 of the Hh tile (lane i the
+    // position i % 8 of row i / 8), L >= 32 rows 4 (L - 32) .. + 3 of the Wd tile (position i % 16 of row i / 16)
+    const char *dbase[kDma];
+    unsigned doff[kDma];
+    size_t dstep[kDma];
+#pragma unroll
+    for (int j = 0; j < kDma; ++j) {
+        const int L = wave * kDma + j;
+        if (L < 32) {
+            const int r = 8 * L + (lane >> 3), c = (lane & 7) ^ pf_swz(r);
+            int g = m0 + r;
+            g = g < M ? g : M - 1;
+            dbase[j] = reinterpret_cast<const char *>(Hh) + (size_t)ks0 * kPfBK2 * sizeof(T);
+            doff[j] = (unsigned)((size_t)g * ldh * sizeof(T)) + (unsigned)c * 16u;
+            dstep[j] = kPfBK2 * sizeof(T);
+        } else {
+            const int k = 4 * (L - 32) + (lane >> 4), c = (lane & 15) ^ pf_swz_b(k);
+            dbase[j] = reinterpret_cast<const char *>(Wd + c0) + (size_t)ks0 * kPfBK2 * H * sizeof(T);
+            doff[j] = (unsigned)k * (unsigned)H * (unsigned)sizeof(T) + (unsigned)c * 16u;
+            dstep[j] = (size_t)kPfBK2 * H * sizeof(T);
+        }
+    }
+    const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint4 *)lds;
+    // Rows of Wd at or beyond n (they meet the zero padding of Hh, but stale rows may hold anything, and
+    // 0 * inf is not 0) are replaced by the last valid row, whose products with the padding are zeros as
+    // long as the weights are finite; only a split's last stages can reach them.
+    auto dma = [&](int stage, int b, bool check) __attribute__((always_inline)) {
+        const bool past = check && (ks0 + stage + 1) * kPfBK2 > n;   // uniform
+#pragma unroll
+        for (int j = 0; j < kDma; ++j) {
+            const unsigned dst = (unsigned)(b * kBuf + (wave * kDma + j) * 64) * 16u + lds_base;
+            const char *src = dbase[j] + (size_t)stage * dstep[j];
+            unsigned off = doff[j];
+            if (past && wave * kDma + j >= 32) {   // uniform: a load of Wd rows
+                const int kt = 4 * (wave * kDma + j - 32) + (lane >> 4), k = (ks0 + stage) * kPfBK2 + kt;
+                const int kc = k < n ? k : (n > 0 ? n - 1 : 0);
+                src = reinterpret_cast<const char *>(Wd + c0);
+                off = (unsigned)kc * (unsigned)H * (unsigned)sizeof(T) + (unsigned)((lane & 15) ^ pf_swz_b(kt)) * 16u;
+            }
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(off), "s"(src) : "memory");
+        }
+    };
+
+    f32x4_t acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    uint4 A[3][2], Bc[4], Bn[4];
+    auto rdA = [&](uint4 (&F)[2], int b, int pair) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            F[i] = lds[b * kBuf + (128 * wm + 32 * pair + 16 * i + l16) * kPfLd1 + ((4 * kh + q) ^ fsw)];
+    };
+    // B fragments through the transposing read: in a group of 16 lanes, lane j hands in the address of four
+    // consecutive columns of row j / 4 and lane i receives column i of the four rows
+    const int bsw = 2 * ((l16 >> 2) | ((q & 1) << 2));   // pf_swz_b of the rows this lane hands in
+    auto rdB = [&](uint4 (&F)[4], int b) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            pf_v4i16_t h[2];
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const int k = 32 * kh + 8 * q + 4 * hh + (l16 >> 2);
+                const int col = 64 * wn + 16 * j + 4 * (l16 & 3);
+                const unsigned short *p16 =
+                    reinterpret_cast<const unsigned short *>(&lds[b * kBuf + kABuf + k * 16 + ((col >> 3) ^ bsw)]) + (col & 7);
+                h[hh] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) pf_v4i16_t *)p16);
+            }
+            typedef short v8i16_t __attribute__((ext_vector_type(8)));
+            F[j] = __builtin_bit_cast(uint4, (v8i16_t)__builtin_shufflevector(h[0], h[1], 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+    };
+    auto mm = [&](const uint4 (&F)[2], const uint4 (&W)[4], int pair) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[2 * pair + i][j] = Mfma<T>::run(F[i], W[j], acc[2 * pair + i][j]);
+    };
+    // One stage, as in prefill_gateup_wide_kernel.  `check` is false in the main loop, whose stages all have loads
+    // to issue and none of them touches rows of Wd at or beyond n.
+    auto stage = [&](int u, int s, bool check) __attribute__((always_inline)) {
+        const int x = u, y = (u + 1) % 3, zz = (u + 2) % 3;
+        const bool load = !check || s + 2 < nst;
+        if (load) dma(s + 2, zz, check);
+        rdA(A[y], u, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(A[x], Bc, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        rdA(A[zz], u, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(A[y], Bc, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        rdA(A[x], u, 3);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(A[zz], Bc, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (load) ST_WAIT_VM_LGKM0(kDma); else ST_WAIT_VM_LGKM0(0);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        rdB(Bn, y);
+        rdA(A[y], y, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(A[x], Bc, 3);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) Bc[j] = Bn[j];
+    };
+
+    if (nst > 0) {
+        dma(0, 0, true);
+        if (nst > 1) dma(1, 1, true);
+        if (nst > 1) ST_WAIT_VM_LGKM0(kDma); else ST_WAIT_VM_LGKM0(0);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        rdB(Bc, 0);
+        rdA(A[0], 0, 0);
+        int nsafe = n / kPfBK2 - ks0;   // stages of this split that lie below row n as a whole
+        nsafe = nsafe < nst ? nsafe : nst;
+        int base = 0;
+        for (; base + 5 <= nsafe; base += 3) {
+            stage(0, base, false);
+            stage(1, base + 1, false);
+            stage(2, base + 2, false);
+        }
+        for (; base < nst; base += 3) {
+            stage(0, base, true);
+            if (base + 1 < nst) stage(1, base + 1, true);
+            if (base + 2 < nst) stage(2, base + 2, true);
+        }
+    }
+
+    // the pair's sums (see prefill_gateup_wide_kernel): kh = 0 finishes the first 64 rows of the tile, kh = 1 the last
+    f32x4_t *red = reinterpret_cast<f32x4_t *>(lds);
+    f32x4_t f[4][4];
+    {
+        f32x4_t *mine = red + (size_t)wave * 16 * 64 + lane;
+        auto hand = [&](int h) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    mine[(i * 4 + j) * 64] = acc[4 * h + i][j];
+                    f[i][j] = acc[4 * (1 - h) + i][j];
+                }
+        };
+        if (kh == 0) hand(1); else hand(0);
+    }
+    __syncthreads();
+    {
+        const f32x4_t *other = red + (size_t)(wave ^ 4) * 16 * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) f[i][j] += other[(i * 4 + j) * 64];
+    }
+    __syncthreads();
+
+    const int mrow0 = m0 + 128 * wm + 64 * kh, colw = c0 + 64 * wn;
+    if (split_k == 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = colw + 16 * j + l16;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int m = mrow0 + 16 * i + 4 * q + e;
+                    if (m < M && col < H) Out[(size_t)m * H + col] = from_float<T>(f[i][j][e]);
+                }
+            }
+        return;
+    }
+    // partial sums leave through a tile of the wave's own in LDS as 16-byte chunks, 256 bytes of a row per 16 lanes
+    constexpr int kSP = 64 + 4;   // floats per staged row
+    static_assert(8 * 64 * kSP * 4 <= (int)sizeof(lds), "staging tiles exceed the stage buffers");
+    float *stg = reinterpret_cast<float *>(lds) + (size_t)wave * 64 * kSP;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) stg[(16 * i + 4 * q + e) * kSP + 16 * j + l16] = f[i][j][e];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+        const int row = 4 * c + q, m = mrow0 + row, col = colw + 4 * l16;
+        if (m < M && col < H)
+            *reinterpret_cast<float4 *>(partial + ((size_t)z * M + m) * H + col) =
+                *reinterpret_cast<const float4 *>(stg + row * kSP + 4 * l16);
+    }
+}
+
 // out[m, c] = sum over splits of partial[z][m][c]
 template <typename T>
 __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__restrict__ partial, int split_k, int M,
@@ -767,6 +1003,25 @@ int prefill_split_k(int M, int H, int n)
     return best;
 }
 
+// The wide down kernel: 256-row tiles, one block per CU.  Taken when the row tiles waste at most a fifth of
+// their rows; the K split then fills the CUs (at least 8 stages of 64 per split, at most 16 splits).
+static bool prefill_down_is_wide(int M, int H, int n, long ldh)
+{
+    const int mt = (M + kPwBM - 1) / kPwBM;
+    return M > 128 && (mt * kPwBM - M) * 5 <= mt * kPwBM && H % kPfBN == 0 && n >= 512 &&
+           (int64_t)M * ldh * 2 < ((int64_t)1 << 32);
+}
+
+static int prefill_split_k_wide(int M, int H, int n)
+{
+    const int tiles = ((M + kPwBM - 1) / kPwBM) * ((H + kPfBN - 1) / kPfBN);
+    const int nk = (n + kPfBK - 1) / kPfBK * (kPfBK / kPfBK2);
+    int s = device_cu_count() / tiles;
+    if (s > nk / 8) s = nk / 8;
+    if (s > 16) s = 16;
+    return s < 1 ? 1 : s;
+}
+
 int64_t prefill_ldh(int64_t n) { return (n + kPfBK - 1) / kPfBK * kPfBK; }
 
 int64_t prefill_workspace_bytes(int64_t M, int64_t H, int64_t n)
@@ -781,15 +1036,22 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
                             const int *n_dev, void *out, void *comb, long ldc, void *workspace, int act, int has_gate,
                             hipStream_t stream)
 {
-    const long ldh = (long)prefill_ldh(n);
-    T *Hh = static_cast<T *>(workspace);
-    const int64_t hh_bytes = (((int64_t)M * ldh * 2) + 255) & ~(int64_t)255;
+    // The intermediate Hh normally sits in the workspace, padded with zero columns to a multiple of 128.  When the
+    // caller's combined buffer can take that padding (16-byte aligned rows with room up to the padded width) the
+    // gate/up kernel writes there only and the down kernel reads it back from there: one store of M x n less.
+    const long ldw = (long)prefill_ldh(n);
+    const bool alias = comb && ldc % 8 == 0 && ldc >= ldw && (reinterpret_cast<uintptr_t>(comb) & 15) == 0;
+    const long ldh = alias ? ldc : ldw;
+    T *Hh = alias ? static_cast<T *>(comb) : static_cast<T *>(workspace);
+    if (alias) comb = nullptr;
+    const int64_t hh_bytes = (((int64_t)M * ldw * 2) + 255) & ~(int64_t)255;
     float *partial = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + hh_bytes);
-    const int split_k = prefill_split_k(M, H, n);
+    const bool wide_down = prefill_down_is_wide(M, H, n, ldh);
+    const int split_k = wide_down ? prefill_split_k_wide(M, H, n) : prefill_split_k(M, H, n);
     {
         ProfScope ps(ST_K_MLP_PREFILL_GATEUP, stream);
         const int cus = device_cu_count();
-        const int jt64 = (int)(ldh / 64), mt128 = (M + 127) / 128;
+        const int jt64 = (int)(ldw / 64), mt128 = (M + 127) / 128;
         // 256-row blocks with 64 + 64 weight rows (one per CU, 25 % less operand traffic; the wide kernel) once
         // 128-row tiles outnumber the CUs.  Below that the K loop of a block, not the chip, is what takes the time: two thread
         // groups per tile with half of K each, on 128 x (64 + 64) tiles while those number more than half the
@@ -821,10 +1083,17 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
     ST_HIP(hipGetLastError());
     {
         ProfScope ps(ST_K_MLP_PREFILL_DOWN, stream);
-        const int ct = (H + kPfBN - 1) / kPfBN, mt = (M + kPfBM - 1) / kPfBM;
-        const int grid = (ct * mt * split_k + kXcds - 1) / kXcds * kXcds;
-        ST_LAUNCH(ps, prefill_down_kernel<T>, dim3(grid), dim3(kPfThreads), 0, stream, Hh, ldh, M,
-                           static_cast<const T *>(down), H, n, n_dev, static_cast<T *>(out), partial, split_k, ct, mt);
+        if (wide_down) {
+            const int ct = (H + kPfBN - 1) / kPfBN, mt = (M + kPwBM - 1) / kPwBM;
+            const int grid = (ct * mt * split_k + kXcds - 1) / kXcds * kXcds;
+            ST_LAUNCH(ps, prefill_down_wide_kernel<T>, dim3(grid), dim3(kPwThreads), 0, stream, Hh, ldh, M,
+                      static_cast<const T *>(down), H, n, n_dev, static_cast<T *>(out), partial, split_k, ct, mt);
+        } else {
+            const int ct = (H + kPfBN - 1) / kPfBN, mt = (M + kPfBM - 1) / kPfBM;
+            const int grid = (ct * mt * split_k + kXcds - 1) / kXcds * kXcds;
+            ST_LAUNCH(ps, prefill_down_kernel<T>, dim3(grid), dim3(kPfThreads), 0, stream, Hh, ldh, M,
+                      static_cast<const T *>(down), H, n, n_dev, static_cast<T *>(out), partial, split_k, ct, mt);
+        }
     }
     ST_HIP(hipGetLastError());
     if (split_k > 1) {
