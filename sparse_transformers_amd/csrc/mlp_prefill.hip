@@ -761,6 +761,7 @@ __global__ __launch_bounds__(kPwThreads) void prefill_down_wide_kernel(const T *
     const int tile = xcd_tile_id(blockIdx.x, ct * mt * split_k);   // row tiles fastest, then column tiles, then splits
     if (tile < 0) return;
     const int z = tile / (ct * mt), c0 = ((tile / mt) % ct) * kPfBN, m0 = (tile % mt) * kPwBM;
+    ST_TL(0);
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kh = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
     const int l16 = lane & 15, q = lane >> 4;
@@ -891,6 +892,7 @@ __global__ __launch_bounds__(kPwThreads) void prefill_down_wide_kernel(const T *
         asm volatile("" ::: "memory");
         rdB(Bc, 0);
         rdA(A[0], 0, 0);
+        ST_TL(1);
         int nsafe = n / kPfBK2 - ks0;   // stages of this split that lie below row n as a whole
         nsafe = nsafe < nst ? nsafe : nst;
         int base = 0;
@@ -906,6 +908,7 @@ __global__ __launch_bounds__(kPwThreads) void prefill_down_wide_kernel(const T *
         }
     }
 
+    ST_TL(2);
     // the pair's sums (see prefill_gateup_wide_kernel): kh = 0 finishes the first 64 rows of the tile, kh = 1 the last
     f32x4_t *red = reinterpret_cast<f32x4_t *>(lds);
     f32x4_t f[4][4];
@@ -932,6 +935,7 @@ __global__ __launch_bounds__(kPwThreads) void prefill_down_wide_kernel(const T *
     }
     __syncthreads();
 
+    ST_TL(3);
     const int mrow0 = m0 + 128 * wm + 64 * kh, colw = c0 + 64 * wn;
     if (split_k == 1) {
 #pragma unroll
@@ -967,6 +971,7 @@ __global__ __launch_bounds__(kPwThreads) void prefill_down_wide_kernel(const T *
             *reinterpret_cast<float4 *>(partial + ((size_t)z * M + m) * H + col) =
                 *reinterpret_cast<const float4 *>(stg + row * kSP + 4 * l16);
     }
+    ST_TL(4);
 }
 
 // out[m, c] = sum over splits of partial[z][m][c]

@@ -211,9 +211,14 @@ def test_prefill_agrees_with_decode_kernel():
     ("ragged rows and columns, K loop with whole groups and a tail", 300, 1152, 6000, "bfloat16", "silu", True),
     ("ungated, K loop shorter than one group", 260, 256, 8500, "float16", "relu", False),
     ("llama-3b prefill, every row active", 512, 3072, 8192, "bfloat16", "silu", True),
+    ("ragged 256-row tile through both wide kernels, intermediate kept in the combined buffer", 448, 1024, 4096, "float16", "silu", True),
+    ("the same with an odd count: combined rows not 16-byte aligned, intermediate in the workspace", 448, 1024, 3001, "bfloat16", "silu", True),
+    ("ungated, combined buffer exactly as wide as the padded intermediate", 512, 512, 5120, "float16", "relu", False),
+    ("more 256-row tiles than CUs: down projection without a K split", 2800, 3072, 640, "bfloat16", "silu", True),
 ])
 def test_prefill_wide_blocks(name, M, H, n, dtype, act, has_gate):
-    """With more 128-row tiles than CUs the gate/up kernel switches to 256-row blocks.  The oracle checks the
+    """With more 128-row tiles than CUs the gate/up kernel switches to 256-row blocks, and from 256 rows on the down
+    projection to 256-row tiles with the K range split over the CUs.  The oracle checks the
     first and the last rows (a full and a ragged row tile); every row is compared with the streaming decode
     kernel, which the tests above hold against the oracle."""
     x, cw, dn = _case(23, M, H, n, dtype, has_gate)
