@@ -191,7 +191,7 @@ def prefill_bench(args, wl, torch, st, _lib, syn):
                    "active_rows_mean": m["n_mean"], "act": wl.act, "has_gate": wl.has_gate},
         "roofline": {"bound": "mfma", "achieved": round(m["achieved_tflops"], 1), "peak": MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(m["achieved_tflops"] / MFMA_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "prefill_gateup_kernel", "flops_per_launch": m["gu_flops"], "mean_us": m["gu_us"]},
+                     "kernel": "prefill_gateup_wide_kernel", "flops_per_launch": m["gu_flops"], "mean_us": m["gu_us"]},
         "stack_tflops": round(m["stack_tflops"], 1),
         "kernels_us": m["kernels_us"],
     }
@@ -516,7 +516,7 @@ def main():
             result["prefill_512"] = {
                 "layers": pl, "rows": 512, "active_rows_mean": m["n_mean"], "tok_s": round(512 / (m["ms_per_step"] * 1e-3), 1),
                 "us_per_layer": round(m["ms_per_step"] * 1e3 / pl, 2), "stack_tflops": round(m["stack_tflops"], 1),
-                "roofline": {"bound": "mfma", "kernel": "prefill_gateup_kernel", "achieved": round(m["achieved_tflops"], 1),
+                "roofline": {"bound": "mfma", "kernel": "prefill_gateup_wide_kernel", "achieved": round(m["achieved_tflops"], 1),
                              "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                              "frac": round(m["achieved_tflops"] / MFMA_PEAK_TFLOPS, 4), "mean_us": m["gu_us"]},
                 "kernels_us": m["kernels_us"]}

@@ -215,6 +215,7 @@ def test_prefill_agrees_with_decode_kernel():
     ("the same with an odd count: combined rows not 16-byte aligned, intermediate in the workspace", 448, 1024, 3001, "bfloat16", "silu", True),
     ("ungated, combined buffer exactly as wide as the padded intermediate", 512, 512, 5120, "float16", "relu", False),
     ("more 256-row tiles than CUs: down projection without a K split", 2800, 3072, 640, "bfloat16", "silu", True),
+    ("two K stages in gate/up; down projection with splits that have nothing to do", 512, 128, 8200, "float16", "silu", True),
 ])
 def test_prefill_wide_blocks(name, M, H, n, dtype, act, has_gate):
     """With more 128-row tiles than CUs the gate/up kernel switches to 256-row blocks, and from 256 rows on the down
