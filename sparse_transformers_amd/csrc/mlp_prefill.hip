@@ -10,9 +10,11 @@
 //             down columns, i.e. K runs down the rows: the tile sits in LDS
 //             as [k][column] and the fragments are read with the
 //             transposing LDS load (ds_read_b64_tr_b16)
-// Kernel 1: 128 or 256 rows of x by 64 active rows of gate and of up per block; kernel 2: block tile
-// 128 x 128 with split-K.  Both: waves of 64 x 64, K stages of 64 through two LDS buffers with the
-// following stages' global loads held in registers, one barrier per stage.
+// Each kernel has two forms.  The first (kernel 1: 64 or 128 rows of x by 32 or 64 active rows of gate and of up
+// per block; kernel 2: block tile 128 x 128 with split-K) has waves of 64 x 64 and K stages of 64 through two LDS
+// buffers with the following stages' global loads held in registers, one barrier per stage; it serves the shapes
+// whose tiles do not fill the chip.  The wide form (256 x 128 block tiles, waves of 128 x 64 whose K the two waves
+// of a SIMD share, operands loaded global -> LDS directly through three buffers) takes over when they do.
 //
 // The reference only runs the sparse path for decode (src/modeling_skip.py:236);
 // this is the same contraction as sparse_mlp_forward_cpu
@@ -39,6 +41,114 @@ __device__ __forceinline__ int xcd_tile_id(int bid, int ntiles)
     const int per = (ntiles + kXcds - 1) / kXcds;
     const int t = (bid % kXcds) * per + bid / kXcds;
     return (bid / kXcds < per && t < ntiles) ? t : -1;
+}
+
+// ---------------------------------------------------------------------------
+// epilogues shared by the two forms of each kernel
+// ---------------------------------------------------------------------------
+// D[m][j] of a 16 x 16 MFMA block: a lane holds rows 4 q + e (e = 0..3) of column l16.
+//
+// Kernel 1: the activation on a wave's 64 x 16 JN gate / up sums, and the product stored into Hh (and `comb`).
+// Columns n .. n_pad are written as zeros so that kernel 2 can run whole K stages.  The results go through a tile
+// of the wave's own in LDS (`stg`, 64 rows of 16 JN + 8 elements; the stage buffers are free by then) and leave as
+// whole 16-byte chunks, 64 bytes of a row per four lanes; storing every element by itself took 5.2 us of the 57
+// the kernel ran.
+template <typename T, bool HG, int JN, int ACT>
+__device__ __forceinline__ void pf_store_hidden_as(const f32x4_t (&ag)[4][JN], const f32x4_t (&au)[4][JN], T *stg,
+                                                   int lane, int mrow0, int colw, int M, int n, int n_pad, T *Hh,
+                                                   long ldh, T *comb, long ldc)
+{
+    constexpr int kSP = 16 * JN + 8;   // elements per staged row (16-byte multiple, spreads the banks)
+    const int l16 = lane & 15, q = lane >> 4;
+    const bool comb16 = comb && ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(comb) & 15) == 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < JN; ++j) {
+            const int col = colw + 16 * j + l16;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float hv = 0.f;
+                if (col < n) hv = HG ? activate_fast(ag[i][j][e], ACT) * au[i][j][e] : activate_fast(au[i][j][e], ACT);
+                stg[(16 * i + 4 * q + e) * kSP + 16 * j + l16] = from_float<T>(hv);
+            }
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int c = 0; c < 2 * JN; ++c) {
+        const int idx = lane + 64 * c, row = idx / (2 * JN), ch = idx % (2 * JN);
+        const int m = mrow0 + row, col0 = colw + 8 * ch;
+        if (m < M && col0 < n_pad) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(stg + row * kSP + 8 * ch);
+            *reinterpret_cast<uint4 *>(Hh + (size_t)m * ldh + col0) = v;
+            if (comb16 && col0 + 8 <= n) {
+                *reinterpret_cast<uint4 *>(comb + (size_t)m * ldc + col0) = v;
+            } else if (comb) {
+                const T *sv = stg + row * kSP + 8 * ch;
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    if (col0 + k < n) comb[(size_t)m * ldc + col0 + k] = sv[k];
+            }
+        }
+    }
+}
+
+// One copy per activation, chosen once per block: with the activation switched per element the whole kernel was
+// 4 us slower (all five bodies live in the loop's register budget).
+template <typename T, bool HG, int JN>
+__device__ __forceinline__ void pf_store_hidden(int act, const f32x4_t (&ag)[4][JN], const f32x4_t (&au)[4][JN], T *stg,
+                                                int lane, int mrow0, int colw, int M, int n, int n_pad, T *Hh, long ldh,
+                                                T *comb, long ldc)
+{
+    switch (act) {
+    case ST_ACT_RELU: pf_store_hidden_as<T, HG, JN, ST_ACT_RELU>(ag, au, stg, lane, mrow0, colw, M, n, n_pad, Hh, ldh, comb, ldc); break;
+    case ST_ACT_SILU: pf_store_hidden_as<T, HG, JN, ST_ACT_SILU>(ag, au, stg, lane, mrow0, colw, M, n, n_pad, Hh, ldh, comb, ldc); break;
+    case ST_ACT_GELU_TANH: pf_store_hidden_as<T, HG, JN, ST_ACT_GELU_TANH>(ag, au, stg, lane, mrow0, colw, M, n, n_pad, Hh, ldh, comb, ldc); break;
+    case ST_ACT_SIGMOID: pf_store_hidden_as<T, HG, JN, ST_ACT_SIGMOID>(ag, au, stg, lane, mrow0, colw, M, n, n_pad, Hh, ldh, comb, ldc); break;
+    default: pf_store_hidden_as<T, HG, JN, ST_ACT_IDENTITY>(ag, au, stg, lane, mrow0, colw, M, n, n_pad, Hh, ldh, comb, ldc); break;
+    }
+}
+
+// Kernel 2: a wave's 64 x 64 sums, either straight into Out (no K split) or as fp32 partial sums of split z through
+// a tile of the wave's own in LDS (`stg`, 64 rows of 68 floats), 256 bytes of a row per 16 lanes.
+constexpr int kPfStgF = 64 + 4;   // floats per staged row
+template <typename T>
+__device__ __forceinline__ void pf_store_out(const f32x4_t (&f)[4][4], float *stg, int lane, int mrow0, int colw, int M,
+                                             int H, T *Out, float *partial_z)
+{
+    const int l16 = lane & 15, q = lane >> 4;
+    if (!partial_z) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = colw + 16 * j + l16;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int m = mrow0 + 16 * i + 4 * q + e;
+                    if (m < M && col < H) Out[(size_t)m * H + col] = from_float<T>(f[i][j][e]);
+                }
+            }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) stg[(16 * i + 4 * q + e) * kPfStgF + 16 * j + l16] = f[i][j][e];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+        const int row = 4 * c + q, m = mrow0 + row, col = colw + 4 * l16;
+        if (m < M && col < H)
+            *reinterpret_cast<float4 *>(partial_z + (size_t)m * H + col) =
+                *reinterpret_cast<const float4 *>(stg + row * kPfStgF + 4 * l16);
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -237,60 +347,12 @@ __global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__
                     }
     }
 
-    // D[m][j]: lane holds rows 4*q + e (e = 0..3) of column l16 in every 16 x 16 block.
-    // Columns n .. n_pad are written as zeros so that kernel 2 can run whole K stages.
-    // The wave's 64 x 16 JN results go through a tile of its own in LDS (free now: the stage loops end with a
-    // barrier) and leave as whole 16-byte chunks, 64 bytes of a row per four lanes; storing every element by
-    // itself took 5.2 us of the 57 the kernel ran.
-    // One copy per activation, chosen once: with the activation switched per element the whole kernel was
-    // 4 us slower (all five bodies live in the loop's register budget).
-    constexpr int kSP = 16 * JN + 8;   // elements per staged row (16-byte multiple, spreads the banks)
+    // the stage loops end with a barrier, so the buffers are free for the epilogue's tiles
+    constexpr int kSP = 16 * JN + 8;
     constexpr size_t kStgOff = KS > 1 ? (size_t)(KS - 1) * kWG * kRedWave * (4 / sizeof(T)) : 0;   // past the sums
     static_assert((kStgOff + (size_t)kWG * 64 * kSP) * sizeof(T) <= sizeof(lds), "epilogue tiles exceed the stage buffers");
     T *stg = reinterpret_cast<T *>(lds) + kStgOff + (size_t)wave * 64 * kSP;
-    const bool comb16 = comb && ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(comb) & 15) == 0;
-    auto store = [&](auto actc) __attribute__((always_inline)) {
-        constexpr int ACT = decltype(actc)::value;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < JN; ++j) {
-                const int col = j0 + 16 * JN * wn + 16 * j + l16;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float hv = 0.f;
-                    if (col < n) hv = HG ? activate_fast(ag[i][j][e], ACT) * au[i][j][e] : activate_fast(au[i][j][e], ACT);
-                    stg[(16 * i + 4 * q + e) * kSP + 16 * j + l16] = from_float<T>(hv);
-                }
-            }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (int c = 0; c < 2 * JN; ++c) {
-            const int idx = lane + 64 * c, row = idx / (2 * JN), ch = idx % (2 * JN);
-            const int m = m0 + 64 * wm + row, col0 = j0 + 16 * JN * wn + 8 * ch;
-            if (m < M && col0 < n_pad) {
-                const uint4 v = *reinterpret_cast<const uint4 *>(stg + row * kSP + 8 * ch);
-                *reinterpret_cast<uint4 *>(Hh + (size_t)m * ldh + col0) = v;
-                if (comb16 && col0 + 8 <= n) {
-                    *reinterpret_cast<uint4 *>(comb + (size_t)m * ldc + col0) = v;
-                } else if (comb) {
-                    const T *sv = stg + row * kSP + 8 * ch;
-#pragma unroll
-                    for (int k = 0; k < 8; ++k)
-                        if (col0 + k < n) comb[(size_t)m * ldc + col0 + k] = sv[k];
-                }
-            }
-        }
-    };
-    switch (act) {
-    case ST_ACT_RELU: store(std::integral_constant<int, ST_ACT_RELU>{}); break;
-    case ST_ACT_SILU: store(std::integral_constant<int, ST_ACT_SILU>{}); break;
-    case ST_ACT_GELU_TANH: store(std::integral_constant<int, ST_ACT_GELU_TANH>{}); break;
-    case ST_ACT_SIGMOID: store(std::integral_constant<int, ST_ACT_SIGMOID>{}); break;
-    default: store(std::integral_constant<int, ST_ACT_IDENTITY>{}); break;
-    }
+    pf_store_hidden<T, HG, JN>(act, ag, au, stg, lane, m0 + 64 * wm, j0 + 16 * JN * wn, M, n, n_pad, Hh, ldh, comb, ldc);
     ST_TL(4);
 }
 
@@ -500,53 +562,8 @@ __global__ __launch_bounds__(kPwThreads) void prefill_gateup_wide_kernel(const T
     __syncthreads();
 
     ST_TL(3);
-    // the wave's 64 x 32 results leave through a tile of its own in LDS as whole 16-byte chunks (see above)
-    constexpr int kSP = 32 + 8;
-    T *stg = reinterpret_cast<T *>(lds) + (size_t)wave * 64 * kSP;
-    const bool comb16 = comb && ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(comb) & 15) == 0;
-    const int mrow0 = m0 + 128 * wm + 64 * kh, colw = j0 + 32 * wn;
-    auto store = [&](auto actc) __attribute__((always_inline)) {
-        constexpr int ACT = decltype(actc)::value;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int col = colw + 16 * j + l16;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float hv = 0.f;
-                    if (col < n) hv = HG ? activate_fast(fg[i][j][e], ACT) * fu[i][j][e] : activate_fast(fu[i][j][e], ACT);
-                    stg[(16 * i + 4 * q + e) * kSP + 16 * j + l16] = from_float<T>(hv);
-                }
-            }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int idx = lane + 64 * c, row = idx / 4, ch = idx % 4;
-            const int m = mrow0 + row, col0 = colw + 8 * ch;
-            if (m < M && col0 < n_pad) {
-                const uint4 v = *reinterpret_cast<const uint4 *>(stg + row * kSP + 8 * ch);
-                *reinterpret_cast<uint4 *>(Hh + (size_t)m * ldh + col0) = v;
-                if (comb16 && col0 + 8 <= n) {
-                    *reinterpret_cast<uint4 *>(comb + (size_t)m * ldc + col0) = v;
-                } else if (comb) {
-                    const T *sv = stg + row * kSP + 8 * ch;
-#pragma unroll
-                    for (int k = 0; k < 8; ++k)
-                        if (col0 + k < n) comb[(size_t)m * ldc + col0 + k] = sv[k];
-                }
-            }
-        }
-    };
-    switch (act) {
-    case ST_ACT_RELU: store(std::integral_constant<int, ST_ACT_RELU>{}); break;
-    case ST_ACT_SILU: store(std::integral_constant<int, ST_ACT_SILU>{}); break;
-    case ST_ACT_GELU_TANH: store(std::integral_constant<int, ST_ACT_GELU_TANH>{}); break;
-    case ST_ACT_SIGMOID: store(std::integral_constant<int, ST_ACT_SIGMOID>{}); break;
-    default: store(std::integral_constant<int, ST_ACT_IDENTITY>{}); break;
-    }
+    T *stg = reinterpret_cast<T *>(lds) + (size_t)wave * 64 * (32 + 8);
+    pf_store_hidden<T, HG, 2>(act, fg, fu, stg, lane, m0 + 128 * wm + 64 * kh, j0 + 32 * wn, M, n, n_pad, Hh, ldh, comb, ldc);
     ST_TL(4);
 }
 
@@ -696,41 +713,11 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__
         }
     }
 
-    if (split_k == 1) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int col = c0 + 64 * wn + 16 * j + l16;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int m = m0 + 64 * wm + 16 * i + 4 * q + e;
-                    if (m < M && col < H) Out[(size_t)m * H + col] = from_float<T>(acc[i][j][e]);
-                }
-            }
-        return;
-    }
-    // Partial sums: the wave's 64 x 64 floats go through a tile of its own in LDS (the stage loop ends with a
-    // barrier, so the buffers are free) and leave as 16-byte chunks, 256 bytes of a row per 16 lanes.
-    constexpr int kSP = 64 + 4;   // floats per staged row
-    static_assert(4 * 64 * kSP * 4 <= (int)sizeof(lds), "staging tiles exceed the stage buffers");
-    float *stg = reinterpret_cast<float *>(lds) + (size_t)wave * 64 * kSP;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) stg[(16 * i + 4 * q + e) * kSP + 16 * j + l16] = acc[i][j][e];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int c = 0; c < 16; ++c) {
-        const int row = 4 * c + q, m = m0 + 64 * wm + row, col = c0 + 64 * wn + 4 * l16;
-        if (m < M && col < H)
-            *reinterpret_cast<float4 *>(partial + ((size_t)z * M + m) * H + col) =
-                *reinterpret_cast<const float4 *>(stg + row * kSP + 4 * l16);
-    }
+    // the stage loop ends with a barrier, so the buffers are free for the waves' tiles
+    static_assert(4 * 64 * kPfStgF * 4 <= (int)sizeof(lds), "staging tiles exceed the stage buffers");
+    float *stg = reinterpret_cast<float *>(lds) + (size_t)wave * 64 * kPfStgF;
+    pf_store_out<T>(acc, stg, lane, m0 + 64 * wm, c0 + 64 * wn, M, H, Out,
+                    split_k == 1 ? nullptr : partial + (size_t)z * M * H);
 }
 
 // ---------------------------------------------------------------------------
@@ -936,41 +923,10 @@ __global__ __launch_bounds__(kPwThreads) void prefill_down_wide_kernel(const T *
     __syncthreads();
 
     ST_TL(3);
-    const int mrow0 = m0 + 128 * wm + 64 * kh, colw = c0 + 64 * wn;
-    if (split_k == 1) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int col = colw + 16 * j + l16;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int m = mrow0 + 16 * i + 4 * q + e;
-                    if (m < M && col < H) Out[(size_t)m * H + col] = from_float<T>(f[i][j][e]);
-                }
-            }
-        return;
-    }
-    // partial sums leave through a tile of the wave's own in LDS as 16-byte chunks, 256 bytes of a row per 16 lanes
-    constexpr int kSP = 64 + 4;   // floats per staged row
-    static_assert(8 * 64 * kSP * 4 <= (int)sizeof(lds), "staging tiles exceed the stage buffers");
-    float *stg = reinterpret_cast<float *>(lds) + (size_t)wave * 64 * kSP;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) stg[(16 * i + 4 * q + e) * kSP + 16 * j + l16] = f[i][j][e];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int c = 0; c < 16; ++c) {
-        const int row = 4 * c + q, m = mrow0 + row, col = colw + 4 * l16;
-        if (m < M && col < H)
-            *reinterpret_cast<float4 *>(partial + ((size_t)z * M + m) * H + col) =
-                *reinterpret_cast<const float4 *>(stg + row * kSP + 4 * l16);
-    }
+    static_assert(8 * 64 * kPfStgF * 4 <= (int)sizeof(lds), "staging tiles exceed the stage buffers");
+    float *stg = reinterpret_cast<float *>(lds) + (size_t)wave * 64 * kPfStgF;
+    pf_store_out<T>(f, stg, lane, m0 + 128 * wm + 64 * kh, c0 + 64 * wn, M, H, Out,
+                    split_k == 1 ? nullptr : partial + (size_t)z * M * H);
     ST_TL(4);
 }
 
