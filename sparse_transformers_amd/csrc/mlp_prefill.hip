@@ -372,6 +372,19 @@ constexpr int kPwBM = 256, kPwWR = 64, kPwThreads = 512, kPwBufs = 3;
 // s_waitcnt immediate: vmcnt in bits 3:0 (and 15:14), expcnt 6:4 left at "no wait", lgkmcnt 11:8 = 0
 #define ST_WAIT_VM_LGKM0(vm) __builtin_amdgcn_s_waitcnt(((vm) & 15) | (7 << 4) | (0 << 8) | (((vm) >> 4) << 14))
 
+// 64 lanes x 16 bytes from `base + off` (uniform base, per-lane byte offset) to the 1 KB of LDS at byte address
+// `dst` (uniform), lane i's 16 bytes at dst + 16 i.  The instruction takes the LDS address from M0; the compiler is not
+// told about M0 (it is a reserved register for inline assembly), so its value is put back, and the write of M0 is
+// followed by the wait state the instruction needs before it may read it.
+__device__ __forceinline__ void pf_load_to_lds(unsigned dst, unsigned off, const char *base)
+{
+    unsigned keep;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 m0, %0"
+                 : "=&s"(keep)
+                 : "s"(dst), "v"(off), "s"(base)
+                 : "memory");
+}
+
 template <typename T, bool HG>
 __global__ __launch_bounds__(kPwThreads) void prefill_gateup_wide_kernel(const T *__restrict__ X, int M, int H,
                                                                          const T *__restrict__ gate,
@@ -422,18 +435,15 @@ __global__ __launch_bounds__(kPwThreads) void prefill_gateup_wide_kernel(const T
     }
     const int nk = H / kPfBK1;
     const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint4 *)lds;
-    // The load is written out as an instruction: the compiler treats the builtin form as a store to LDS that
-    // every later LDS read has to wait for (vmcnt(0) right behind the loads), which is exactly what the
+    // The load is written out as an instruction (pf_load_to_lds): the compiler treats the builtin form as a store to
+    // LDS that every later LDS read has to wait for (vmcnt(0) right behind the loads), which is exactly what the
     // three buffers are there to avoid; the waits are placed by hand below.
     auto dma = [&](int stage, int b) __attribute__((always_inline)) {
         const size_t k0 = (size_t)stage * kPfBK1 * sizeof(T);
 #pragma unroll
         for (int j = 0; j < kDma; ++j) {
             const unsigned dst = (unsigned)(b * kBuf + (wave * kDma + j) * 64) * 16u + lds_base;
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         :
-                         : "s"(dst), "v"(doff[j]), "s"(dbase[j] + k0)
-                         : "memory");
+            pf_load_to_lds(dst, doff[j], dbase[j] + k0);
         }
     };
 
@@ -799,7 +809,7 @@ __global__ __launch_bounds__(kPwThreads) void prefill_down_wide_kernel(const T *
                 src = reinterpret_cast<const char *>(Wd + c0);
                 off = (unsigned)kc * (unsigned)H * (unsigned)sizeof(T) + (unsigned)((lane & 15) ^ pf_swz_b(kt)) * 16u;
             }
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(off), "s"(src) : "memory");
+            pf_load_to_lds(dst, off, src);
         }
     };
 
