@@ -268,3 +268,43 @@ def test_fused_surplus_removals(I, n0, hint_slack):
         _same_state(fused, plain, (step, surplus, added, where))
         assert fused.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist(), (step, where)
         assert fused.sync_state()["n_removed"] - fused.sync_state()["n_added"] == surplus
+
+
+@pytest.mark.parametrize("I,H,dtype,has_gate,frac", [
+    (8192, 256, "float16", True, 0.35), (4096, 256, "bfloat16", False, 0.5), (16384, 256, "float16", True, 0.25),
+    (1000, 128, "float16", True, 0.3), (14336, 256, "bfloat16", True, 0.25), (11008, 512, "float16", True, 0.1),
+])
+def test_fused_random_count_changes(I, H, dtype, has_gate, frac):
+    """Random walks of the mask as a predictor's threshold produces them: the count drifts by a few percent per step
+    (more removals than additions in about half the steps), jumps by up to 30 % now and then, stays put, or lands
+    anywhere in 1 .. I; 0-40 % of the active set is swapped on top.  After every step the ordered list equals the
+    oracle's, and every seventh step the output carries the same bits as update followed by forward."""
+    for seed in (300, 301):
+        rng = np.random.default_rng(seed)
+        tdt = getattr(torch, dtype)
+        m = syn.initial_mask(rng, I, max(1, int(frac * I)))
+        fused, plain, (gate, up, down), g = _pair(I, H, dtype, has_gate, seed, torch.from_numpy(m))
+        oc = oracle.OracleWeightCache(m, H, gate.float().numpy() if has_gate else None, up.float().numpy(),
+                                      down.float().numpy(), has_gate)
+        n0 = int(m.sum())
+        for t in range(150):
+            kind, cur = int(rng.integers(0, 10)), int(m.sum())
+            if kind < 6:
+                target = int(round(cur * (1.0 + rng.uniform(-0.08, 0.08))))
+            elif kind < 8:
+                target = int(round(n0 * (1.0 + rng.uniform(-0.3, 0.3))))
+            elif kind == 8 or rng.random() >= 0.3:
+                target = cur
+            else:
+                target = int(rng.integers(1, I + 1))
+            m = syn.churn_step(rng, m, float(rng.choice([0.0, 0.02, 0.1, 0.15, 0.4])), max(1, min(I, target)))
+            mt = torch.from_numpy(m).to(DEV)
+            x = torch.randn(1, H, generator=g).to(tdt).to(DEV)
+            yf = fused.update_and_forward(mt, x, "silu")
+            oc.update_active_weights(m)
+            assert fused.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist(), (seed, t, cur, target)
+            plain.update_active_weights_async(mt)
+            if t % 7 == 0:
+                yp = plain.forward(x, "silu")
+                torch.cuda.synchronize()
+                assert torch.equal(yf, yp), (seed, t)
