@@ -172,6 +172,13 @@ def prefill_measure(stack, wl, T, layers, K, W, profile_steps, seed, torch, _lib
             "stack_tflops": layers * flops_layer / (ms_per_step * 1e-3) / 1e12}
 
 
+def prefill_gateup_name(rows: int, n_active: float, cus: int = 256) -> str:
+    """Which form of the gate/up kernel the library takes for this shape (mlp_prefill.hip: the wide form once 128-row
+    tiles of 64 + 64 weight rows outnumber the CUs)."""
+    tiles = ((int(n_active) + 127) // 128 * 2) * ((rows + 127) // 128)
+    return "prefill_gateup_wide_kernel" if rows > 128 and tiles > cus else "prefill_gateup_kernel"
+
+
 def prefill_bench(args, wl, torch, st, _lib, syn):
     """One step = `--prefill` rows of x through the sparse MLP of every layer (see prefill_measure)."""
     if wl.dtype == "float32":
@@ -191,7 +198,7 @@ def prefill_bench(args, wl, torch, st, _lib, syn):
                    "active_rows_mean": m["n_mean"], "act": wl.act, "has_gate": wl.has_gate},
         "roofline": {"bound": "mfma", "achieved": round(m["achieved_tflops"], 1), "peak": MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(m["achieved_tflops"] / MFMA_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "prefill_gateup_wide_kernel", "flops_per_launch": m["gu_flops"], "mean_us": m["gu_us"]},
+                     "kernel": prefill_gateup_name(T, m["n_mean"]), "flops_per_launch": m["gu_flops"], "mean_us": m["gu_us"]},
         "stack_tflops": round(m["stack_tflops"], 1),
         "kernels_us": m["kernels_us"],
     }
@@ -516,7 +523,7 @@ def main():
             result["prefill_512"] = {
                 "layers": pl, "rows": 512, "active_rows_mean": m["n_mean"], "tok_s": round(512 / (m["ms_per_step"] * 1e-3), 1),
                 "us_per_layer": round(m["ms_per_step"] * 1e3 / pl, 2), "stack_tflops": round(m["stack_tflops"], 1),
-                "roofline": {"bound": "mfma", "kernel": "prefill_gateup_wide_kernel", "achieved": round(m["achieved_tflops"], 1),
+                "roofline": {"bound": "mfma", "kernel": prefill_gateup_name(512, m["n_mean"]), "achieved": round(m["achieved_tflops"], 1),
                              "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                              "frac": round(m["achieved_tflops"] / MFMA_PEAK_TFLOPS, 4), "mean_us": m["gu_us"]},
                 "kernels_us": m["kernels_us"]}
