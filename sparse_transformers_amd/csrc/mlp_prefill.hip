@@ -952,8 +952,15 @@ __global__ __launch_bounds__(256) void prefill_reduce_kernel(const float *__rest
         const float4 v = *reinterpret_cast<const float4 *>(partial + (size_t)z * total + i4);
         s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
-    T *o = out + i4;
-    o[0] = from_float<T>(s.x); o[1] = from_float<T>(s.y); o[2] = from_float<T>(s.z); o[3] = from_float<T>(s.w);
+    // (T is a 16-bit type here; M * H is a multiple of 4 and `out` a tensor's base, so the four results are one 8-byte store)
+    const uint32_t lo = (uint32_t)from_float<T>(s.x).bits | ((uint32_t)from_float<T>(s.y).bits << 16);
+    const uint32_t hi = (uint32_t)from_float<T>(s.z).bits | ((uint32_t)from_float<T>(s.w).bits << 16);
+    if ((reinterpret_cast<uintptr_t>(out) & 7) == 0) {
+        *reinterpret_cast<uint2 *>(out + i4) = make_uint2(lo, hi);
+    } else {
+        T *o = out + i4;
+        o[0] = from_float<T>(s.x); o[1] = from_float<T>(s.y); o[2] = from_float<T>(s.z); o[3] = from_float<T>(s.w);
+    }
 }
 
 int prefill_split_k(int M, int H, int n)
