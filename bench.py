@@ -105,6 +105,10 @@ def parse_args():
     ap.add_argument("--prefill", type=int, default=0,
                     help="time the MFMA path instead: this many rows of x per step through the stack's sparse MLPs, "
                          "each cache at the union of the rows' masks (roofline against the dense MFMA peak)")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the short passes over the other workloads / batch sizes and the count-wobble pass that "
+                         "the default line carries as `other_workloads` (they only run for the default workload, "
+                         "depth and batch)")
     ap.add_argument("--seed", type=int, default=1236)
     return ap.parse_args()
 
@@ -293,42 +297,21 @@ def cpu_baseline(wl, stack, trace, x_in, x_pred, layers, steps, torch):
     }
 
 
-def main():
-    args = parse_args()
-    if args.gpus != 1:
-        print(f"bench.py: this build runs on ONE GPU (every box has one); --gpus {args.gpus} is not supported. "
-              "The path would shard along the intermediate dimension, but no multi-GPU code exists.",
-              file=sys.stderr)
-        sys.exit(2)
-
-    import torch
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
-        sys.exit(3)
-    import sparse_transformers_amd as st
-    from sparse_transformers_amd import _lib, synthetic as syn
-
-    wl = syn.WORKLOADS[args.workload]
-    if args.active_frac > 0.0 or args.churn >= 0.0:
-        import dataclasses
-        wl = dataclasses.replace(wl, active_frac=args.active_frac if args.active_frac > 0.0 else wl.active_frac,
-                                 churn_lo=args.churn if args.churn >= 0.0 else wl.churn_lo,
-                                 churn_hi=args.churn if args.churn >= 0.0 else wl.churn_hi)
-    if args.prefill > 0:
-        prefill_bench(args, wl, torch, st, _lib, syn)
-        return
-    layers = args.layers or wl.layers
-    B = args.batch or wl.batch
+def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wobble=0.0, wall=True):
+    """One decode workload: W warm-up + K timed steps (one token through `layers` layers each, replayed from a HIP
+    graph), then an eager pass over P of the same steps with per-kernel events.  Returns the result dict and what the
+    CPU baseline needs (stack, trace, x_in, x_pred)."""
     dev = torch.device("cuda:0")
     dt = getattr(torch, wl.dtype)
     esz = 4 if wl.dtype == "float32" else 2
     H, I, n = wl.hidden, wl.intermediate, wl.n_active
-    K, W, P = args.steps, args.warmup, args.profile_steps
+    # the per-kernel pass walks the trace backwards from the last timed step and must stay inside it
+    P = max(1, min(P, W + K - 1))
 
     stack, g = build_stack(wl, layers, B, args.seed, torch, st)
     T = W + K + 1
     trace = torch.from_numpy(syn.mask_trace(args.seed + 7, layers, I, n, T, wl.churn_lo, wl.churn_hi,
-                                             args.count_wobble)).to(dev)
+                                             count_wobble)).to(dev)
     # predictor inputs per layer and step, MLP input of the first layer per step
     x_pred = torch.randn(T, layers, B, H, generator=g, device=dev, dtype=torch.float32).to(dt)
     x_in = torch.randn(T, B, H, generator=g, device=dev, dtype=torch.float32).to(dt)
@@ -425,7 +408,7 @@ def main():
     # ---- begin/end events cannot show what it costs inside the chain: an empty kernel already reads 4 us
     # ---- between its two events, while a dependent empty kernel adds only 1.6 us to a replayed chain)
     wall_parts = None
-    if use_graph and not args.overlap:
+    if wall and use_graph and not args.overlap:
         def part_predictor():
             for l, layer in enumerate(stack.layers):
                 layer.predict_mask(stack.xp_stage[l], stack._t_ws)
@@ -491,7 +474,7 @@ def main():
         "dtype": {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[wl.dtype], "data": "synthetic",
         "config": {"workload": wl.name, "layers": layers, "hidden": H, "intermediate": I, "predictor_rank": wl.rank,
                    "batch": B, "act": wl.act, "has_gate": wl.has_gate, "n_active": n,
-                   "churn": [wl.churn_lo, wl.churn_hi], "count_wobble": args.count_wobble, "mask_source": "trace",
+                   "churn": [wl.churn_lo, wl.churn_hi], "count_wobble": count_wobble, "mask_source": "trace",
                    "launch": "hip_graph" if use_graph else "eager",
                    "streams": 2 if args.overlap else 1, "update_fused_into_decode": bool(stack.fused),
                    "kernel_timing": "hip events stamped at kernel begin/end (hipExtLaunchKernelGGL), eager second pass"},
@@ -513,7 +496,40 @@ def main():
         "kernels_us": per_kernel,
         "kernels_us_unfused": unfused,
         "churn_mean": churn_mean,
+        "profile_pass": {"steps": P, "trace_steps": [t_lo + 1, W + K - 1],
+                         "note": "eager pass with per-kernel events, backwards over the last steps of the timed range"},
     }
+    return result, (stack, trace, x_in, x_pred)
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (every box has one); --gpus {args.gpus} is not supported. "
+              "The path would shard along the intermediate dimension, but no multi-GPU code exists.",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    import sparse_transformers_amd as st
+    from sparse_transformers_amd import _lib, synthetic as syn
+
+    wl = syn.WORKLOADS[args.workload]
+    if args.active_frac > 0.0 or args.churn >= 0.0:
+        import dataclasses
+        wl = dataclasses.replace(wl, active_frac=args.active_frac if args.active_frac > 0.0 else wl.active_frac,
+                                 churn_lo=args.churn if args.churn >= 0.0 else wl.churn_lo,
+                                 churn_hi=args.churn if args.churn >= 0.0 else wl.churn_hi)
+    if args.prefill > 0:
+        prefill_bench(args, wl, torch, st, _lib, syn)
+        return
+    layers = args.layers or wl.layers
+    B = args.batch or wl.batch
+    result, (stack, trace, x_in, x_pred) = decode_measure(args, wl, torch, st, _lib, syn, layers, B, args.steps, args.warmup,
+                                                          args.profile_steps, args.count_wobble)
     if not args.no_prefill_probe and wl.dtype != "float32" and B == 1:
         # the MFMA path in the same line: 512 rows of x through the first layers' sparse MLPs (caches at the union of
         # the rows' masks).  Runs last: it moves those caches away from the decode trace.
@@ -536,7 +552,50 @@ def main():
         except Exception as exc:  # the baseline is reported, never required for the GPU numbers
             result["cpu_baseline"] = {"value": None, "unit": "tok/s", "cores": 0, "kind": "port",
                                       "sample": f"failed: {exc!r}"}
+    default_run = (args.workload == "llama3b_stack_fp16" and not args.layers and not args.batch and args.churn < 0.0
+                   and args.active_frac <= 0.0 and args.count_wobble == 0.0 and not args.no_graph and not args.overlap
+                   and not args.no_fused)
+    if default_run and not args.no_other_workloads:
+        del stack, trace, x_in, x_pred
+        result["other_workloads"] = other_workloads(args, torch, st, _lib, syn)
     print(json.dumps(result))
+
+
+# (workload, rows of x): the configurations of the other benchmark shapes, each as a short pass
+OTHER_WORKLOADS = [("llama1b_layer_fp32", 1), ("llama3b_stack_fp16", 4), ("llama3b_stack_fp16", 16),
+                   ("mistral7b_stack_bf16", 1), ("mistral7b_stack_bf16", 8), ("relullama7b_stack_fp16", 1),
+                   ("relullama7b_ungated_fp16", 1)]
+
+
+def other_workloads(args, torch, st, _lib, syn, steps=12, warmup=4, profile_steps=6):
+    """Short passes (no CPU baseline, no prefill probe) over the other workloads and batch sizes, and one over the
+    headline workload with the active count wobbling by 3 % per layer-step, as a predictor's threshold makes it."""
+    import dataclasses
+    import gc
+
+    def brief(r):
+        rf = r["roofline"]
+        return {"tok_s": r["value"], "ms_per_step": r["ms_per_step"], "layers": r["config"]["layers"],
+                "us_per_layer": round(r["ms_per_step"] * 1e3 / r["config"]["layers"], 2), "kernel": rf["kernel"],
+                "kernel_mean_us": rf["mean_us"], "frac": rf["frac"], "frac_mlp_bytes_only": rf["frac_mlp_bytes_only"],
+                "stack_hbm_gbps": r["stack_hbm_gbps"], "kernels_us": {k: v["median_us"] for k, v in r["kernels_us"].items()}}
+
+    out = {"steps": steps, "warmup": warmup}
+    runs = [(name, b, 0.0) for name, b in OTHER_WORKLOADS] + [("llama3b_stack_fp16", 1, 0.03)]
+    for name, b, wobble in runs:
+        wl = syn.WORKLOADS[name]
+        layers = wl.layers if wl.layers > 1 else 16     # a single layer's weights would sit in the Infinity Cache
+        key = f"{name}_b{b}" if wobble == 0.0 else f"{name}_b{b}_count_wobble_{wobble}"
+        try:
+            r, keep = decode_measure(args, wl, torch, st, _lib, syn, layers, b, steps if wobble == 0.0 else 20, warmup,
+                                     profile_steps, wobble, wall=False)
+            out[key] = brief(r)
+            del keep
+        except Exception as exc:
+            out[key] = {"error": repr(exc)}
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
 
 
 if __name__ == "__main__":

@@ -1534,12 +1534,8 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
     {
         ProfScope ps(ST_K_CACHE_UPDATE, s);
         auto launch = [&](auto kern) -> int {
-            static std::atomic<bool> attr_set{false};   // (setting the attribute twice from two threads is harmless)
-            if (!attr_set.load(std::memory_order_acquire)) {
-                ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
-                attr_set.store(true, std::memory_order_release);
-            }
+            const int arc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), 160 * 1024 - 256);
+            if (arc != ST_OK) return arc;
             ST_LAUNCH(ps, kern, dim3(grid), dim3(tpb), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state,
                                I, gs_log2, idx_cap);
             return ST_OK;
@@ -1609,12 +1605,8 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
     {
         ProfScope ps(ST_K_CACHE_UPDATE_DECODE, s);
         auto launch = [&](auto kern, auto *xt, auto *ct) -> int {
-            static std::atomic<bool> attr_set{false};   // (setting the attribute twice from two threads is harmless)
-            if (!attr_set.load(std::memory_order_acquire)) {
-                ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 148 * 1024));
-                attr_set.store(true, std::memory_order_release);
-            }
+            const int arc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), 148 * 1024);
+            if (arc != ST_OK) return arc;
             ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, fr, mask, c->b.cur_mask, c->b.indices, c->b.state, I, xt,
                       (int)B, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint);
             return ST_OK;

@@ -3,6 +3,8 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
+#include <unordered_set>
 #include <vector>
 
 namespace st {
@@ -34,6 +36,19 @@ int device_cu_count()
         cached[dev] = cus;
     }
     return cached[dev];
+}
+
+// hipFuncAttributeMaxDynamicSharedMemorySize, set once per kernel symbol (keyed by the kernel's address: the
+// instantiations of one kernel template share a function-pointer type, so a flag per call site is not enough).
+int allow_dynamic_lds(const void *kernel, int bytes)
+{
+    static std::mutex mu;
+    static std::unordered_set<const void *> done;
+    std::lock_guard<std::mutex> lock(mu);
+    if (done.count(kernel)) return ST_OK;
+    ST_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    done.insert(kernel);
+    return ST_OK;
 }
 
 // ---- per-kernel event timing ------------------------------------------------

@@ -986,8 +986,9 @@ int prefill_split_k(int M, int H, int n)
 static bool prefill_down_is_wide(int M, int H, int n, long ldh)
 {
     const int mt = (M + kPwBM - 1) / kPwBM;
+    // (the wide kernels address their operands with 32-bit byte offsets: Hh and the rows of Wd have to stay below 4 GiB)
     return M > 128 && (mt * kPwBM - M) * 5 <= mt * kPwBM && H % kPfBN == 0 && n >= 512 &&
-           (int64_t)M * ldh * 2 < ((int64_t)1 << 32);
+           (int64_t)M * ldh * 2 < ((int64_t)1 << 32) && (int64_t)n * H * 2 < ((int64_t)1 << 32);
 }
 
 static int prefill_split_k_wide(int M, int H, int n)
@@ -1036,7 +1037,8 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         // CUs and on 128 x (32 + 32) tiles (twice the blocks) when there are fewer -- four groups with a quarter
         // of K each on 64 x (32 + 32) tiles while those fit one per CU.  What is left (one row tile and more
         // than 16384 active rows) takes 128 x (32 + 32) tiles without K groups.
-        const bool big = M > 128 && jt64 * mt128 > cus;
+        // (32-bit byte offsets into x and the weight rows in the wide kernel)
+        const bool big = M > 128 && jt64 * mt128 > cus && (int64_t)(M > n ? M : n) * H * 2 < ((int64_t)1 << 32);
         const bool halves = !big && 2 * jt64 * mt128 <= cus;
         // 64-row tiles: four K groups fit the LDS
         const bool quarters = !big && H % 256 == 0 && 2 * jt64 * ((M + 63) / 64) <= cus;

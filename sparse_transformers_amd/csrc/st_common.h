@@ -238,6 +238,8 @@ int hip_fail(hipError_t e, const char *what);
     } while (0)
 
 int device_cu_count();
+// Lets `kernel` be launched with up to `bytes` of dynamic LDS (set once per kernel symbol).
+int allow_dynamic_lds(const void *kernel, int bytes);
 
 // Rows a thread group of the single-row decode kernels keeps in flight (18 16-byte loads per thread).
 // The stand-alone and the fused kernel must agree on it: it decides which block sums which rows, and the

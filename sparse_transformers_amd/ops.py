@@ -109,6 +109,22 @@ def check_mlp_args(x2: torch.Tensor, out: torch.Tensor, combined: Optional[torch
                              f"{tuple(combined.shape)} strides {combined.stride()}")
 
 
+def combined_for_launch(combined: Optional[torch.Tensor], B: int, n: int):
+    """The tensor to hand to the C entry points as ``combined`` and the view to copy it back into afterwards (or
+    None).  With 32 or more rows of x in fp16 / bf16 the GEMM kernels may keep their intermediate in ``combined``
+    when its row stride has room for n rounded up to a multiple of 128, and then zero the columns between n and
+    that width.  The C ABI describes the buffer by its stride alone; a column slice of a wider tensor whose own
+    width ends before the padded one would have its parent's columns zeroed, so such a view goes through a
+    contiguous stand-in of its own width (whose stride is too short for the padding, so nothing is written
+    outside it)."""
+    if combined is None or B < 32 or combined.dtype == torch.float32:
+        return combined, None
+    padded = (int(n) + 127) // 128 * 128
+    if combined.stride(0) == combined.size(1) or combined.size(1) >= padded:
+        return combined, None
+    return torch.empty(B, combined.size(1), dtype=combined.dtype, device=combined.device), combined[:B]
+
+
 def mlp_forward_rows(x2: torch.Tensor, gate_rows: Optional[torch.Tensor], up_rows: torch.Tensor,
                      down_rows: torch.Tensor, n: int, n_dev: Optional[torch.Tensor], out: torch.Tensor,
                      combined: Optional[torch.Tensor], act: str, has_gate: bool, n_hint: int = 0,
@@ -139,12 +155,15 @@ def mlp_forward_rows(x2: torch.Tensor, gate_rows: Optional[torch.Tensor], up_row
     ws = mlp_workspace(dev, B, H, n) if workspace is None else _check_workspace(workspace, dev, need)
     if act not in _lib.ACT_CODES:
         raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
+    combined, copy_back = combined_for_launch(combined, B, n)
     rc = _lib.lib().st_mlp_forward(
         x2.data_ptr(), B, H, gate_rows.data_ptr() if has_gate else None, up_rows.data_ptr(), down_rows.data_ptr(),
         n, n_dev.data_ptr() if n_dev is not None else None, int(n_hint), out.data_ptr(),
         combined.data_ptr() if combined is not None else None, combined.stride(0) if combined is not None else 0,
         ws.data_ptr(), ws.numel(), _lib.ACT_CODES[act], dtype_code(x2), int(bool(has_gate)), current_stream_ptr(dev))
     _lib.check(rc, "st_mlp_forward")
+    if copy_back is not None:
+        copy_back.copy_(combined)
 
 
 _warned_layout = False

@@ -13,8 +13,8 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .ops import (_check_workspace, check_mlp_args, current_stream_ptr, dtype_code, mlp_forward_rows, mlp_workspace,
-                  mlp_workspace_bytes, require_gpu)
+from .ops import (_check_workspace, check_mlp_args, combined_for_launch, current_stream_ptr, dtype_code,
+                  mlp_forward_rows, mlp_workspace, mlp_workspace_bytes, require_gpu)
 
 
 class ConcatWeightHandle(torch.Tensor):
@@ -242,6 +242,7 @@ class WeightCache:
         ws = mlp_workspace(self.device, B, H, I) if workspace is None else _check_workspace(workspace, self.device, need)
         if act not in _lib.ACT_CODES:
             raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
+        combined, copy_back = combined_for_launch(combined, B, I)
         rc = _lib.lib().st_cache_update_forward(
             self._h, m.data_ptr(), x2.data_ptr(), B,
             int(self._host_state[_lib.STATE_N_ACTIVE]) if n_hint is None else int(n_hint), out.data_ptr(),
@@ -249,6 +250,8 @@ class WeightCache:
             ws.data_ptr(), ws.numel(), _lib.ACT_CODES[act], current_stream_ptr(self.device))
         _lib.check(rc, "st_cache_update_forward")
         self._dirty = True
+        if copy_back is not None:
+            copy_back.copy_(combined)
         return out.view(x.shape)
 
     def forward(self, x: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor] = None,

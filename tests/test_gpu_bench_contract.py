@@ -20,7 +20,8 @@ def _run(*args):
 
 
 def test_decode_line():
-    d = _run("--layers", "2", "--steps", "6", "--warmup", "2", "--profile-steps", "2", "--cpu-layers", "1",
+    # (more profile steps than the run has: the per-kernel pass must clamp itself to the trace, not wrap around it)
+    d = _run("--layers", "2", "--steps", "6", "--warmup", "2", "--profile-steps", "32", "--cpu-layers", "1",
              "--cpu-steps", "4")
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
                 "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
@@ -31,6 +32,12 @@ def test_decode_line():
     r = d["roofline"]
     assert r["bound"] == "hbm" and r["peak"] == 8000.0 and r["unit"] == "GB/s"
     assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3 and 0 < r["frac"] < 1
+    pp = d["profile_pass"]
+    assert pp["steps"] == 7 and pp["trace_steps"] == [1, 7], pp
+    # every update of the pass has the configured churn: no launch moves many times the usual number of rows
+    ku = d["kernels_us"]["cache_update_decode"]
+    assert ku["launches"] == 2 * 7 and ku["p90_us"] < 1.5 * ku["median_us"], ku
+    assert "other_workloads" not in d      # only the default workload, depth and batch carry them
     c = d["cpu_baseline"]
     assert c["value"] > 0 and c["cores"] >= 1 and c["kind"] in ("reference", "port") and c["sample"]
 

@@ -219,14 +219,16 @@ def test_prefill_agrees_with_decode_kernel():
 ])
 def test_prefill_wide_blocks(name, M, H, n, dtype, act, has_gate):
     """With more 128-row tiles than CUs the gate/up kernel switches to 256-row blocks, and from 256 rows on the down
-    projection to 256-row tiles with the K range split over the CUs.  The oracle checks the
-    first and the last rows (a full and a ragged row tile); every row is compared with the streaming decode
-    kernel, which the tests above hold against the oracle."""
+    projection to 256-row tiles with the K range split over the CUs.  Every row of the output and of the
+    intermediate is held against the oracle; a sample of row groups is also compared with the streaming decode
+    kernel."""
     x, cw, dn = _case(23, M, H, n, dtype, has_gate)
     out, _, cb = _run(x, cw, dn, act, has_gate)
     out, cb = out.float().cpu().numpy().copy(), cb.float().cpu().numpy().copy()
-    for rows in (slice(0, 6), slice(M - 3, M)):
-        want, wantc = oracle.mlp_forward(x[rows].float().numpy(), cw.float().numpy(), dn.float().numpy().T, act, has_gate)
+    xf, cwf, dnf = x.float().numpy(), cw.float().numpy(), np.ascontiguousarray(dn.float().numpy().T)
+    for r0 in range(0, M, 128):
+        rows = slice(r0, min(M, r0 + 128))
+        want, wantc = oracle.mlp_forward(xf[rows], cwf, dnf, act, has_gate)
         assert_close(out[rows], want, dtype, f"{name} rows {rows}")
         assert_close(cb[rows, :n], wantc[:, :n], dtype, f"{name} combined rows {rows}")
     step = 8
@@ -234,6 +236,23 @@ def test_prefill_wide_blocks(name, M, H, n, dtype, act, has_gate):
         small, _, cs = _run(x[b0:b0 + step], cw, dn, act, has_gate)
         assert_close(out[b0:b0 + step], small.float().cpu().numpy(), dtype, f"{name} rows {b0}.. vs decode kernel")
         assert_close(cb[b0:b0 + step, :n], cs.float().cpu().numpy()[:, :n], dtype, f"{name} combined rows {b0}..")
+
+
+def test_prefill_leaves_the_parent_of_a_column_slice_alone():
+    """`combined` given as a column slice of a wider tensor (ungated, 64 rows of x, n not a multiple of 128): the
+    GEMM kernels keep their intermediate in a buffer whose row stride has room for n rounded up to 128 and zero the
+    padding, which must not happen to the parent's columns."""
+    B, H, n = 64, 512, 700
+    x, cw, dn = _case(29, B, H, n, "float16", False)
+    parent = torch.full((B, 1024), 7.0, dtype=torch.float16, device=DEV)
+    out = torch.empty(B, H, dtype=torch.float16, device=DEV)
+    mlp_forward_rows(x.to(DEV), None, cw.to(DEV), dn.to(DEV), n, None, out, parent[:, :n], "relu", False)
+    torch.cuda.synchronize()
+    assert bool((parent[:, n:] == 7.0).all()), "columns outside the view were written"
+    want, wantc = oracle.mlp_forward(x.float().numpy(), cw.float().numpy(), np.ascontiguousarray(dn.float().numpy().T),
+                                     "relu", False)
+    assert_close(out.float().cpu().numpy(), want, "float16", "out")
+    assert_close(parent[:, :n].float().cpu().numpy(), wantc[:, :n], "float16", "combined view")
 
 
 # ---- MFMA batch kernels (3 <= B <= 32, fp16 / bf16, H in {2048, 3072, 4096}) ----

@@ -20,12 +20,13 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _threshold_in_gap(s: np.ndarray, frac: float, guard_rel: float = 4e-6) -> float:
-    """A threshold with about `frac` of the columns of s [B,I] active (any row >= t), placed in the widest gap
-    between ALL scores near that quantile; asserts that no score lies within guard_rel * max|s| of it (the GPU
-    scores differ from the oracle's by less than half of that, see test_gpu_predictor)."""
+def _threshold_in_gap(s: np.ndarray, frac: float, guard_rel: float = 4e-6, per_row: bool = False) -> float:
+    """A threshold with about `frac` of the columns of s [B,I] active (any row >= t) -- with `per_row`, about `frac`
+    of every row's scores -- placed in the widest gap between ALL scores near that quantile; asserts that no score
+    lies within guard_rel * max|s| of it (the GPU scores differ from the oracle's by less than half of that, see
+    test_gpu_predictor)."""
     a = np.sort(s.astype(np.float64).ravel())
-    t0 = np.quantile(s.max(0).astype(np.float64), 1.0 - frac)
+    t0 = np.quantile((s if per_row else s.max(0)).astype(np.float64), 1.0 - frac)
     j = int(np.searchsorted(a, t0))
     lo, hi = max(1, j - 16), min(a.size - 1, j + 16)
     gaps = a[lo:hi + 1] - a[lo - 1:hi]
@@ -51,30 +52,51 @@ def _build(dtype, L, H, I, r, has_gate, act, seed):
     return st.SparseMLPStack(layers), oracles
 
 
-# name, L, H, I, r, dtype, B, act, gate, active fraction, (rho_lo, rho_hi), steps, expected churn band
+# name, L, H, I, r, dtype, B, act, gate, active fraction, (rho_lo, rho_hi), steps, expected churn band, shared
+# `shared` = 0: the rows of a step are independent and `frac` is the fraction of the UNION that is active;
+# `shared` > 0: every row has `frac` of its own scores active and the rows share that part of their variance, so
+# that the per-row masks overlap (0.6 for the batched bf16 configuration); the cache sees their union.
 CASES = [
-    ("llama3b_fp16_b1", 2, 3072, 8192, 128, "float16", 1, "silu", True, 0.35, (0.95, 0.995), 64, (0.03, 0.17)),
-    ("mistral7b_bf16_b2", 2, 4096, 14336, 256, "bfloat16", 2, "silu", True, 0.25, (0.98, 0.98), 16, (0.05, 0.2)),
+    ("llama1b_fp32_b1", 1, 2048, 8192, 64, "float32", 1, "silu", True, 0.30, (0.97, 0.97), 32, (0.05, 0.25), 0.0),
+    ("llama3b_fp16_b1", 2, 3072, 8192, 128, "float16", 1, "silu", True, 0.35, (0.95, 0.995), 64, (0.03, 0.17), 0.0),
+    ("llama3b_bf16_b16_union", 1, 3072, 8192, 128, "bfloat16", 16, "silu", True, 0.30, (0.9, 0.9), 8, (0.0, 0.2), 0.72),
+    ("mistral7b_bf16_b2", 2, 4096, 14336, 256, "bfloat16", 2, "silu", True, 0.25, (0.98, 0.98), 16, (0.05, 0.2), 0.0),
+    ("relullama7b_gated_fp16_b1", 2, 4096, 11008, 440, "float16", 1, "relu", True, 0.10, (0.95, 0.95), 16,
+     (0.1, 0.35), 0.0),
     ("relullama7b_ungated_fp16_b1", 2, 4096, 11008, 440, "float16", 1, "relu", False, 0.10, (0.95, 0.95), 16,
-     (0.1, 0.35)),
+     (0.1, 0.35), 0.0),
 ]
 
 
-@pytest.mark.parametrize("name,L,H,I,r,dtype,B,act,has_gate,frac,rho,steps,churn_band", CASES,
+def _step_inputs(rng, state, rh, shared):
+    """Predictor inputs [L,B,H] of the next step: AR(1) in time; with `shared` the rows of a step share that
+    fraction of their variance."""
+    common, own = state
+    L, B, H = own.shape
+    own = rh * own + np.sqrt(1.0 - rh * rh) * rng.standard_normal((L, B, H))
+    if shared > 0.0:
+        common = rh * common + np.sqrt(1.0 - rh * rh) * rng.standard_normal((L, 1, H))
+        xp = np.sqrt(shared) * common + np.sqrt(1.0 - shared) * own
+    else:
+        xp = own
+    return (common, own), xp.astype(np.float32)
+
+
+@pytest.mark.parametrize("name,L,H,I,r,dtype,B,act,has_gate,frac,rho,steps,churn_band,shared", CASES,
                          ids=[c[0] for c in CASES])
-def test_full_shape_decode_sequence(name, L, H, I, r, dtype, B, act, has_gate, frac, rho, steps, churn_band):
+def test_full_shape_decode_sequence(name, L, H, I, r, dtype, B, act, has_gate, frac, rho, steps, churn_band, shared):
     stack, oracles = _build(dtype, L, H, I, r, has_gate, act, seed=31)
     tdt = getattr(torch, dtype)
     rng = np.random.default_rng(7)
     stack.prepare(B)                 # fused update + decode kernel, the stack's own scratch
     stack.use_trace_masks = False    # the predictor's masks drive the caches
     assert stack.fused
-    xp = rng.standard_normal((L, B, H)).astype(np.float32)
-    churns, surplus_add, surplus_rem = [], 0, 0
+    state = (rng.standard_normal((L, 1, H)), rng.standard_normal((L, B, H)))
+    churns, overlaps, surplus_add, surplus_rem = [], [], 0, 0
     prev = [np.ones(I, bool) for _ in range(L)]
     for t in range(steps):
         rh = rng.uniform(*rho) if rho[1] > rho[0] else rho[0]
-        xp = (rh * xp + np.sqrt(1.0 - rh * rh) * rng.standard_normal((L, B, H))).astype(np.float32)
+        state, xp = _step_inputs(rng, state, rh, shared)
         xph = round_to(xp, dtype)
         x = round_to(rng.standard_normal((B, H)).astype(np.float32), dtype)
         # thresholds: the step's target fraction (wobbling by a few percent of the set), placed in a score gap
@@ -83,9 +105,12 @@ def test_full_shape_decode_sequence(name, L, H, I, r, dtype, B, act, has_gate, f
         for l, (oc, w) in enumerate(oracles):
             s = oracle.predictor_scores(xph[l], w["A"], w["Bm"])
             f = frac * (1.0 + rng.uniform(-0.03, 0.03))
-            thr = _threshold_in_gap(s, f)
+            thr = _threshold_in_gap(s, f, per_row=shared > 0.0)
             stack.layers[l].thr = thr
             m = oracle.mask_threshold(s, thr, True)
+            if shared > 0.0:   # overlap of consecutive rows' own masks
+                rows = s >= thr
+                overlaps.append(float((rows[:-1] & rows[1:]).sum() / max(1, rows[:-1].sum())))
             want_masks.append(m)
             if t > 0:
                 na, nr = int((m & ~prev[l]).sum()), int((prev[l] & ~m).sum())
@@ -107,3 +132,5 @@ def test_full_shape_decode_sequence(name, L, H, I, r, dtype, B, act, has_gate, f
     mean_churn = float(np.mean(churns))
     assert churn_band[0] <= mean_churn <= churn_band[1], f"mean churn {mean_churn:.3f} outside {churn_band}"
     assert surplus_add > 0 and surplus_rem > 0, "the sequence must exercise appends and surplus removals"
+    if shared > 0.0:
+        assert 0.5 <= float(np.mean(overlaps)) <= 0.7, f"mean overlap of the rows' masks {np.mean(overlaps):.3f}"

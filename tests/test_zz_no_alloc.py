@@ -55,6 +55,43 @@ def test_static_scratch_forward_matches_workspace_forward(dtype, H, has_gate):
         assert_close(got.float().cpu().numpy(), want, dtype, f"B={B} n={n}")
 
 
+def test_static_scratch_forward_under_graph_capture():
+    """What the entry point is for: a caller that records a HIP graph.  After one eager call on the device (which
+    resolves the address of the library's scratch array; nothing but launches happens afterwards) the call is
+    captured, replayed with other work between the replays, and every replay equals the eager result."""
+    L = _lib.lib()
+    H, n, B = 3072, 900, 1
+    tdt = torch.float16
+    g = torch.Generator(device=DEV)
+    g.manual_seed(5)
+    w = [(torch.randn(n, H, generator=g, device=DEV) * 0.05).to(tdt) for _ in range(3)]
+    x = torch.randn(B, H, generator=g, device=DEV).to(tdt)
+    out = torch.zeros(B, H, dtype=tdt, device=DEV)
+
+    def call():
+        rc = L.st_mlp_forward_static(x.data_ptr(), B, H, w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), n, None, 0,
+                                     out.data_ptr(), None, 0, _lib.ACT_CODES["silu"], _lib.ST_F16, 1,
+                                     torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "st_mlp_forward_static")
+
+    call()                                   # eager: also the first call on this device
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for rep in range(4):
+        x.copy_(torch.randn(B, H, generator=g, device=DEV).to(tdt))
+        call()
+        torch.cuda.synchronize()
+        eager = out.clone()
+        out.zero_()
+        other = _call(False, x, w[0], w[1], w[2], n // 2, "silu", True)    # unrelated work between the replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
+        del other
+
+
 def test_static_scratch_limits():
     L = _lib.lib()
     assert L.st_mlp_static_scratch_bytes() == 8 << 20
