@@ -102,6 +102,11 @@ def parse_args():
                     help="let the active count of every layer-step vary by this fraction around the workload's value "
                          "(as a predictor's threshold would: some updates add more than they remove, others remove "
                          "more); 0 keeps the count fixed, which is what the headline is quoted on")
+    ap.add_argument("--mask-source", choices=("trace", "predictor"), default="trace",
+                    help="what drives the caches: the pre-generated mask trace with exactly the configured count and churn "
+                         "(the predictor's mask is computed and dropped), or the layer's own predictor mask (threshold "
+                         "at the workload's active fraction; predictor inputs follow an AR(1) process whose correlation "
+                         "gives about the configured churn; count and churn then wobble as they do in a model)")
     ap.add_argument("--prefill", type=int, default=0,
                     help="time the MFMA path instead: this many rows of x per step through the stack's sparse MLPs, "
                          "each cache at the union of the rows' masks (roofline against the dense MFMA peak)")
@@ -297,7 +302,23 @@ def cpu_baseline(wl, stack, trace, x_in, x_pred, layers, steps, torch):
     }
 
 
-def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wobble=0.0, wall=True):
+def ar1_inputs(torch, g, T, layers, B, H, churn_lo, churn_hi, dt, dev):
+    """Predictor inputs [T, layers, B, H]: every (layer, row) follows x[t] = rho x[t-1] + sqrt(1 - rho^2) eps with
+    N(0,1) marginals; rho is drawn per step so that a threshold mask changes by about churn_lo .. churn_hi of its
+    set per step (measured for Gaussian scores at 35 % active: churn = 0.61 sqrt(1 - rho))."""
+    x = torch.randn(layers, B, H, generator=g, device=dev, dtype=torch.float32)
+    out = torch.empty(T, layers, B, H, device=dev, dtype=dt)
+    out[0] = x.to(dt)
+    for t in range(1, T):
+        c = churn_lo if churn_hi <= churn_lo else float(torch.empty(1).uniform_(churn_lo, churn_hi, generator=None))
+        rho = max(0.0, 1.0 - (c / 0.61) ** 2)
+        x = rho * x + (1.0 - rho * rho) ** 0.5 * torch.randn(layers, B, H, generator=g, device=dev, dtype=torch.float32)
+        out[t] = x.to(dt)
+    return out
+
+
+def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wobble=0.0, wall=True,
+                   mask_source="trace"):
     """One decode workload: W warm-up + K timed steps (one token through `layers` layers each, replayed from a HIP
     graph), then an eager pass over P of the same steps with per-kernel events.  Returns the result dict and what the
     CPU baseline needs (stack, trace, x_in, x_pred)."""
@@ -313,7 +334,12 @@ def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wob
     trace = torch.from_numpy(syn.mask_trace(args.seed + 7, layers, I, n, T, wl.churn_lo, wl.churn_hi,
                                              count_wobble)).to(dev)
     # predictor inputs per layer and step, MLP input of the first layer per step
-    x_pred = torch.randn(T, layers, B, H, generator=g, device=dev, dtype=torch.float32).to(dt)
+    from_predictor = mask_source == "predictor"
+    if from_predictor:
+        torch.manual_seed(args.seed + 3)
+        x_pred = ar1_inputs(torch, g, T, layers, B, H, wl.churn_lo, wl.churn_hi, dt, dev)
+    else:
+        x_pred = torch.randn(T, layers, B, H, generator=g, device=dev, dtype=torch.float32).to(dt)
     x_in = torch.randn(T, B, H, generator=g, device=dev, dtype=torch.float32).to(dt)
 
     # bring every cache to the first mask of the trace (the big one-off shrink from all-ones)
@@ -323,13 +349,21 @@ def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wob
 
     use_graph = not args.no_graph
     stack.prepare(B, overlap=args.overlap, fused=not args.no_fused)
+    if from_predictor:
+        # the layers' own masks drive the caches; the first one brings each cache from the trace's first mask to
+        # the predictor's (a larger change than the steps that follow: inside the warm-up)
+        stack.use_trace_masks = False
+        trace_arg = None
     if use_graph:
-        stack.step_staged(x_in[0], x_pred[0], trace[0])     # first launches outside capture
+        stack.step_staged(x_in[0], x_pred[0], None if from_predictor else trace[0])     # first launches outside capture
         torch.cuda.synchronize()
         stack.capture()
 
+    def masks_of(t):
+        return None if from_predictor else trace[t]
+
     def run(t):
-        stack.step_staged(x_in[t], x_pred[t], trace[t], replay=use_graph)
+        stack.step_staged(x_in[t], x_pred[t], masks_of(t), replay=use_graph)
 
     for t in range(1, W + 1):
         run(t)
@@ -385,11 +419,18 @@ def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wob
         return out
 
     t_lo = W + K - 1 - P
+    seen_changed, seen_active = [], []
     for t in range(W + K - 1, t_lo, -1):
         _lib.check(L.st_profile_enable(per_step), "st_profile_enable")
-        stack.step_staged(x_in[t], x_pred[t], trace[t], replay=False)
+        stack.step_staged(x_in[t], x_pred[t], masks_of(t), replay=False)
         torch.cuda.synchronize()
         collect()
+        if from_predictor:      # what the updates of this step really did (read back from the caches' state words)
+            for layer in stack.layers:
+                layer.cache._dirty = True
+                stt = layer.cache.sync_state()
+                seen_changed.append(stt["n_changed"])
+                seen_active.append(stt["n_active"])
     per_kernel = summarise()
     # the cache update on its own (it has no kernel of its own in the fused path): a few more steps, forwards again
     unfused = None
@@ -397,7 +438,7 @@ def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wob
         stack.fused = False
         for t in range(t_lo + 2, min(t_lo + 2 + max(4, P // 4), W + K)):
             _lib.check(L.st_profile_enable(per_step), "st_profile_enable")
-            stack.step_staged(x_in[t], x_pred[t], trace[t], replay=False)
+            stack.step_staged(x_in[t], x_pred[t], masks_of(t), replay=False)
             torch.cuda.synchronize()
             collect()
         unfused = summarise()
@@ -408,7 +449,7 @@ def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wob
     # ---- begin/end events cannot show what it costs inside the chain: an empty kernel already reads 4 us
     # ---- between its two events, while a dependent empty kernel adds only 1.6 us to a replayed chain)
     wall_parts = None
-    if wall and use_graph and not args.overlap:
+    if wall and use_graph and not args.overlap and not from_predictor:
         def part_predictor():
             for l, layer in enumerate(stack.layers):
                 layer.predict_mask(stack.xp_stage[l], stack._t_ws)
@@ -460,6 +501,10 @@ def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wob
         mlp_us += per_kernel["mlp_batch_down"]["mean_us"]
     # changed rows per update over the timed steps (the trace swaps as many rows in as out)
     k_changed = float((trace[W + 1:W + K + 1] & ~trace[W:W + K]).sum(dim=-1).float().mean())
+    if from_predictor:
+        k_changed = float(np.mean(seen_changed))
+        n = int(round(float(np.mean(seen_active))))
+        alg_bytes = mats * n * H * esz
     upd_bytes = int(2 * mats * k_changed * H * esz)      # cache update: changed rows read + written
     launch_bytes = alg_bytes + (upd_bytes if dom == "cache_update_decode" else 0)
     achieved = launch_bytes / (mlp_us * 1e-6) / 1e9
@@ -529,7 +574,8 @@ def main():
     layers = args.layers or wl.layers
     B = args.batch or wl.batch
     result, (stack, trace, x_in, x_pred) = decode_measure(args, wl, torch, st, _lib, syn, layers, B, args.steps, args.warmup,
-                                                          args.profile_steps, args.count_wobble)
+                                                          args.profile_steps, args.count_wobble,
+                                                          mask_source=args.mask_source)
     if not args.no_prefill_probe and wl.dtype != "float32" and B == 1:
         # the MFMA path in the same line: 512 rows of x through the first layers' sparse MLPs (caches at the union of
         # the rows' masks).  Runs last: it moves those caches away from the decode trace.
@@ -554,7 +600,7 @@ def main():
                                       "sample": f"failed: {exc!r}"}
     default_run = (args.workload == "llama3b_stack_fp16" and not args.layers and not args.batch and args.churn < 0.0
                    and args.active_frac <= 0.0 and args.count_wobble == 0.0 and not args.no_graph and not args.overlap
-                   and not args.no_fused)
+                   and not args.no_fused and args.mask_source == "trace")
     if default_run and not args.no_other_workloads:
         del stack, trace, x_in, x_pred
         result["other_workloads"] = other_workloads(args, torch, st, _lib, syn)
@@ -581,15 +627,22 @@ def other_workloads(args, torch, st, _lib, syn, steps=12, warmup=4, profile_step
                 "stack_hbm_gbps": r["stack_hbm_gbps"], "kernels_us": {k: v["median_us"] for k, v in r["kernels_us"].items()}}
 
     out = {"steps": steps, "warmup": warmup}
-    runs = [(name, b, 0.0) for name, b in OTHER_WORKLOADS] + [("llama3b_stack_fp16", 1, 0.03)]
-    for name, b, wobble in runs:
+    runs = [(name, b, 0.0, "trace") for name, b in OTHER_WORKLOADS] + [("llama3b_stack_fp16", 1, 0.03, "trace"),
+                                                                       ("llama3b_stack_fp16", 1, 0.0, "predictor")]
+    for name, b, wobble, source in runs:
         wl = syn.WORKLOADS[name]
         layers = wl.layers if wl.layers > 1 else 16     # a single layer's weights would sit in the Infinity Cache
         key = f"{name}_b{b}" if wobble == 0.0 else f"{name}_b{b}_count_wobble_{wobble}"
+        if source == "predictor":
+            key += "_mask_source_predictor"
+        short = wobble == 0.0 and source == "trace"
         try:
-            r, keep = decode_measure(args, wl, torch, st, _lib, syn, layers, b, steps if wobble == 0.0 else 20, warmup,
-                                     profile_steps, wobble, wall=False)
+            r, keep = decode_measure(args, wl, torch, st, _lib, syn, layers, b, steps if short else 20, warmup,
+                                     profile_steps, wobble, wall=False, mask_source=source)
             out[key] = brief(r)
+            if source == "predictor":
+                out[key]["n_active_mean"] = r["config"]["n_active"]
+                out[key]["changed_rows_mean"] = r["config"]["changed_rows_mean"]
             del keep
         except Exception as exc:
             out[key] = {"error": repr(exc)}
