@@ -519,7 +519,8 @@ def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wob
         "dtype": {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[wl.dtype], "data": "synthetic",
         "config": {"workload": wl.name, "layers": layers, "hidden": H, "intermediate": I, "predictor_rank": wl.rank,
                    "batch": B, "act": wl.act, "has_gate": wl.has_gate, "n_active": n,
-                   "churn": [wl.churn_lo, wl.churn_hi], "count_wobble": count_wobble, "mask_source": "trace",
+                   "churn": [wl.churn_lo, wl.churn_hi], "count_wobble": count_wobble, "mask_source": mask_source,
+                   "changed_rows_mean": round(k_changed, 1),
                    "launch": "hip_graph" if use_graph else "eager",
                    "streams": 2 if args.overlap else 1, "update_fused_into_decode": bool(stack.fused),
                    "kernel_timing": "hip events stamped at kernel begin/end (hipExtLaunchKernelGGL), eager second pass"},

@@ -74,9 +74,10 @@ const char *st_last_error(void);
  *   workspace          scratch of st_mlp_workspace_bytes(B,H,n) bytes
  * All rows must be 16-byte aligned (H*sizeof(dtype) % 16 == 0). B <= 4096.
  * B <= 2 (and any B < 32 in fp32 or with a hidden size the MFMA kernels do not
- * cover) runs the streaming decode kernel; 3 <= B <= 32 in fp16 / bf16 with H in
- * {2048, 3072, 4096} runs the MFMA batch kernels (still HBM-bound, one pass over
- * the weights); otherwise B >= 32 in fp16 / bf16 with H % 128 == 0
+ * cover) runs the streaming decode kernel; 3 <= B <= 32 in fp16 / bf16 with
+ * H % 256 == 0 (H <= 16384) runs the MFMA batch kernels (still HBM-bound; one
+ * pass over the weights per 32 rows of x for H in {2048, 3072, 4096}, per 16
+ * rows otherwise); otherwise B >= 32 in fp16 / bf16 with H % 128 == 0
  * runs the MFMA GEMM kernels (then only columns [0,n) of `combined` carry results; when its rows are 16-byte
  * aligned and have room, the kernels keep their intermediate there and also zero the columns from n up to the next
  * multiple of 128).
@@ -116,7 +117,8 @@ int st_mlp_forward_static(const void *x, int64_t B, int64_t H, const void *gate_
  *   scores  optional float [B,I] (NULL = not written)
  *   mask    uint8 [I]: mask[i] = any_b(score[b,i] >= thr)  (cmp_ge != 0)
  *                               any_b(score[b,i] >  thr)  (cmp_ge == 0)
- * H*sizeof(dtype) and r*sizeof(dtype) must be multiples of 16. B <= 64.
+ * H*sizeof(dtype) and r*sizeof(dtype) must be multiples of 16.  More than 64 rows
+ * of x (fewer for ranks above 224) run as several passes over the predictor's weights.
  * ------------------------------------------------------------------------ */
 int st_predictor_mask(const void *x, int64_t B, int64_t H, const void *A, int64_t r, const void *Bm, int64_t I,
                       int dtype, float thr, int cmp_ge, float *t_ws, float *scores, uint8_t *mask, void *stream);

@@ -220,6 +220,140 @@ __global__ __launch_bounds__(kBtThreads) void batch_gateup_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// kernel 1 for any hidden size that is a multiple of 256 (the hidden sizes above have instantiations of their own):
+// the number of k-steps per wave is a run-time value, the weight fragments go through a ring of kBtRing slots, and
+// the x fragments come from LDS while a 16-row tile of x fits there (XLDS: H <= 4096) or straight from memory
+// (hits in L1 / L2 after the first tile) beyond.  One tile of 16 rows of x per pass; same block / tile / wave
+// decomposition and the same sums as batch_gateup_kernel<T, KSW, HG, 1>.
+// ---------------------------------------------------------------------------
+constexpr int kBtRing = 4;
+
+template <typename T, bool HG, bool XLDS>
+__global__ __launch_bounds__(kBtThreads) void batch_gateup_anyh_kernel(
+    const T *__restrict__ x, int B, int H, const T *__restrict__ gate, const T *__restrict__ up, int n_host,
+    const int *__restrict__ n_dev, T *__restrict__ hbuf, int ldh, T *__restrict__ combined, long ldc, int act)
+{
+    const int KSW = H / 256, XP = H + kBtXPad;
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    T *xs = reinterpret_cast<T *>(lds_raw);                                                      // [16][XP] (XLDS)
+    float *red = reinterpret_cast<float *>(lds_raw + (XLDS ? (size_t)kBtRows * XP * 2 : 0));     // [8][2][4][64]
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), w = tid >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const int G = gridDim.x, blk = blockIdx.x;
+
+    const int n = device_count(n_host, n_dev);
+    const int R = (n + G - 1) / G;
+    const int row0 = blk * R;
+    const int jcount = n - row0 < R ? n - row0 : R;
+    if (jcount <= 0) return;
+
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+    const int ntile = (jcount + kBtTile - 1) / kBtTile;
+
+    bool v0, v1;
+    size_t o0, o1;
+    auto setup = [&](int t) __attribute__((always_inline)) {
+        const int j0 = t * kBtTile + r, j1 = j0 + 16;
+        v0 = j0 < jcount; v1 = j1 < jcount;
+        o0 = (size_t)(row0 + (v0 ? j0 : 0)) * H + 8 * q + 32 * w;
+        o1 = (size_t)(row0 + (v1 ? j1 : 0)) * H + 8 * q + 32 * w;
+    };
+    uint4 g0[kBtRing], u0[kBtRing], g1[kBtRing], u1[kBtRing];
+    auto issue = [&](int slot, int j) __attribute__((always_inline)) {
+        const int col = 256 * j;
+        u0[slot] = zero4; u1[slot] = zero4;
+        if (HG) { g0[slot] = zero4; g1[slot] = zero4; }
+        if (v0) {
+            u0[slot] = ld16(up + o0 + col);
+            if (HG) g0[slot] = ld16(gate + o0 + col);
+        }
+        if (v1) {
+            u1[slot] = ld16(up + o1 + col);
+            if (HG) g1[slot] = ld16(gate + o1 + col);
+        }
+    };
+
+    const bool xrow_ok = r < B;
+    const T *xglob = x + (size_t)(xrow_ok ? r : 0) * H + 8 * q + 32 * w;
+    const T *xfrag = xs + (size_t)r * XP + 8 * q + 32 * w;
+    if constexpr (XLDS) {   // stage the tile of x: 16 rows x H/8 chunks, KSW chunks per thread
+        const int chunks = H / 8;
+        for (int i = 0; i < KSW; ++i) {
+            const int idx = tid + kBtThreads * i;
+            const int b = idx / chunks, c = idx - b * chunks;
+            uint4 xv = zero4;
+            if (b < B) xv = ld16(x + (size_t)b * H + c * 8);
+            *reinterpret_cast<uint4 *>(xs + (size_t)b * XP + c * 8) = xv;
+        }
+    }
+    setup(0);
+#pragma unroll
+    for (int sl = 0; sl < kBtRing; ++sl)
+        if (sl < KSW) issue(sl, sl);
+    if constexpr (XLDS) __syncthreads();
+
+    for (int t = 0; t < ntile; ++t) {
+        if (t > 0) {
+            setup(t);
+#pragma unroll
+            for (int sl = 0; sl < kBtRing; ++sl)
+                if (sl < KSW) issue(sl, sl);
+        }
+        f32x4_t dg0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, du0 = dg0, dg1 = dg0, du1 = dg0;
+        for (int jb = 0; jb < KSW; jb += kBtRing) {
+#pragma unroll
+            for (int sl = 0; sl < kBtRing; ++sl) {
+                const int j = jb + sl;
+                if (j < KSW) {   // uniform
+                    uint4 xf;
+                    if constexpr (XLDS) xf = *reinterpret_cast<const uint4 *>(xfrag + 256 * j);
+                    else xf = xrow_ok ? ld16(xglob + 256 * j) : zero4;
+                    du0 = Mfma<T>::run(u0[sl], xf, du0);
+                    if (HG) dg0 = Mfma<T>::run(g0[sl], xf, dg0);
+                    du1 = Mfma<T>::run(u1[sl], xf, du1);
+                    if (HG) dg1 = Mfma<T>::run(g1[sl], xf, dg1);
+                    if (j + kBtRing < KSW) issue(sl, j + kBtRing);
+                }
+            }
+        }
+        // sum the 8 waves' partial tiles, one 16-row subtile at a time (as in batch_gateup_kernel)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            if (s == 1 && jcount - t * kBtTile <= 16) break;
+            float *mine = red + (size_t)w * 512 + lane;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (HG) mine[e * 64] = s == 0 ? dg0[e] : dg1[e];
+                mine[(4 + e) * 64] = s == 0 ? du0[e] : du1[e];
+            }
+            __syncthreads();
+            if (tid < 256) {
+                const int e = (tid >> 6) & 3, dl = tid & 63;
+                float sg = 0.f, su = 0.f;
+#pragma unroll
+                for (int ww = 0; ww < kBtWaves; ++ww) {
+                    if (HG) sg += red[(size_t)ww * 512 + e * 64 + dl];
+                    su += red[(size_t)ww * 512 + (4 + e) * 64 + dl];
+                }
+                const int j = t * kBtTile + 16 * s + 4 * (dl >> 4) + e;
+                const int b = dl & 15;
+                if (j < jcount) {
+                    const float hv = HG ? activate(sg, act) * su : activate(su, act);
+                    const int row = row0 + j;
+                    hbuf[(size_t)b * ldh + row] = from_float<T>(hv);
+                    if (combined && b < B) {
+                        combined[(size_t)b * ldc + row] = from_float<T>(hv);
+                        if (HG) combined[(size_t)b * ldc + n + row] = from_float<T>(su);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // kernel 2.  Block = (column group cg, row split rs); NP = 64-column pieces per
 // block; NX = tiles of 16 rows of x.  partial[(rs * 16 NX + b) * H + col], fp32.
 // ---------------------------------------------------------------------------
@@ -351,13 +485,14 @@ __global__ __launch_bounds__(kBtThreads) void batch_down_kernel(
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
-struct BatchShape { int ksw, np, cg, rs; };
+struct BatchShape { int ksw, np, cg, rs; bool special; };
+constexpr int kBtMaxH = 16384;
 
 static bool batch_shape(int H, BatchShape &s)
 {
-    if (H % 256 != 0) return false;
+    if (H % 256 != 0 || H < 256 || H > kBtMaxH) return false;
     s.ksw = H / 256;
-    if (s.ksw != 8 && s.ksw != 12 && s.ksw != 16) return false;
+    s.special = s.ksw == 8 || s.ksw == 12 || s.ksw == 16;   // hidden sizes with kernels instantiated for them
     const int pieces = H / 64;
     s.np = pieces % 3 == 0 ? 3 : 2;   // 4 pieces with two chunks in flight would not fit the register file
     s.cg = pieces / s.np;
@@ -399,6 +534,27 @@ static int launch_gateup(const T *x, int B, const T *gate, const T *up, int n, c
     return ST_OK;
 }
 
+template <typename T, bool HG>
+static int launch_gateup_anyh(const T *x, int B, int H, const T *gate, const T *up, int n, const int *n_dev, T *hbuf,
+                              int ldh, T *comb, long ldc, int act, hipStream_t stream)
+{
+    const bool xlds = H <= 4096;
+    const size_t lds = (xlds ? (size_t)kBtRows * (H + kBtXPad) * 2 : 0) + (size_t)kBtRedFloats * 4;
+    ProfScope ps(ST_K_MLP_BATCH_GATEUP, stream);
+    if (xlds) {
+        auto kern = batch_gateup_anyh_kernel<T, HG, true>;
+        const int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), 152 * 1024);
+        if (rc != ST_OK) return rc;
+        ST_LAUNCH(ps, kern, dim3(device_cu_count()), dim3(kBtThreads), lds, stream, x, B, H, gate, up, n, n_dev, hbuf,
+                  ldh, comb, ldc, act);
+    } else {
+        auto kern = batch_gateup_anyh_kernel<T, HG, false>;
+        ST_LAUNCH(ps, kern, dim3(device_cu_count()), dim3(kBtThreads), lds, stream, x, B, H, gate, up, n, n_dev, hbuf,
+                  ldh, comb, ldc, act);
+    }
+    return ST_OK;
+}
+
 template <typename T, int NP, int NX>
 static int launch_down(const T *hbuf, int ldh, int B, const T *down, int H, int n, const int *n_dev, float *partial,
                        int cg, int rs, hipStream_t stream)
@@ -430,9 +586,10 @@ static int launch_batch_t(const void *x_, int B, int H, const void *gate_, const
     float *partial = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + hh_bytes);
     const T *gate = static_cast<const T *>(gate_), *up = static_cast<const T *>(up_);
     const T *down = static_cast<const T *>(down_);
-    // gate / up: one pass over the weights per 32 rows of x; down: one per 16
-    for (int b0 = 0; b0 < B; b0 += 2 * kBtRows) {
-        const int bc = B - b0 < 2 * kBtRows ? B - b0 : 2 * kBtRows;
+    // gate / up: one pass over the weights per 32 rows of x (16 with the kernel for other hidden sizes); down: one per 16
+    const int pass_rows = s.special ? 2 * kBtRows : kBtRows;
+    for (int b0 = 0; b0 < B; b0 += pass_rows) {
+        const int bc = B - b0 < pass_rows ? B - b0 : pass_rows;
         const T *x = static_cast<const T *>(x_) + (size_t)b0 * H;
         T *comb = comb_ ? static_cast<T *>(comb_) + (size_t)b0 * ldc : nullptr;
         int rc;
@@ -442,7 +599,10 @@ static int launch_batch_t(const void *x_, int B, int H, const void *gate_, const
                          : launch_gateup<T, KSW, false, 2>(x, bc, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream)) \
              : (has_gate ? launch_gateup<T, KSW, true, 1>(x, bc, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream)   \
                          : launch_gateup<T, KSW, false, 1>(x, bc, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream))
-        if (s.ksw == 8) ST_BT_GATEUP(8);
+        if (!s.special)
+            rc = has_gate ? launch_gateup_anyh<T, true>(x, bc, H, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream)
+                          : launch_gateup_anyh<T, false>(x, bc, H, gate, up, n, n_dev, hbuf, ldh, comb, ldc, act, stream);
+        else if (s.ksw == 8) ST_BT_GATEUP(8);
         else if (s.ksw == 12) ST_BT_GATEUP(12);
         else ST_BT_GATEUP(16);
 #undef ST_BT_GATEUP

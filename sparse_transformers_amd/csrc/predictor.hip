@@ -95,7 +95,8 @@ template <typename T, int LPR, int RPW>
 __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_kernel(const float *__restrict__ t, int B, int r,
                                                                   const T *__restrict__ Bm, int I, float thr,
                                                                   int cmp_ge, float *__restrict__ scores,
-                                                                  uint8_t *__restrict__ mask, int round_storage)
+                                                                  uint8_t *__restrict__ mask, int round_storage,
+                                                                  int accumulate)
 {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int RPI = kWave / LPR;                                          // rows per iteration
@@ -184,7 +185,8 @@ __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_kernel(const
     for (int it = 0; it < NIT; ++it) {
         const int ro = it * RPI + gidx;
         const int row = tile + ro;
-        if (cl == 0 && ro < RPW && row < I) mask[row] = any[it] ? 1 : 0;
+        // (accumulate: a later pass over more rows of x only ever switches bytes on)
+        if (cl == 0 && ro < RPW && row < I && (any[it] || !accumulate)) mask[row] = any[it] ? 1 : 0;
     }
 }
 
@@ -197,7 +199,8 @@ template <typename T, int LPR, int NITER>
 __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_rows_kernel(const float *__restrict__ t, int B, int r,
                                                                        const T *__restrict__ Bm, int I, float thr,
                                                                        int cmp_ge, float *__restrict__ scores,
-                                                                       uint8_t *__restrict__ mask, int round_storage)
+                                                                       uint8_t *__restrict__ mask, int round_storage,
+                                                                       int accumulate)
 {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int RPI = kWave / LPR;   // rows per iteration
@@ -267,24 +270,24 @@ __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_rows_kernel(
 #pragma unroll
     for (int it = 0; it < NITER; ++it) {
         const int row = tile + it * RPI + gidx;
-        if (cl == 0 && row < I) mask[row] = (any >> it) & 1u;
+        if (cl == 0 && row < I && (((any >> it) & 1u) || !accumulate)) mask[row] = (any >> it) & 1u;
     }
 }
 
 template <typename T, int LPR, int RPW>
 static void launch_up_rpw(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
-                          float *scores, uint8_t *mask, int round_storage, hipStream_t stream)
+                          float *scores, uint8_t *mask, int round_storage, int accumulate, hipStream_t stream)
 {
     constexpr size_t batch = (size_t)kPredUpThreads * 2 * 16;   // the staging buffer is padded to whole batches
     const size_t lds = ((size_t)B * r * sizeof(float) + batch - 1) / batch * batch;
     constexpr int rows = RPW * (kPredUpThreads / kWave);
     ST_LAUNCH(ps, (predictor_up_mask_kernel<T, LPR, RPW>), dim3((I + rows - 1) / rows), dim3(kPredUpThreads), lds,
-              stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask, round_storage);
+              stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask, round_storage, accumulate);
 }
 
 template <typename T, int LPR>
 static void launch_up(ProfScope &ps, const float *t_ws, int B, int r, const void *Bm, int I, float thr, int cmp_ge,
-                      float *scores, uint8_t *mask, int round_storage, hipStream_t stream)
+                      float *scores, uint8_t *mask, int round_storage, int accumulate, hipStream_t stream)
 {
     constexpr int NITER = LPR >= 16 ? LPR / 16 : 1;   // about four rows of Bm per wave (measured against 1, 2 and 8 per lane)
     if (B > 1 && r / Elem<T>::kVec <= LPR) {
@@ -292,15 +295,17 @@ static void launch_up(ProfScope &ps, const float *t_ws, int B, int r, const void
         const size_t lds = ((size_t)B * r * sizeof(float) + batch - 1) / batch * batch;
         constexpr int rows = (kWave / LPR) * NITER * (kPredUpThreads / kWave);
         ST_LAUNCH(ps, (predictor_up_mask_rows_kernel<T, LPR, NITER>), dim3((I + rows - 1) / rows), dim3(kPredUpThreads),
-                  lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask, round_storage);
+                  lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask, round_storage, accumulate);
         return;
     }
-    launch_up_rpw<T, LPR, pred_rows_per_wave(LPR)>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
+    launch_up_rpw<T, LPR, pred_rows_per_wave(LPR)>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage,
+                                                   accumulate, stream);
 }
 
 template <typename T>
 static int launch_predictor(const void *x, int B, int H, const void *A, int r, const void *Bm, int I, float thr,
-                            int cmp_ge, float *t_ws, float *scores, uint8_t *mask, int round_storage, hipStream_t stream)
+                            int cmp_ge, float *t_ws, float *scores, uint8_t *mask, int round_storage, int accumulate,
+                            hipStream_t stream)
 {
     constexpr int VEC = Elem<T>::kVec;
     {
@@ -319,11 +324,11 @@ static int launch_predictor(const void *x, int B, int H, const void *A, int r, c
     const int chunks = r / VEC;
     {
         ProfScope ps(ST_K_PRED_UP_MASK, stream);
-        if (chunks <= 4) launch_up<T, 4>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
-        else if (chunks <= 8) launch_up<T, 8>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
-        else if (chunks <= 16) launch_up<T, 16>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
-        else if (chunks <= 32) launch_up<T, 32>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
-        else launch_up<T, 64>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, stream);
+        if (chunks <= 4) launch_up<T, 4>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, accumulate, stream);
+        else if (chunks <= 8) launch_up<T, 8>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, accumulate, stream);
+        else if (chunks <= 16) launch_up<T, 16>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, accumulate, stream);
+        else if (chunks <= 32) launch_up<T, 32>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, accumulate, stream);
+        else launch_up<T, 64>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage, accumulate, stream);
     }
     ST_HIP(hipGetLastError());
     return ST_OK;
@@ -339,24 +344,36 @@ extern "C" int st_predictor_mask_ex(const void *x, int64_t B, int64_t H, const v
     ST_REQUIRE(x && A && Bm && t_ws && mask, "st_predictor_mask_ex: null pointer");
     ST_REQUIRE(dtype >= ST_F32 && dtype <= ST_BF16, "st_predictor_mask_ex: unknown dtype %d", dtype);
     const int esz = dtype == ST_F32 ? 4 : 2;
-    ST_REQUIRE(B >= 1 && B <= 64, "st_predictor_mask_ex: B=%lld out of range [1,64]", (long long)B);
+    ST_REQUIRE(B >= 1 && B <= (1 << 20), "st_predictor_mask_ex: B=%lld out of range", (long long)B);
     ST_REQUIRE(H >= 1 && (H * esz) % 16 == 0, "st_predictor_mask_ex: H=%lld rows are not 16-byte multiples",
                (long long)H);
     ST_REQUIRE(r >= 1 && (r * esz) % 16 == 0, "st_predictor_mask_ex: rank %lld rows are not 16-byte multiples",
                (long long)r);
     ST_REQUIRE(I >= 1 && I <= (1 << 24), "st_predictor_mask_ex: I=%lld out of range", (long long)I);
-    ST_REQUIRE(B * r * 4 <= 56 * 1024, "st_predictor_mask_ex: B*r=%lld too large for the LDS staging buffer",
-               (long long)(B * r));
+    ST_REQUIRE(r * 4 <= 56 * 1024, "st_predictor_mask_ex: rank %lld too large for the LDS staging buffer", (long long)r);
     const uintptr_t align = (uintptr_t)x | (uintptr_t)A | (uintptr_t)Bm;
     ST_REQUIRE((align & 15) == 0, "st_predictor_mask_ex: pointers must be 16-byte aligned");
     ST_REQUIRE((flags & ~ST_PRED_ROUND_STORAGE) == 0, "st_predictor_mask_ex: unknown flags %d", flags);
     const int round_storage = (flags & ST_PRED_ROUND_STORAGE) && dtype != ST_F32 ? 1 : 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    switch (dtype) {
-    case ST_F32: return launch_predictor<float>(x, (int)B, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, scores, mask, round_storage, s);
-    case ST_F16: return launch_predictor<f16_t>(x, (int)B, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, scores, mask, round_storage, s);
-    default: return launch_predictor<bf16_t>(x, (int)B, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, scores, mask, round_storage, s);
+    // Rows of x per pass: what the staging buffer of the second kernel holds, 64 at most.  Further passes reuse
+    // the front of t_ws (the launches are ordered on the stream) and only ever switch mask bytes on.
+    int64_t per = (56 * 1024) / (r * 4);
+    per = per > 64 ? 64 : per;
+    for (int64_t b0 = 0; b0 < B; b0 += per) {
+        const int bc = (int)(B - b0 < per ? B - b0 : per);
+        const void *xp = static_cast<const unsigned char *>(x) + (size_t)b0 * H * esz;
+        float *sp = scores ? scores + (size_t)b0 * I : nullptr;
+        const int acc = b0 > 0 ? 1 : 0;
+        int rc;
+        switch (dtype) {
+        case ST_F32: rc = launch_predictor<float>(xp, bc, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, sp, mask, round_storage, acc, s); break;
+        case ST_F16: rc = launch_predictor<f16_t>(xp, bc, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, sp, mask, round_storage, acc, s); break;
+        default: rc = launch_predictor<bf16_t>(xp, bc, (int)H, A, (int)r, Bm, (int)I, thr, cmp_ge, t_ws, sp, mask, round_storage, acc, s); break;
+        }
+        if (rc != ST_OK) return rc;
     }
+    return ST_OK;
 }
 
 extern "C" int st_predictor_mask(const void *x, int64_t B, int64_t H, const void *A, int64_t r, const void *Bm,

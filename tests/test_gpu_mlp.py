@@ -255,7 +255,7 @@ def test_prefill_leaves_the_parent_of_a_column_slice_alone():
     assert_close(parent[:, :n].float().cpu().numpy(), wantc[:, :n], "float16", "combined view")
 
 
-# ---- MFMA batch kernels (3 <= B <= 32, fp16 / bf16, H in {2048, 3072, 4096}) ----
+# ---- MFMA batch kernels (3 <= B <= 32, fp16 / bf16, hidden sizes that are multiples of 256) ----
 @pytest.mark.parametrize("name,B,H,n,dtype,act,has_gate", [
     ("llama-3b bf16, 4 rows", 4, 3072, 4620, "bfloat16", "silu", True),
     ("llama-3b bf16, 16 rows", 16, 3072, 7660, "bfloat16", "silu", True),
@@ -266,6 +266,13 @@ def test_prefill_leaves_the_parent_of_a_column_slice_alone():
     ("32 rows: two full passes", 32, 3072, 2867, "float16", "silu", True),
     ("one active row", 5, 2048, 1, "float16", "silu", True),
     ("33 rows per block (two tiles)", 3, 2048, 8450, "float16", "silu", False),
+    # hidden sizes without a kernel instantiated for them (run-time K loop; x from LDS up to 4096 columns, from memory beyond)
+    ("qwen2-7b width 3584, 8 rows", 8, 3584, 2500, "bfloat16", "silu", True),
+    ("width 5120, 4 rows (x straight from memory)", 4, 5120, 1800, "float16", "silu", True),
+    ("opt-125m width 768, 16 rows, ungated relu", 16, 768, 1111, "float16", "relu", False),
+    ("qwen2-1.5b width 1536, 20 rows (two passes of 16 + 4)", 20, 1536, 3000, "bfloat16", "silu", True),
+    ("width 8192, 3 rows, ragged tiles", 3, 8192, 1031, "float16", "gelu_pytorch_tanh", True),
+    ("width 256, 5 rows: a single k-step per wave", 5, 256, 300, "float16", "silu", True),
 ])
 def test_batch_mfma_vs_oracle(name, B, H, n, dtype, act, has_gate):
     x, cw, dn = _case(4242 + B + n, B, H, n, dtype, has_gate)

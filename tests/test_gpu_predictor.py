@@ -31,6 +31,8 @@ def _weights(seed, B, H, r, I, dtype):
     (3, 128, 8, 50, "float16", 0.5),           # tiny / ragged
     (2, 64, 4, 17, "float32", 0.5),
     (1, 1024, 1024, 300, "float16", 0.4),      # rank rows longer than one pass of the wave
+    (150, 1024, 64, 2048, "float16", 0.02),    # more rows than one pass takes (64): three passes, mask bytes accumulate
+    (70, 512, 256, 1024, "bfloat16", 0.02),    # rank 256: a pass takes 56 rows
 ])
 def test_scores_and_mask(B, H, r, I, dtype, frac):
     x, A, Bm = _weights(B * 7 + r, B, H, r, I, dtype)
