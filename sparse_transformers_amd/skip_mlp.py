@@ -114,7 +114,15 @@ class SkipMLP(torch.nn.Module):
     multiplies ``x`` with ``get_concat_weight()`` in torch (src/modeling_skip.py:114-117) and therefore never
     reaches ``sparse_mlp_forward``; replacing the module is what puts the kernels on the path.
     ``use_sparse=False`` is the dense MLP in torch, which is what the reference runs for prefill.
-    Like the reference's cache path, the sparse forward ignores biases."""
+    Like the reference's cache path, the sparse forward ignores biases.
+
+    ``lazy_cache_updates`` (class attribute, default True): the module's cache only remembers the mask handed to
+    ``weight_cache.update_active_weights`` -- the decoder layer's call, made before attention
+    (src/modeling_skip.py:217,235-238) -- and applies it together with this module's forward as one fused
+    update + MLP launch.  The price: an update that leaves nothing active is reported by the next synchronising
+    call instead of by ``update_active_weights``.  Set it to False for the reference's timing of that error."""
+
+    lazy_cache_updates = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, sparsity: float, bias: bool = False,
                  act_fn: str = "silu", use_weight_cache: bool = True, has_gate: bool = True):
@@ -163,6 +171,7 @@ class SkipMLP(torch.nn.Module):
             self.weight_cache = WeightCache(self.init_mask, self.hidden_size,
                                             self.gate_proj.weight if self.has_gate else None, self.up_proj.weight,
                                             self.down_proj.weight, self.has_gate)
+            self.weight_cache.lazy_updates = bool(self.lazy_cache_updates)
 
     def reset_cache(self) -> None:
         """What the reference's model-level ``reset_cache`` does per layer (src/modeling_skip.py:492-497): drop

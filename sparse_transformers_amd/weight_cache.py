@@ -8,6 +8,7 @@ tensors; the bookkeeping (ordered active list, mask diff, pairing, swap-with-las
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 from typing import Optional
 
 import torch
@@ -23,8 +24,12 @@ class ConcatWeightHandle(torch.Tensor):
     gate / up rows in place, so the reference's call sequence costs no ``[2n,H]`` copy (the reference pays a
     ``torch::cat`` per update, weight_cache.h:138).  Any other torch operation on it (``.t()``, ``matmul``,
     indexing, ``.cpu()`` ...) first materialises the contiguous tensor with one device copy and then runs on
-    that.  Like the reference's tensor it describes the cache as of the update it was fetched after; using it
-    after a later update raises instead of silently showing newer rows under the old shape."""
+    that.  Like the reference's tensor it describes the cache as of the update it was fetched after: a handle that is
+    still alive when the next update is enqueued through this object is filled first (one device copy), so it stays a
+    snapshot as the reference's ``torch::cat`` result does; when nobody holds it any more -- the usual case, a handle
+    fetched for one forward -- nothing is copied.  Updates that bypass this object's methods (a replayed HIP graph)
+    cannot do that: a handle that was not filled before such an update raises when it is used, instead of silently
+    showing newer rows under the old shape."""
 
     @staticmethod
     def __new__(cls, cache: "WeightCache", n: int, serial: int):
@@ -72,6 +77,12 @@ class WeightCache:
     Fast path (nothing is read back, everything is stream-ordered):
       ``update_active_weights_async(mask)`` then ``forward(x, act, ...)``; the kernels take the active
       count from device memory.
+    ``lazy_updates = True`` (off by default; the drop-in ``SkipMLP`` module switches it on for its cache) makes
+    ``update_active_weights(mask)`` only remember the mask: the update then runs with the next ``forward`` as ONE
+    fused update + MLP launch (``update_and_forward``) -- the order a decoder layer produces, where the mask is
+    computed before attention and the MLP runs after it (src/modeling_skip.py:234-261) -- or, if a getter or
+    another update comes first, on its own.  The caller must leave the mask tensor alone until then, and "No active
+    weights" is reported by the next call that synchronises instead of by ``update_active_weights`` itself.
     """
 
     def __init__(self, init_mask: torch.Tensor, hidden_size: int, gate_weight: Optional[torch.Tensor],
@@ -128,7 +139,9 @@ class WeightCache:
         self._host_state = (C.c_int32 * _lib.STATE_WORDS)()
         self._host_serial = -1      # serial the host copy of the state belongs to
         self._dirty = True          # updates enqueued since the last read-back
-        self._concat: Optional[torch.Tensor] = None
+        self.lazy_updates = False
+        self._pending_mask: Optional[torch.Tensor] = None
+        self._concat_ref = None     # weak reference to the handle get_concat_weight() handed out last
         self._concat_serial = -1
         # weight_cache.h:226: the constructor ends with update_active_weights(init_mask)
         self.update_active_weights(init_mask)
@@ -148,15 +161,34 @@ class WeightCache:
             raise ValueError(f"mask must have {self.intermediate_size} elements, got {mask.numel()}")
         return mask if mask.is_contiguous() else mask.contiguous()
 
+    def _keep_snapshot(self) -> None:
+        """Before an update overwrites packed rows: a concat handle somebody still holds is filled now (the
+        reference's tensor is a copy and survives later updates, weight_cache.h:138)."""
+        h = self._concat_ref() if self._concat_ref is not None else None
+        if h is not None and h._real is None and h.fresh():
+            h.materialize()
+
+    def _flush_pending(self) -> None:
+        """A remembered mask (``lazy_updates``) that no forward has consumed is applied now, on its own."""
+        m, self._pending_mask = self._pending_mask, None
+        if m is not None:
+            self.update_active_weights_async(m)
+
     def update_active_weights_async(self, mask: torch.Tensor) -> None:
         """Enqueue the differential update on the current stream; never waits for the device."""
         m = self._mask_arg(mask)
+        self._flush_pending()
+        self._keep_snapshot()
         rc = _lib.lib().st_cache_update_async(self._h, m.data_ptr(), current_stream_ptr(self.device))
         _lib.check(rc, "st_cache_update_async")
         self._dirty = True
 
     def update_active_weights(self, mask: torch.Tensor) -> None:
         """weight_cache.h:229: raises RuntimeError("No active weights") when the mask empties the cache."""
+        if self.lazy_updates:
+            self._flush_pending()
+            self._pending_mask = self._mask_arg(mask)
+            return
         known = not self._dirty
         serial = int(self._host_state[_lib.STATE_SERIAL])
         self.update_active_weights_async(mask)
@@ -172,6 +204,7 @@ class WeightCache:
 
     def sync_state(self) -> dict:
         """Read the state words back (waits for the current stream)."""
+        self._flush_pending()
         if self._dirty:
             rc = _lib.lib().st_cache_sync_state(self._h, self._host_state, current_stream_ptr(self.device))
             self._dirty = False
@@ -201,9 +234,11 @@ class WeightCache:
         """``[2n,H]`` (gate rows then up rows; ``[n,H]`` when ungated), valid until the next update.  Returned
         as a ``ConcatWeightHandle``: no copy is made unless something other than ``sparse_mlp_forward`` reads it."""
         st = self._require_valid()
-        if self._concat is None or self._concat_serial != st["serial"]:
-            self._concat, self._concat_serial = ConcatWeightHandle(self, int(st["n_active"]), st["serial"]), st["serial"]
-        return self._concat
+        h = self._concat_ref() if self._concat_ref is not None else None
+        if h is None or self._concat_serial != st["serial"]:
+            h = ConcatWeightHandle(self, int(st["n_active"]), st["serial"])
+            self._concat_ref, self._concat_serial = weakref.ref(h), st["serial"]
+        return h
 
     def get_active_down_weight(self) -> torch.Tensor:
         """[H,n] view with strides (1,H) over the packed down rows (zero-copy)."""
@@ -231,6 +266,7 @@ class WeightCache:
         ``workspace``: a caller-owned uint8 buffer of ``mlp_workspace_bytes(B, H, I)`` bytes (default: one
         kept per device and stream)."""
         m = self._mask_arg(mask)
+        self._flush_pending()
         H, I = self.hidden_size, self.intermediate_size
         x2 = self._x_rows(x)
         B = x2.size(0)
@@ -243,6 +279,7 @@ class WeightCache:
         if act not in _lib.ACT_CODES:
             raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
         combined, copy_back = combined_for_launch(combined, B, I)
+        self._keep_snapshot()
         rc = _lib.lib().st_cache_update_forward(
             self._h, m.data_ptr(), x2.data_ptr(), B,
             int(self._host_state[_lib.STATE_N_ACTIVE]) if n_hint is None else int(n_hint), out.data_ptr(),
@@ -257,6 +294,11 @@ class WeightCache:
     def forward(self, x: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor] = None,
                 combined: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Sparse MLP on the cache's packed rows; the active count is read on the device."""
+        if self._pending_mask is not None:      # lazy_updates: the remembered update and this forward as one call
+            m, self._pending_mask = self._pending_mask, None
+            if combined is None or combined.size(-1) >= (2 if self.has_gate else 1) * self.intermediate_size:
+                return self.update_and_forward(m, x, act, out=out, combined=combined, workspace=workspace)
+            self.update_active_weights_async(m)   # `combined` is sized for the current count only: two calls
         x2 = self._x_rows(x)
         if out is None:
             out = torch.empty_like(x2)

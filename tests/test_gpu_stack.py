@@ -182,6 +182,45 @@ def test_skip_mlp_full_shape_vs_oracle(variant):
         assert mlp.weight_cache.get_active_indices().cpu().tolist() == oc.get_active_indices().tolist()
 
 
+def test_lazy_cache_updates_fuse_with_the_next_forward():
+    """The decoder layer's order (src/modeling_skip.py:234-261): update_active_weights(mask) early, the MLP later.
+    With lazy updates the module's cache remembers the mask and runs update + MLP as one launch at the forward;
+    outputs, ordered list and state equal those of a cache that updates at once, bit for bit; a getter or a second
+    update in between applies the remembered mask first; an emptying mask is reported by the next synchronising call."""
+    H, I = 1024, 2048
+    g = torch.Generator().manual_seed(4)
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.05).half().to(DEV)
+    gate, up, down = mk(I, H), mk(I, H), mk(H, I)
+    lazy = st.SkipMLP.from_weights(gate, up, down, 0.5, "silu")
+    eager = st.SkipMLP.from_weights(gate, up, down, 0.5, "silu")
+    eager.lazy_cache_updates = False
+    lazy.initialize_weight_cache()
+    eager.initialize_weight_cache()
+    assert lazy.weight_cache.lazy_updates and not eager.weight_cache.lazy_updates
+    m = torch.rand(I, generator=g) < 0.4
+    for step in range(6):
+        m = m ^ (torch.rand(I, generator=g) < 0.1)
+        md = m.to(DEV)
+        x = mk(1 if step != 3 else 3, H)
+        lazy.weight_cache.update_active_weights(md)
+        eager.weight_cache.update_active_weights(md)
+        assert lazy.weight_cache._pending_mask is not None
+        if step == 2:      # a getter before the forward: the remembered update runs on its own
+            assert lazy.weight_cache.get_num_active() == int(m.sum()) and lazy.weight_cache._pending_mask is None
+        if step == 4:      # a second update before any forward: both are applied, in order
+            m = m ^ (torch.rand(I, generator=g) < 0.1)
+            md = m.to(DEV)
+            lazy.weight_cache.update_active_weights(md)
+            eager.weight_cache.update_active_weights(md)
+        y_lazy, y_eager = lazy(x), eager(x)
+        assert lazy.weight_cache._pending_mask is None
+        assert torch.equal(y_lazy, y_eager), step
+        assert torch.equal(lazy.weight_cache.get_active_indices(), eager.weight_cache.get_active_indices()), step
+    lazy.weight_cache.update_active_weights(torch.zeros(I, dtype=torch.bool, device=DEV))   # accepted silently ...
+    with pytest.raises(RuntimeError, match="No active weights"):
+        lazy.weight_cache.get_num_active()                                                   # ... and reported here
+
+
 def test_reference_call_sequence_reads_the_cache_in_place():
     """update_active_weights -> get_concat_weight -> get_active_down_weight -> sparse_mlp_forward, as a caller of
     the reference's operator writes it: the concat weight is a handle that sparse_mlp_forward resolves to the
@@ -214,6 +253,20 @@ def test_reference_call_sequence_reads_the_cache_in_place():
     assert fresh is not stale and tuple(fresh.shape) == (2 * (I - n), H)
     with pytest.raises(RuntimeError):
         st.sparse_mlp_forward(x, ConcatStale(stale, wc, n), dw, db, cb, "silu")
+    # a handle that is still held when the next update comes is filled first and stays a snapshot of its update,
+    # as the reference's torch::cat result does; one that nobody holds costs nothing
+    order2 = wc.get_active_indices()
+    held = wc.get_concat_weight()
+    assert held._real is None
+    wc.update_active_weights(m)
+    assert held._real is not None and torch.equal(held + 0, torch.cat([gate[order2], up[order2]]))
+    dropped = wc.get_concat_weight()
+    assert dropped._real is None
+    del dropped
+    import gc
+    gc.collect()
+    assert wc._concat_ref() is None
+    wc.update_active_weights(~m)      # nothing left to fill
 
 
 def ConcatStale(stale, wc, n):
