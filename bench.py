@@ -139,20 +139,29 @@ def prefill_measure(stack, wl, T, layers, K, W, profile_steps, seed, torch, _lib
         ns.append(int(union.sum()))
     x0 = torch.randn(T, H, generator=g, device=dev, dtype=torch.float32).to(dt)
     bufs = [torch.empty(T, H, device=dev, dtype=dt) for _ in range(2)]
+    from sparse_transformers_amd.ops import mlp_workspace_bytes
+    ws = torch.empty(mlp_workspace_bytes(T, H, I), dtype=torch.uint8, device=dev)
 
     def step():
         x = x0
         for l, layer in enumerate(sub):
-            x = layer.cache.forward(x, wl.act, out=bufs[l & 1])
+            x = layer.cache.forward(x, wl.act, out=bufs[l & 1], workspace=ws)
         return x
 
-    for _ in range(W):
+    # the timed steps replay a HIP graph of the step, like the decode bench (launched one call at a time from
+    # Python the GPU waits for the host between the three kernels of a layer)
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
         step()
+    for _ in range(W):
+        graph.replay()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(K):
-        step()
+        graph.replay()
     e1.record()
     torch.cuda.synchronize()
     ms_per_step = e0.elapsed_time(e1) / K

@@ -713,16 +713,32 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     if (plan_wave) {
         // ---- per-word prefix counts of added / removed indices, eight words per lane at most
         const int wpl = (W32 + kWave - 1) >> 6;
-        uint32_t la[kSparseMaxW32 / kWave], lr[kSparseMaxW32 / kWave];
+        // (words per lane: at most 4 per 8-byte mask word a thread reads -- the host launches NW = 1 up to I = 8192 --
+        // so that the unrolled loops below are no longer than this launch needs: the code of this branch is run by one
+        // wave per block, once, and what it costs is mostly fetching it)
+        constexpr int kWpl = 4 * NW;
+        static_assert(kWpl * kWave * 32 >= 8 * TPB * NW, "the planning wave covers every mask word of the launch");
+        uint32_t la[kWpl], lr[kWpl], aw[kWpl];
         uint32_t ca = 0, cr = 0;
+        // (all reads of the bitmaps are issued together, from clamped addresses; the words stay in registers for the
+        // second pass)
+        uint32_t nwd[kWpl], owd[kWpl];
 #pragma unroll
-        for (int j = 0; j < kSparseMaxW32 / kWave; ++j) {
+        for (int j = 0; j < kWpl; ++j) {
+            const int t = lane * wpl + j;
+            const int tc = t < W32 ? t : W32 - 1;
+            nwd[j] = sh.newbits[tc];
+            owd[j] = sh.oldbits[tc];
+        }
+#pragma unroll
+        for (int j = 0; j < kWpl; ++j) {
             const int t = lane * wpl + j;
             const bool in = j < wpl && t < W32;
-            const uint32_t nwd = in ? sh.newbits[t] : 0u, owd = in ? sh.oldbits[t] : 0u;
+            const uint32_t nw = in ? nwd[j] : 0u, ow = in ? owd[j] : 0u;
             la[j] = ca; lr[j] = cr;
-            ca += (uint32_t)__popc(nwd & ~owd);
-            cr += (uint32_t)__popc(owd & ~nwd);
+            aw[j] = nw & ~ow;
+            ca += (uint32_t)__popc(aw[j]);
+            cr += (uint32_t)__popc(ow & ~nw);
         }
         const uint32_t packed = ca | (cr << 16);
         const uint32_t incl = wave_incl_scan_dpp(packed, lane);
@@ -730,15 +746,21 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
         // removed: per-word prefix counts (a position looks its old index's rank up); added: the ascending list itself
         uint16_t *added_list = reinterpret_cast<uint16_t *>(smem);   // (the region of the per-index plan, unused on this path)
 #pragma unroll
-        for (int j = 0; j < kSparseMaxW32 / kWave; ++j) {
+        for (int j = 0; j < kWpl; ++j) {
             const int t = lane * wpl + j;
             if (j < wpl && t < W32) {
                 sh.pr[t] = (uint16_t)((excl >> 16) + lr[j]);
-                uint32_t aw = sh.newbits[t] & ~sh.oldbits[t];
+                // (a word rarely holds more than two added indices: the first two go out without a loop)
+                uint32_t a = aw[j];
                 int o = (int)((excl & 0xffffu) + la[j]);
-                while (aw) {
-                    added_list[o++] = (uint16_t)(t * 32 + __ffs((int)aw) - 1);
-                    aw &= aw - 1u;
+                const uint32_t a2 = a & (a - 1u);
+                if (a) added_list[o] = (uint16_t)(t * 32 + __ffs((int)a) - 1);
+                if (a2) added_list[o + 1] = (uint16_t)(t * 32 + __ffs((int)a2) - 1);
+                a = a2 & (a2 - 1u);
+                o += 2;
+                while (a) {
+                    added_list[o++] = (uint16_t)(t * 32 + __ffs((int)a) - 1);
+                    a &= a - 1u;
                 }
             }
         }
