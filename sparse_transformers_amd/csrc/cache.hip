@@ -548,7 +548,7 @@ struct SparseShared {
     uint16_t pr[kSparseMaxW32];   // removed indices below each word
     int na, nr, n;
     int src[kSparseMaxQ];
-    int found, paired_tail, replay_ok, nchg;   // surplus removals (removed > added)
+    int found, paired_tail, replay_ok, fast_ok, nchg;   // surplus removals (removed > added)
 };
 
 // 0x01-per-element bytes -> 8 bits (element k -> bit k)
@@ -796,6 +796,141 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
                 if ((na_w | nr_w) != 0) indices2[(size_t)(ep ^ 1) * I + my_p] = newidx;
             }
             if (lane == 0) sh.n = nn;
+        } else {
+            // ---- Removals outnumber additions: the surplus ones are taken out one by one, in ascending index order,
+            // each by moving the last entry of the list into its place (weight_cache.h:310-353).  With S of them the list
+            // ends as its first n_old - S positions ("base"); step k moves the entry that sits in tail slot S-1-k at
+            // that time to where the k-th surplus index sits at that time.  Only the tail (S entries of the list, fetched
+            // up front) has to be looked at: a surplus index that starts below the tail stays where it is until its own
+            // step, so the lane that owns its position asks what step k moves ("land[k]"), and if that is another
+            // surplus index (one that started in the tail and is taken out later), what that one's step moves, and
+            // so on.  Inside the tail the moves depend on each other through the surplus indices that START there
+            // (few: about S^2 / n_old): their slot at their own step is resolved first, one lane each, in rounds (a
+            // lane whose chase runs into one that is not resolved yet tries again; the smallest always gets through);
+            // then every entry of the tail follows the moves until a step takes it below the tail.  All of it is this
+            // wave's work: the others keep streaming.  Used when S <= min(1024, I/4), at most 64 surplus indices start
+            // in the tail and the list was fetched far enough up front; else the whole block works it out behind the
+            // barrier (below), or the per-index plan does.
+            const int S = nr_w - na_w, base = n_old - S;   // uniform
+            const int smax_w = (I >> 2) < TPB ? (I >> 2) : TPB;
+            const int sm8 = (smax_w + 7) & ~7;
+            constexpr int kMark = 0x8000, kNone = 0xffff, kOut = 0xfffe, kPop = 0xfffd, kUnres = 0xfffc;
+            // (LDS behind the list of added indices: the fetched list, then five arrays of smax entries: 6.5 bytes per index at most)
+            uint16_t *const loc = scan_idx + ((scan_cap + 7) & ~7);   // k -> tail slot the k-th surplus index starts in
+            uint16_t *const tailv = loc + sm8;                        // tail slot -> entry after the paired replacements, or kMark | k
+            uint16_t *const jres = tailv + sm8;                       // k (starting in the tail) -> its slot at step k
+            uint16_t *const land = jres + sm8;                        // k -> what step k moves below the tail
+            uint16_t *const jlist = land + sm8;                       // the surplus indices that start in the tail
+            bool ok = S <= smax_w && base >= 0 && n_old <= scan_cap && I >= 256;
+            if (ok) {
+#pragma unroll 1
+                for (int c = lane; c < S; c += kWave) loc[c] = (uint16_t)kNone;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+                int in_tail = 0, paired_tail = 0;
+#pragma unroll 1
+                for (int c = 0; c < S; c += kWave) {
+                    const int j = c + lane;
+                    const bool in = j < S;
+                    const int e = (int)scan_idx[base + (in ? j : 0)];
+                    const int word = (e >> 5) & (kSparseMaxW32 - 1), bit = e & 31;
+                    const uint32_t remw = sh.oldbits[word] & ~sh.newbits[word];
+                    const bool rem = in && ((remw >> bit) & 1u);
+                    const int rank = (int)sh.pr[word] + __popc(remw & ((1u << bit) - 1u));
+                    const bool paired = rem && rank < na_w, extra = rem && rank >= na_w;
+                    const int k = extra ? rank - na_w : 0;
+                    int v = e;
+                    if (paired) v = (int)added_list[rank];
+                    if (extra) v = kMark | k;
+                    if (in) tailv[j] = (uint16_t)v;
+                    const uint64_t mx = __builtin_amdgcn_ballot_w64(extra);
+                    if (extra) {
+                        const int jj = in_tail + __popcll(mx & ((1ull << lane) - 1ull));
+                        loc[k] = (uint16_t)j;
+                        jres[k] = (uint16_t)kUnres;
+                        if (jj < kWave) jlist[jj] = (uint16_t)k;
+                    }
+                    in_tail += __popcll(mx);
+                    paired_tail += __popcll(__builtin_amdgcn_ballot_w64(paired));
+                }
+                ok = in_tail <= kWave;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+                if (ok) {
+                    // ---- the surplus indices that start in the tail: where each sits at its own step
+                    const int kk = lane < in_tail ? (int)jlist[lane] : -1;
+                    bool open = kk >= 0;
+#pragma unroll 1
+                    for (int round = 0; round <= kWave && __builtin_amdgcn_ballot_w64(open) != 0; ++round) {
+                        bool done = false;
+                        int res = 0;
+                        if (open) {
+                            int pos = loc[kk];
+#pragma unroll 1
+                            for (int it = 0; it <= S; ++it) {
+                                const int i = S - 1 - pos;   // the step that takes the entry of that slot
+                                if (i > kk) { res = pos; done = true; break; }    // still there at its own step
+                                if (i == kk) { res = kPop; done = true; break; }  // the last entry at its own step: nothing moves
+                                const int li = loc[i], ji = jres[i];
+                                if (li == kNone || ji == kOut) {   // step i moves it below the tail
+                                    land[i] = (uint16_t)(kMark | kk);
+                                    res = kOut; done = true; break;
+                                }
+                                if (ji == kUnres) break;   // next round
+                                pos = ji;                  // step i moved it to that slot
+                            }
+                        }
+                        if (open && done) jres[kk] = (uint16_t)res;
+                        open = open && !done;
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+                        __builtin_amdgcn_wave_barrier();
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+                    }
+                    // ---- every other entry of the tail follows the moves until one takes it below the tail
+#pragma unroll 1
+                    for (int c = lane; c < S; c += kWave) {
+                        const int v = tailv[c];
+                        if (v & kMark) continue;
+                        int k = S - 1 - c;
+#pragma unroll 1
+                        for (int it = 0; it <= S; ++it) {
+                            const int lk = loc[k], jk = jres[k];
+                            if (lk == kNone || jk == kOut) { land[k] = (uint16_t)v; break; }
+                            k = S - 1 - (jk < S ? jk : 0);
+                        }
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+                    if (lane < Q && my_p < base) {
+                        const int e = ep ? i_old1 : i_old0;
+                        const int word = (e >> 5) & (kSparseMaxW32 - 1), bit = e & 31;
+                        const uint32_t remw = sh.oldbits[word] & ~sh.newbits[word];
+                        int newidx = e;
+                        if ((remw >> bit) & 1u) {
+                            const int rank = (int)sh.pr[word] + __popc(remw & ((1u << bit) - 1u));
+                            if (rank < na_w) {
+                                newidx = (int)added_list[rank];
+                            } else {
+                                int v = land[(rank - na_w) < S ? rank - na_w : 0];
+#pragma unroll 1
+                                for (int it = 0; it < S && (v & kMark); ++it) v = land[(v & (kMark - 1)) < S ? (v & (kMark - 1)) : 0];
+                                newidx = v < I ? v : e;   // (consistent bookkeeping always ends at an entry of the list)
+                            }
+                        }
+                        s = newidx != e ? (newidx | kSrcPool) : my_p;
+                        indices2[(size_t)(ep ^ 1) * I + my_p] = newidx;
+                    }
+                    if (lane == 0) {
+                        sh.n = base;
+                        // rewritten positions: the pairs' below the tail, and the places of the surplus indices below it
+                        sh.nchg = na_w - paired_tail + (S - in_tail);
+                    }
+                }
+            }
+            if (lane == 0) sh.fast_ok = ok ? 1 : 0;
         }
         sh.src[lane] = s;
         if (lane == 0) { sh.na = na_w; sh.nr = nr_w; sh.found = 0; sh.paired_tail = 0; }
@@ -816,12 +951,14 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     // step came earlier (then it has travelled on with that step's move, possibly again).  So the places follow
     // from the start positions by chasing through tail slots, which only surplus indices that START in the tail
     // need (few: about S^2 / n_old); they are resolved one after the other, then every surviving tail entry finds
-    // its final place on its own.  Used when S <= min(1024, I/4) and the list was fetched far enough up front;
-    // else the per-index plan.
+    // its final place on its own.  This is the whole block's form of it, for the case that more than 64 surplus
+    // indices start in the tail (the planning wave has done the others on its own, `fast`).  Used when
+    // S <= min(1024, I/4) and the list was fetched far enough up front; else the per-index plan.
     const int surplus = nr - na, tail_base = n_old - surplus;
+    const bool fast = surplus > 0 && sh.fast_ok != 0;
     const int smax = (I >> 2) < TPB ? (I >> 2) : TPB;
     // (LDS behind the list of added indices: the fetched list, then five arrays of smax entries: 6.5 bytes per index at most)
-    bool replay = surplus > 0 && surplus <= smax && tail_base >= 0 && n_old <= scan_cap && I >= 256;
+    bool replay = surplus > 0 && !fast && surplus <= smax && tail_base >= 0 && n_old <= scan_cap && I >= 256;
     constexpr uint16_t kGone = 0xffffu;   // hole[]: removed as the last entry, nothing moves; tailv[]: a surplus index
     uint16_t *const hole = scan_idx + ((scan_cap + 7) & ~7);   // start position of the k-th surplus index, then its place at step k
     uint16_t *const tailv = hole + ((smax + 7) & ~7);          // entry of tail slot j after the paired replacements
@@ -950,8 +1087,8 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
             lds_barrier();
         }
     }
-    if (surplus <= 0 || replay) {
-        const int n_changed = replay ? sh.nchg : na;
+    if (surplus <= 0 || fast || replay) {
+        const int n_changed = fast || replay ? sh.nchg : na;
         n = sh.n;
         if (changed) {
             // the remembered mask: 8-byte words dealt to the blocks round-robin (the reference keeps the old

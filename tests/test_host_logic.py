@@ -184,3 +184,118 @@ def test_surplus_removal_closed_form():
         m2[drop] = False
         oc.update_active_weights(m2)
         assert closed_form(order, list(drop)) == oc.get_active_indices().tolist(), trial
+
+
+def test_surplus_removal_tail_only_form():
+    """The form of the surplus removals that one wave of the fused update + decode kernel works out from the tail of
+    the list alone (S surplus indices: the last S entries), against the reference's sequential rule
+    (weight_cache.h:248-277 pairs in place, :310-353 each surplus index, ascending, replaced by the then-last entry).
+    `kernel_form` follows the kernel step by step: the tail scan, the rounds that resolve the surplus indices which
+    start in the tail (lanes of a round see the state before the round), the entries that travel until a step takes
+    them below the tail, and the chain a position follows through `land`."""
+    NONE, OUT, POP, UNRES = 0xffff, 0xfffe, 0xfffd, 0xfffc
+    MARK = 0x8000
+
+    def sequential(order, removed_sorted, added_sorted):
+        """weight_cache.h:248-353 restated: pairs in place, then surplus removals by swap-with-last."""
+        lst = list(order); na, nr = len(added_sorted), len(removed_sorted)
+        pos = {e: i for i, e in enumerate(lst)}
+        for i in range(min(na, nr)):
+            p = pos.pop(removed_sorted[i]); lst[p] = added_sorted[i]; pos[added_sorted[i]] = p
+        m = len(lst)
+        for e in removed_sorted[na:]:
+            p, last = pos[e], m - 1
+            if p != last:
+                lst[p] = lst[last]; pos[lst[p]] = p
+            m -= 1
+        return lst[:m]
+
+    def kernel_form(order, removed_sorted, added_sorted, group=64):
+        n, na, nr = len(order), len(added_sorted), len(removed_sorted)
+        S = nr - na; base = n - S
+        rank = {e: i for i, e in enumerate(removed_sorted)}
+        T = [0] * S; loc = [NONE] * S
+        for j in range(S):
+            e = order[base + j]
+            if e in rank:
+                r = rank[e]
+                if r < na: T[j] = added_sorted[r]
+                else: T[j] = MARK | (r - na); loc[r - na] = j
+            else: T[j] = e
+        jlist = [k for k in range(S) if loc[k] != NONE]
+        jres = [UNRES if loc[k] != NONE else NONE for k in range(S)]
+        land = [NONE] * S
+        rounds_max = 0
+        for j0 in range(0, len(jlist), group):
+            grp = jlist[j0:j0 + group]; open_ = set(grp); rounds = 0
+            while open_:
+                rounds += 1
+                writes = []
+                for kk in sorted(open_):
+                    pos = loc[kk]; res = None
+                    for _ in range(S + 1):
+                        i = S - 1 - pos
+                        if i > kk: res = pos; break
+                        if i == kk: res = POP; break
+                        if loc[i] == NONE or jres[i] == OUT: writes.append(('land', i, MARK | kk)); res = OUT; break
+                        if jres[i] == UNRES: break
+                        assert jres[i] < S
+                        pos = jres[i]
+                    if res is not None: writes.append(('jres', kk, res))
+                for w, a, b in writes:      # lanes of a round see the state before the round
+                    if w == 'land': land[a] = b
+                    else: jres[a] = b; open_.discard(a)
+                assert rounds <= group + 1
+            rounds_max = max(rounds_max, rounds)
+        for s in range(S):
+            v = T[s]
+            if v & MARK: continue
+            k = S - 1 - s
+            for _ in range(S + 1):
+                if loc[k] == NONE or jres[k] == OUT: land[k] = v; break
+                assert jres[k] < S, (jres[k], k)
+                k = S - 1 - jres[k]
+            else: raise AssertionError
+        out = []
+        for p in range(base):
+            e = order[p]
+            if e in rank:
+                r = rank[e]
+                if r < na: out.append(added_sorted[r])
+                else:
+                    v = land[r - na]
+                    for _ in range(S + 1):
+                        if not (v & MARK): break
+                        assert v != NONE
+                        v = land[v & (MARK - 1)]
+                    assert not (v & MARK)
+                    out.append(v)
+            else: out.append(e)
+        return out, rounds_max
+
+    rng = np.random.default_rng(0)
+    worst = 0
+    for trial in range(12000):
+        I = int(rng.choice([16, 64, 300]))
+        n = int(rng.integers(2, min(I, 200)))
+        order = rng.permutation(I)[:n].tolist()
+        nr = int(rng.integers(1, n + 1))
+        mode = rng.integers(0, 4)
+        if mode == 0:
+            removed = rng.choice(order, nr, replace=False)
+        elif mode == 1:
+            removed = np.array(order[n - nr:])               # the tail itself
+        elif mode == 2:
+            removed = np.array(sorted(order)[-nr:])          # the largest indices
+        else:                                                # mostly the tail
+            removed = np.array([e if rng.random() < 0.7 else order[int(rng.integers(0, n))] for e in order[n - nr:]])
+        removed = np.sort(np.unique(removed)).tolist()
+        nr = len(removed)
+        free = sorted(set(range(I)) - set(order))
+        na = int(rng.integers(0, min(nr, len(free) + 1)))    # na < nr: at least one surplus removal
+        added = sorted(rng.choice(free, na, replace=False).tolist()) if na else []
+        want = sequential(order, removed, added)
+        got, rounds = kernel_form(order, removed, added, group=int(rng.choice([2, 4, 64])))
+        worst = max(worst, rounds)
+        assert got == want, (trial, order, removed, added)
+    assert worst >= 3      # the cases did reach chains of dependent surplus indices
