@@ -30,7 +30,9 @@ typedef enum st_status {
     ST_ERR_INVALID = -4    /* cache has no valid contents yet: the reference's "Cache is not valid" */
 } st_status;
 
-typedef enum st_dtype { ST_F32 = 0, ST_F16 = 1, ST_BF16 = 2 } st_dtype;
+/* ST_F64: st_mlp_forward only (the reference's operator is dtype-generic, sparse_mlp_op.cpp:151-161, and its CUDA
+ * kernels are instantiated for double, sparse_mlp_cuda.cu:90-151); caches and the predictor take the first three. */
+typedef enum st_dtype { ST_F32 = 0, ST_F16 = 1, ST_BF16 = 2, ST_F64 = 3 } st_dtype;
 
 typedef enum st_act {
     ST_ACT_RELU = 0,      /* what sparse_mlp_op.cpp:157,183 computes */
@@ -81,8 +83,11 @@ const char *st_last_error(void);
  * runs the MFMA GEMM kernels (then only columns [0,n) of `combined` carry results; when its rows are 16-byte
  * aligned and have room, the kernels keep their intermediate there and also zero the columns from n up to the next
  * multiple of 128).
+ * ST_F64 (any B, H % 2 == 0): three plain kernels with every sum in double and in a fixed order, eight rows of x
+ * per pass; the workspace must then hold st_mlp_f64_workspace_bytes(B,H,n) bytes.
  * ------------------------------------------------------------------------ */
 int64_t st_mlp_workspace_bytes(int64_t B, int64_t H, int64_t n);
+int64_t st_mlp_f64_workspace_bytes(int64_t B, int64_t H, int64_t n);
 int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *gate_rows, const void *up_rows,
                    const void *down_rows, int64_t n, const int32_t *n_dev, int64_t n_hint, void *out, void *combined,
                    int64_t ldc, void *workspace, int64_t workspace_bytes, int act, int dtype, int has_gate,

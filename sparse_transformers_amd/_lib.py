@@ -17,7 +17,7 @@ ST_ERR_NO_ACTIVE = -2
 ST_ERR_HIP = -3
 ST_ERR_INVALID = -4
 
-ST_F32, ST_F16, ST_BF16 = 0, 1, 2
+ST_F32, ST_F16, ST_BF16, ST_F64 = 0, 1, 2, 3
 ACT_CODES = {"relu": 0, "silu": 1, "gelu_pytorch_tanh": 2, "sigmoid": 3, "identity": 4}
 
 STATE_N_ACTIVE, STATE_N_CHANGED, STATE_STATUS, STATE_VALID = 0, 1, 2, 3
@@ -38,6 +38,7 @@ SIGNATURES = {
     "st_version": (_ci, []),
     "st_last_error": (C.c_char_p, []),
     "st_mlp_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "st_mlp_f64_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "st_mlp_forward": (_ci, [_vp, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _ci, _ci, _ci,
                              _vp]),
     "st_mlp_static_scratch_bytes": (_i64, []),

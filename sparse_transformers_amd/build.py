@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libsparse_mlp_amd.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 SOURCES = ["capi.hip", "mlp_decode.hip", "mlp_batch.hip", "mlp_prefill.hip", "predictor.hip", "mask_select.hip",
-           "cache.hip"]
+           "mlp_f64.hip", "cache.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

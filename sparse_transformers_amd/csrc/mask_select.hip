@@ -15,8 +15,6 @@
 // change the result.
 #include "st_common.h"
 
-#include <atomic>
-
 namespace st {
 
 constexpr int kSelThreads = 1024;
@@ -446,11 +444,9 @@ extern "C" int st_mask_select(const float *scores, int64_t B, int64_t I, int met
         rowmask = static_cast<uint8_t *>(workspace) + 16;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    static std::atomic<bool> attr_set{false};   // (setting the attribute twice from two threads is harmless)
-    if (!attr_set.load(std::memory_order_acquire)) {
-        ST_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(mask_select_kernel<0>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kSelMaxLdsKeys * 4));
-        attr_set.store(true, std::memory_order_release);
+    {
+        const int rc = allow_dynamic_lds(reinterpret_cast<const void *>(mask_select_kernel<0>), kSelMaxLdsKeys * 4);
+        if (rc != ST_OK) return rc;
     }
     ProfScope ps(ST_K_MASK_SELECT, s);
     const dim3 grid((unsigned)B), block(kSelThreads);

@@ -464,15 +464,16 @@ int launch_mlp_reduce(int dtype, const float *partials, int G, int NB, int bcoun
 // Argument checks shared by the MLP entry points (everything but the workspace size).
 static int check_mlp_args(const char *who, const void *x, int64_t B, int64_t H, const void *gate_rows,
                           const void *up_rows, const void *down_rows, int64_t n, const void *out, const void *combined,
-                          int64_t ldc, const void *workspace, int act, int dtype, int has_gate)
+                          int64_t ldc, const void *workspace, int act, int dtype, int has_gate, bool f64_ok = false)
 {
     ST_REQUIRE(x && up_rows && down_rows && out && workspace, "%s: null pointer", who);
     ST_REQUIRE(!has_gate || gate_rows, "%s: has_gate set but gate_rows is null", who);
     ST_REQUIRE(B >= 1 && B <= 4096, "%s: B=%lld out of range [1,4096]", who, (long long)B);
     ST_REQUIRE(n >= 0 && n <= (1 << 24), "%s: n=%lld out of range", who, (long long)n);
     ST_REQUIRE(act >= ST_ACT_RELU && act <= ST_ACT_IDENTITY, "%s: unknown activation %d", who, act);
-    ST_REQUIRE(dtype >= ST_F32 && dtype <= ST_BF16, "%s: unknown dtype %d", who, dtype);
-    const int esz = dtype == ST_F32 ? 4 : 2;
+    ST_REQUIRE((dtype >= ST_F32 && dtype <= ST_BF16) || (f64_ok && dtype == ST_F64), "%s: unknown dtype %d%s", who, dtype,
+               dtype == ST_F64 ? " (double precision: st_mlp_forward only)" : "");
+    const int esz = dtype == ST_F64 ? 8 : dtype == ST_F32 ? 4 : 2;
     ST_REQUIRE(H >= 1 && (H * esz) % 16 == 0, "%s: H=%lld rows are not 16-byte multiples", who, (long long)H);
     ST_REQUIRE(!combined || ldc >= (has_gate ? 2 * n : n), "%s: ldc=%lld too small for n=%lld", who, (long long)ldc,
                (long long)n);
@@ -577,8 +578,15 @@ extern "C" int st_mlp_forward(const void *x, int64_t B, int64_t H, const void *g
 {
     using namespace st;
     const int rc = check_mlp_args("st_mlp_forward", x, B, H, gate_rows, up_rows, down_rows, n, out, combined, ldc,
-                                  workspace, act, dtype, has_gate);
+                                  workspace, act, dtype, has_gate, true);
     if (rc != ST_OK) return rc;
+    if (dtype == ST_F64) {
+        ST_REQUIRE(workspace_bytes >= f64_workspace_bytes(B, H, n),
+                   "st_mlp_forward: workspace too small for double precision (%lld < %lld, st_mlp_f64_workspace_bytes)",
+                   (long long)workspace_bytes, (long long)f64_workspace_bytes(B, H, n));
+        return launch_f64(x, (int)B, (int)H, gate_rows, up_rows, down_rows, (int)n, n_dev, out, combined, (long)ldc,
+                          workspace, act, has_gate ? 1 : 0, static_cast<hipStream_t>(stream));
+    }
     ST_REQUIRE(workspace_bytes >= st_mlp_workspace_bytes(B, H, n), "st_mlp_forward: workspace too small (%lld < %lld)",
                (long long)workspace_bytes, (long long)st_mlp_workspace_bytes(B, H, n));
 

@@ -270,6 +270,11 @@ int launch_batch(int dtype, const void *x, int B, int H, const void *gate, const
                  const int *n_dev, void *out, void *comb, long ldc, void *workspace, int act, int has_gate,
                  hipStream_t stream);
 
+// Double precision forward (plain kernels, for checking a model in fp64).
+int64_t f64_workspace_bytes(int64_t B, int64_t H, int64_t n);
+int launch_f64(const void *x, int B, int H, const void *gate, const void *up, const void *down, int n, const int *n_dev,
+               void *out, void *comb, long ldc, void *workspace, int act, int has_gate, hipStream_t stream);
+
 // Timing slot for one kernel launch; inert unless profiling is enabled.  ST_LAUNCH hands the slot's
 // events to hipExtLaunchKernelGGL, which stamps them at the kernel's own begin and end (so the elapsed
 // time is the kernel's execution time, without dispatch latency).

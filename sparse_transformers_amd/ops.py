@@ -23,14 +23,15 @@ import torch
 
 from . import _lib
 
-_DTYPES = {torch.float32: _lib.ST_F32, torch.float16: _lib.ST_F16, torch.bfloat16: _lib.ST_BF16}
+_DTYPES = {torch.float32: _lib.ST_F32, torch.float16: _lib.ST_F16, torch.bfloat16: _lib.ST_BF16,
+           torch.float64: _lib.ST_F64}   # (double precision: the stand-alone forward only)
 
 
 def dtype_code(t: torch.Tensor) -> int:
     try:
         return _DTYPES[t.dtype]
     except KeyError:
-        raise TypeError(f"unsupported dtype {t.dtype}; expected float32, float16 or bfloat16") from None
+        raise TypeError(f"unsupported dtype {t.dtype}; expected float32, float16, bfloat16 or float64") from None
 
 
 def require_gpu(*tensors: torch.Tensor) -> torch.device:
@@ -56,11 +57,13 @@ def current_stream_ptr(device: torch.device) -> int:
 _workspaces: dict = {}
 
 
-def mlp_workspace_bytes(B: int, H: int, n: int) -> int:
+def mlp_workspace_bytes(B: int, H: int, n: int, dtype: Optional[torch.dtype] = None) -> int:
+    if dtype == torch.float64:
+        return int(_lib.lib().st_mlp_f64_workspace_bytes(B, H, n))
     return int(_lib.lib().st_mlp_workspace_bytes(B, H, n))
 
 
-def mlp_workspace(device: torch.device, B: int, H: int, n: int) -> torch.Tensor:
+def mlp_workspace(device: torch.device, B: int, H: int, n: int, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """Scratch for one forward on the current stream of ``device``.
 
     One list of buffers per (device, stream): two streams never share scratch, and a buffer that has been
@@ -68,7 +71,7 @@ def mlp_workspace(device: torch.device, B: int, H: int, n: int) -> torch.Tensor:
     baked in, so growing must not free it.  Callers that replay graphs or know their largest batch should
     own a buffer instead (``torch.empty(mlp_workspace_bytes(B, H, I), dtype=torch.uint8)``) and pass it as
     ``workspace=``."""
-    need = mlp_workspace_bytes(B, H, n)
+    need = mlp_workspace_bytes(B, H, n, dtype)
     key = (device.index if device.index is not None else torch.cuda.current_device(),
            torch.cuda.current_stream(device).cuda_stream)
     bufs = _workspaces.setdefault(key, [])
@@ -117,7 +120,7 @@ def combined_for_launch(combined: Optional[torch.Tensor], B: int, n: int):
     width ends before the padded one would have its parent's columns zeroed, so such a view goes through a
     contiguous stand-in of its own width (whose stride is too short for the padding, so nothing is written
     outside it)."""
-    if combined is None or B < 32 or combined.dtype == torch.float32:
+    if combined is None or B < 32 or combined.dtype in (torch.float32, torch.float64):
         return combined, None
     padded = (int(n) + 127) // 128 * 128
     if combined.stride(0) == combined.size(1) or combined.size(1) >= padded:
@@ -151,8 +154,8 @@ def mlp_forward_rows(x2: torch.Tensor, gate_rows: Optional[torch.Tensor], up_row
     check_mlp_args(x2, out, combined, up_rows.dtype, dev, H, (2 if has_gate else 1) * n)
     if n_dev is not None and (n_dev.dtype != torch.int32 or n_dev.numel() < 1):
         raise TypeError("n_dev must be an int32 GPU tensor")
-    need = mlp_workspace_bytes(B, H, n)
-    ws = mlp_workspace(dev, B, H, n) if workspace is None else _check_workspace(workspace, dev, need)
+    need = mlp_workspace_bytes(B, H, n, x2.dtype)
+    ws = mlp_workspace(dev, B, H, n, x2.dtype) if workspace is None else _check_workspace(workspace, dev, need)
     if act not in _lib.ACT_CODES:
         raise ValueError(f"unknown activation {act!r}; expected one of {sorted(_lib.ACT_CODES)}")
     combined, copy_back = combined_for_launch(combined, B, n)

@@ -102,6 +102,9 @@ class WeightCache:
             raise ValueError(f"gate must be [{I},{H}], got {tuple(gate_weight.shape)}")
         if down_weight.dtype != self.dtype or (self.has_gate and gate_weight.dtype != self.dtype):
             raise TypeError("gate, up and down weights must share one dtype")
+        if self.dtype == torch.float64:
+            raise TypeError("the weight cache holds float32, float16 or bfloat16 rows (float64 is served by "
+                            "sparse_mlp_forward on caller-owned rows only)")
         code = dtype_code(up_weight)
         L = _lib.lib()
         if I > L.st_cache_max_intermediate():

@@ -69,7 +69,9 @@ def round_to(a: np.ndarray, dtype: str) -> np.ndarray:
 
 # tolerances of the north star: fp32 1e-5 relative; fp16/bf16 2e-2 absolute / 1e-2 relative
 TOL = {"float32": dict(rtol=1e-5, atol_rel=1e-5), "float16": dict(rtol=1e-2, atol=2e-2),
-       "bfloat16": dict(rtol=1e-2, atol=2e-2)}
+       "bfloat16": dict(rtol=1e-2, atol=2e-2),
+       # double precision against a float64 library evaluation: summation order only
+       "float64": dict(rtol=1e-12, atol_rel=1e-12)}
 
 
 def assert_close(got: np.ndarray, want: np.ndarray, dtype: str, what: str = ""):

@@ -69,6 +69,38 @@ def test_forward_vs_oracle_config_shapes(name, B, H, n, dtype, act, has_gate):
     assert_close(cb.float().cpu().numpy(), wantc, dtype, name + " combined")
 
 
+@pytest.mark.parametrize("act", ["silu", "relu", "gelu_pytorch_tanh", "sigmoid"])
+@pytest.mark.parametrize("has_gate", [True, False])
+def test_forward_float64(act, has_gate):
+    """Double precision (the reference's operator is dtype-generic, sparse_mlp_op.cpp:151-161): against numpy's
+    float64 matrix products (1e-12 of the output's scale: only the order of the sums differs) and, on inputs that
+    float32 holds exactly, against the oracle (whose sums are in double and whose outputs are rounded to float32)."""
+    acts = {"silu": lambda v: v / (1 + np.exp(-v)), "relu": lambda v: np.maximum(v, 0), "sigmoid": lambda v: 1 / (1 + np.exp(-v)),
+            "gelu_pytorch_tanh": lambda v: 0.5 * v * (1 + np.tanh(np.sqrt(2 / np.pi) * (v + 0.044715 * v ** 3)))}
+    for seed, (B, H, n) in enumerate([(1, 64, 5), (1, 3072, 700), (3, 256, 300), (8, 130, 77), (9, 1024, 129), (19, 512, 1000)]):
+        x, cw, dn = _case(seed, B, H, n, "float32", has_gate, std=0.05)      # float32 values, held in double
+        out, db, cb = _run(x.double(), cw.double(), dn.double(), act, has_gate)
+        assert out.dtype == torch.float64 and tuple(cb.shape) == (B, cw.shape[0])
+        xd, cwd, dnd = x.double().numpy(), cw.double().numpy(), dn.double().numpy()
+        up = xd @ cwd[n:].T if has_gate else xd @ cwd.T
+        h = acts[act](xd @ cwd[:n].T) * up if has_gate else acts[act](up)
+        assert_close(out.cpu().numpy(), h @ dnd, "float64", f"float64 out B={B} H={H} n={n}")
+        assert_close(cb.cpu().numpy()[:, :n], h, "float64", "float64 combined")
+        if has_gate:
+            assert_close(cb.cpu().numpy()[:, n:], up, "float64", "float64 combined, up half")
+        want, wantc = oracle.mlp_forward(x.numpy(), cw.numpy(), dn.numpy().T, act, has_gate)
+        assert_close(out.cpu().numpy(), want, "float32", "float64 against the oracle")
+        assert_close(cb.cpu().numpy(), wantc, "float32", "float64 combined against the oracle")
+    # an odd hidden size has rows that are not 16-byte multiples
+    x, cw, dn = _case(3, 1, 33, 8, "float32", True)
+    with pytest.raises(ValueError, match="16-byte"):
+        _run(x.double(), cw.double(), dn.double(), "silu", True)
+    # caches and the predictor do not take double
+    with pytest.raises(TypeError, match="float64"):
+        st.WeightCache(torch.ones(8, dtype=torch.bool, device=DEV), 16, torch.zeros(8, 16, dtype=torch.float64, device=DEV),
+                       torch.zeros(8, 16, dtype=torch.float64, device=DEV), torch.zeros(16, 8, dtype=torch.float64, device=DEV))
+
+
 def test_matches_reference_operator_vectors(golden_mlp):
     """Outputs of the reference's compiled ReLU operator (tests/golden/mlp_forward.json)."""
     for case in golden_mlp:
