@@ -440,7 +440,7 @@ def decode_measure(args, wl, torch, st, _lib, syn, layers, B, K, W, P, count_wob
     stack.step_staged(x_in[W + K - 1], x_pred[W + K - 1], masks_of(W + K - 1), replay=False)   # (the masks the caches hold)
     host_ms = (time.perf_counter() - h0) * 1e3
     torch.cuda.synchronize()
-    hold_cycles = int(min(2.0 * host_ms + 0.3, 20.0) * cycles_per_ms)
+    hold_cycles = int(min(3.0 * host_ms + 0.5, 20.0) * cycles_per_ms)
 
     t_lo = W + K - 1 - P
     seen_changed, seen_active = [], []
