@@ -139,6 +139,33 @@ def test_device_count_and_hint_paths():
     assert not out.any()                                       # empty active set -> zeros
 
 
+def test_float64_device_count_and_empty_set():
+    """Double precision with the count on the device: rows beyond it are ignored, the result carries the same bits
+    as with the host's count (fixed summation order), and an empty set gives zeros."""
+    I, H, n = 700, 256, 333
+    g = torch.Generator().manual_seed(4)
+    gate = torch.randn(I, H, generator=g, dtype=torch.float64).to(DEV)
+    up = torch.randn(I, H, generator=g, dtype=torch.float64).to(DEV)
+    dn = torch.randn(I, H, generator=g, dtype=torch.float64).to(DEV)
+    x = torch.randn(3, H, generator=g, dtype=torch.float64).to(DEV)
+    ref = torch.empty(3, H, dtype=torch.float64, device=DEV)
+    mlp_forward_rows(x, gate, up, dn, n, None, ref, None, "silu", True)
+    gu = x @ gate[:n].T
+    want = ((gu / (1 + torch.exp(-gu))) * (x @ up[:n].T)) @ dn[:n]
+    assert_close(ref.cpu().numpy(), want.cpu().numpy(), "float64", "float64, host count")
+    n_dev = torch.tensor([n], dtype=torch.int32, device=DEV)
+    out = torch.full((3, H), float("nan"), dtype=torch.float64, device=DEV)
+    comb = torch.zeros(3, 2 * I, dtype=torch.float64, device=DEV)
+    mlp_forward_rows(x, gate, up, dn, I, n_dev, out, comb, "silu", True)
+    assert_close(out.cpu().numpy(), want.cpu().numpy(), "float64", "float64, device count")
+    n_dev.fill_(0)
+    mlp_forward_rows(x, gate, up, dn, I, n_dev, out, None, "silu", True)
+    assert not out.any()
+    out.fill_(1.0)
+    mlp_forward_rows(x, gate, up, dn, 0, None, out, None, "silu", True)
+    assert not out.any()
+
+
 def test_run_to_run_determinism_and_linearity_full_size():
     x, cw, dn = _case(5, 1, 3072, 2867, "float16", True)
     a, _, _ = _run(x, cw, dn, "silu", True)
