@@ -808,7 +808,7 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
             // (few: about S^2 / n_old): their slot at their own step is resolved first, one lane each, in rounds (a
             // lane whose chase runs into one that is not resolved yet tries again; the smallest always gets through);
             // then every entry of the tail follows the moves until a step takes it below the tail.  All of it is this
-            // wave's work: the others keep streaming.  Used when S <= min(1024, I/4), at most 64 surplus indices start
+            // wave's work: the others keep streaming.  Used when S <= min(256, I/4), at most 64 surplus indices start
             // in the tail and the list was fetched far enough up front; else the whole block works it out behind the
             // barrier (below), or the per-index plan does.
             const int S = nr_w - na_w, base = n_old - S;   // uniform
@@ -821,7 +821,8 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
             uint16_t *const jres = tailv + sm8;                       // k (starting in the tail) -> its slot at step k
             uint16_t *const land = jres + sm8;                        // k -> what step k moves below the tail
             uint16_t *const jlist = land + sm8;                       // the surplus indices that start in the tail
-            bool ok = S <= smax_w && base >= 0 && n_old <= scan_cap && I >= 256;
+            // (S <= 256: one wave walks the tail 64 slots at a time, and beyond four passes the whole block is faster)
+            bool ok = S <= smax_w && S <= 4 * kWave && base >= 0 && n_old <= scan_cap && I >= 256;
             if (ok) {
 #pragma unroll 1
                 for (int c = lane; c < S; c += kWave) loc[c] = (uint16_t)kNone;
