@@ -48,3 +48,18 @@ def test_prefill_line():
     r = d["roofline"]
     assert d["dtype"] == "bf16" and r["bound"] == "mfma" and r["unit"] == "TFLOP/s" and r["peak"] == 2500.0
     assert 0 < r["frac"] < 1 and d["value"] > 0 and d["config"]["rows"] == 128
+
+
+def test_default_line_carries_the_other_workloads():
+    """The line a bare `bench.py --steps K --warmup W` prints: the other workloads, a wobbling count and predictor-driven
+    masks ride along as short passes, and the measured traffic belongs to the sources in the tree."""
+    d = _run("--steps", "6", "--warmup", "2", "--no-cpu-baseline")
+    ow = d["other_workloads"]
+    for key in ("llama1b_layer_fp32_b1", "llama3b_stack_fp16_b4", "llama3b_stack_fp16_b16", "mistral7b_stack_bf16_b1",
+                "mistral7b_stack_bf16_b8", "relullama7b_stack_fp16_b1", "relullama7b_ungated_fp16_b1",
+                "llama3b_stack_fp16_b1_count_wobble_0.03", "llama3b_stack_fp16_b1_mask_source_predictor"):
+        assert ow[key]["tok_s"] > 0 and 0 < ow[key]["frac"] < 1, key
+    assert d["config"]["mask_source"] == "trace" and d["config"]["count_wobble"] == 0.0
+    assert d["roofline"]["traffic"] is not None, d["roofline"]["traffic_source"]
+    assert 0.9 < d["roofline"]["traffic"] / d["roofline"]["bytes_per_launch"] < 1.3
+    assert d["prefill_512"]["roofline"]["bound"] == "mfma"

@@ -119,6 +119,20 @@ def test_bench_refuses_more_than_one_gpu():
     assert p.returncode != 0 and "ONE GPU" in p.stderr
 
 
+def test_traffic_table_was_measured_on_these_sources():
+    """profiles/hbm_traffic.md: the rows bench.py reads carry the hash of the HIP sources they were measured on; a
+    change to the sources without a new measurement would silently drop `roofline.traffic` from the bench line."""
+    import importlib.util
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_for_hash", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    for wl in ("llama3b_stack_fp16", "mistral7b_stack_bf16", "relullama7b_stack_fp16"):
+        nbytes, source = bench.measured_traffic(wl, "cache_update_decode", 1)
+        assert nbytes is not None and nbytes > 0, (wl, source)
+
+
 def test_surplus_removal_closed_form():
     """The closed form the fused update + decode kernel uses when removals outnumber additions, against the
     reference's sequential rule (weight_cache.h:310-353: each surplus index, ascending, is replaced by the then-last
