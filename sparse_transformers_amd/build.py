@@ -28,6 +28,10 @@ FLAGS = [
     # the pass that aggregates uniform atomics per wave reads their result back at once; the cache kernels
     # issue one atomic per block and look at its result much later on purpose
     "-mllvm", "-amdgpu-atomic-optimizer-strategy=None",
+    # the first kernel arguments arrive in scalar registers with the wave instead of through a load at its start
+    # (one memory round trip less in front of every kernel of a chain of short dependent kernels; structs passed by
+    # value end the preloaded part, so the cache kernels take theirs last)
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall",
     "-Wno-unused-command-line-argument",
 ]

@@ -455,11 +455,11 @@ __device__ __forceinline__ void plan_finish(const PlanView &pv, int32_t *__restr
 
 // update = plan + this block's share of the row copies
 template <bool VEC, int TPB>
-__global__ __launch_bounds__(TPB) void cache_update_kernel(CopyPlan cp, const uint8_t *__restrict__ new_mask,
+__global__ __launch_bounds__(TPB) void cache_update_kernel(const uint8_t *__restrict__ new_mask,
                                                                     uint8_t *__restrict__ cur_mask2,
                                                                     int32_t *__restrict__ indices2,
                                                                     int32_t *__restrict__ state, int I, int gs_log2,
-                                                                    int idx_cap)
+                                                                    int idx_cap, CopyPlan cp)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ PlanShared ps;
@@ -559,9 +559,9 @@ __device__ __forceinline__ uint32_t pack_bits8(uint64_t ones)
 
 template <typename T, int RB, int TPB, int NB = 1, int NW = 1, int SPECN = RB / 2>
 __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
-    FusedRows fr, const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
-    int32_t *__restrict__ state, int I, const T *__restrict__ x, int B, int H, T *__restrict__ combined, long ldc,
-    float *__restrict__ partials, int act, int gs_log2, int plan_bytes, int n_hint)
+    const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
+    int32_t *__restrict__ state, int I, int G, const T *__restrict__ x, int H, int B, int n_hint, int gs_log2,
+    T *__restrict__ combined, long ldc, float *__restrict__ partials, int act, int plan_bytes, FusedRows fr)
 {
     constexpr int VEC = Elem<T>::kVec;
     // Slots of the first batch that are requested ahead of the plan, on the caller's guess of the count and from the
@@ -578,7 +578,9 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     __shared__ PlanShared plan_shared;
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const int G = gridDim.x, blk = blockIdx.x;
+    // (what the first loads need comes first in the argument list, the number of blocks included: those arguments are
+    // in scalar registers when the wave starts, anything else -- the launch dimensions too -- arrives by a load)
+    const int blk = blockIdx.x;
     const int chunks = H / VEC;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
     const int GS = 1 << gs_log2, ngrp = TPB >> gs_log2, wpg = GS >> 6;
@@ -1274,7 +1276,7 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     // the block that arrived last resets the arrivals and sets the epoch (the atomic's result is first looked at here)
     if (arriver) {
         asm volatile("" : "+v"(arrival));
-        if ((arrival & 0xffffu) == gridDim.x - 1)
+        if ((arrival & 0xffffu) == (uint32_t)G - 1u)
             atomicExch(reinterpret_cast<uint32_t *>(&state[ST_STATE_TICKET]), (uint32_t)next_epoch << 16);
     }
     ST_TL(7);
@@ -1323,10 +1325,10 @@ __device__ __forceinline__ int big_select(const uint32_t *bits, const uint32_t *
     return lo * 32 + pos;
 }
 
-__global__ __launch_bounds__(kBigThreads) void cache_update_big_kernel(FusedRows fr, const uint8_t *__restrict__ new_mask,
+__global__ __launch_bounds__(kBigThreads) void cache_update_big_kernel(const uint8_t *__restrict__ new_mask,
                                                                       uint8_t *__restrict__ cur_mask2,
                                                                       int32_t *__restrict__ indices2,
-                                                                      int32_t *__restrict__ state, int I)
+                                                                      int32_t *__restrict__ state, int I, FusedRows fr)
 {
     constexpr int TPB = kBigThreads;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -1649,8 +1651,8 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
             big_attr.store(true, std::memory_order_release);
         }
         ProfScope ps(ST_K_CACHE_UPDATE, s);
-        ST_LAUNCH(ps, cache_update_big_kernel, dim3(device_cu_count()), dim3(kBigThreads), lds_big, s, fr, mask,
-                  c->b.cur_mask, c->b.indices, c->b.state, I);
+        ST_LAUNCH(ps, cache_update_big_kernel, dim3(device_cu_count()), dim3(kBigThreads), lds_big, s, mask,
+                  c->b.cur_mask, c->b.indices, c->b.state, I, fr);
         ST_HIP(hipGetLastError());
         return ST_OK;
     }
@@ -1696,8 +1698,8 @@ extern "C" int st_cache_update_async(st_cache *c, const uint8_t *mask, void *str
         auto launch = [&](auto kern) -> int {
             const int arc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), 160 * 1024 - 256);
             if (arc != ST_OK) return arc;
-            ST_LAUNCH(ps, kern, dim3(grid), dim3(tpb), lds, s, cp, mask, c->b.cur_mask, c->b.indices, c->b.state,
-                               I, gs_log2, idx_cap);
+            ST_LAUNCH(ps, kern, dim3(grid), dim3(tpb), lds, s, mask, c->b.cur_mask, c->b.indices, c->b.state,
+                               I, gs_log2, idx_cap, cp);
             return ST_OK;
         };
         int rc;
@@ -1767,8 +1769,8 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
         auto launch = [&](auto kern, auto *xt, auto *ct) -> int {
             const int arc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), 148 * 1024);
             if (arc != ST_OK) return arc;
-            ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, fr, mask, c->b.cur_mask, c->b.indices, c->b.state, I, xt,
-                      (int)B, H, ct, (long)ldc, partials, act, gs_log2, (int)plan_bytes, hint);
+            ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, mask, c->b.cur_mask, c->b.indices, c->b.state, I, G, xt,
+                      H, (int)B, hint, gs_log2, ct, (long)ldc, partials, act, (int)plan_bytes, fr);
             return ST_OK;
         };
         int rc;

@@ -58,7 +58,7 @@ __device__ __forceinline__ void wave_lds_fence()
 // ---------------------------------------------------------------------------
 template <typename T, int KSW, bool HG, int NT>
 __global__ __launch_bounds__(kBtThreads) void batch_gateup_kernel(
-    const T *__restrict__ x, int B, const T *__restrict__ gate, const T *__restrict__ up, int n_host,
+    const T *__restrict__ x, int B, int G, const T *__restrict__ gate, const T *__restrict__ up, int n_host,
     const int *__restrict__ n_dev, T *__restrict__ hbuf, int ldh, T *__restrict__ combined, long ldc, int act)
 {
     constexpr int H = KSW * 256;
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(kBtThreads) void batch_gateup_kernel(
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), w = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
-    const int G = gridDim.x, blk = blockIdx.x;
+    const int blk = blockIdx.x;  // G: the grid's size, an argument so that it arrives preloaded
 
     const int n = device_count(n_host, n_dev);
     const int R = (n + G - 1) / G;             // rows per block
@@ -230,7 +230,7 @@ constexpr int kBtRing = 4;
 
 template <typename T, bool HG, bool XLDS>
 __global__ __launch_bounds__(kBtThreads) void batch_gateup_anyh_kernel(
-    const T *__restrict__ x, int B, int H, const T *__restrict__ gate, const T *__restrict__ up, int n_host,
+    const T *__restrict__ x, int B, int H, int G, const T *__restrict__ gate, const T *__restrict__ up, int n_host,
     const int *__restrict__ n_dev, T *__restrict__ hbuf, int ldh, T *__restrict__ combined, long ldc, int act)
 {
     const int KSW = H / 256, XP = H + kBtXPad;
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(kBtThreads) void batch_gateup_anyh_kernel(
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), w = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
-    const int G = gridDim.x, blk = blockIdx.x;
+    const int blk = blockIdx.x;  // G: the grid's size, an argument so that it arrives preloaded
 
     const int n = device_count(n_host, n_dev);
     const int R = (n + G - 1) / G;
@@ -529,7 +529,8 @@ static int launch_gateup(const T *x, int B, const T *gate, const T *up, int n, c
         attr_set.store(true, std::memory_order_release);
     }
     ProfScope ps(ST_K_MLP_BATCH_GATEUP, stream);
-    ST_LAUNCH(ps, kern, dim3(device_cu_count()), dim3(kBtThreads), lds, stream, x, B, gate, up, n, n_dev, hbuf,
+    const int G = device_cu_count();
+    ST_LAUNCH(ps, kern, dim3(G), dim3(kBtThreads), lds, stream, x, B, G, gate, up, n, n_dev, hbuf,
                        ldh, comb, ldc, act);
     return ST_OK;
 }
@@ -541,15 +542,16 @@ static int launch_gateup_anyh(const T *x, int B, int H, const T *gate, const T *
     const bool xlds = H <= 4096;
     const size_t lds = (xlds ? (size_t)kBtRows * (H + kBtXPad) * 2 : 0) + (size_t)kBtRedFloats * 4;
     ProfScope ps(ST_K_MLP_BATCH_GATEUP, stream);
+    const int G = device_cu_count();
     if (xlds) {
         auto kern = batch_gateup_anyh_kernel<T, HG, true>;
         const int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), 152 * 1024);
         if (rc != ST_OK) return rc;
-        ST_LAUNCH(ps, kern, dim3(device_cu_count()), dim3(kBtThreads), lds, stream, x, B, H, gate, up, n, n_dev, hbuf,
+        ST_LAUNCH(ps, kern, dim3(G), dim3(kBtThreads), lds, stream, x, B, H, G, gate, up, n, n_dev, hbuf,
                   ldh, comb, ldc, act);
     } else {
         auto kern = batch_gateup_anyh_kernel<T, HG, false>;
-        ST_LAUNCH(ps, kern, dim3(device_cu_count()), dim3(kBtThreads), lds, stream, x, B, H, gate, up, n, n_dev, hbuf,
+        ST_LAUNCH(ps, kern, dim3(G), dim3(kBtThreads), lds, stream, x, B, H, G, gate, up, n, n_dev, hbuf,
                   ldh, comb, ldc, act);
     }
     return ST_OK;

@@ -45,7 +45,7 @@ template <int RB, int CPT> struct RowBatch {
 // measures faster when all rows of a block fit in it).
 template <typename T, int NB, int RB, int CPT, int TPB, bool DB>
 __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
-    const T *__restrict__ x, int B, int H, const T *__restrict__ gate, const T *__restrict__ up,
+    const T *__restrict__ x, int B, int H, int G, const T *__restrict__ gate, const T *__restrict__ up,
     const T *__restrict__ down, int n_host, const int *__restrict__ n_dev, int n_hint, T *__restrict__ combined,
     long ldc, float *__restrict__ partials, int act, int has_gate, int gs_log2)
 {
@@ -55,7 +55,7 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
     __shared__ float hs[TPB / kWave][RB][NB];                 // h of the rows being computed
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const int G = gridDim.x, blk = blockIdx.x;
+    const int blk = blockIdx.x;  // G: the grid's size, passed as an argument so that it arrives preloaded
     // Active count: requested first, consumed only after the first two batches
     // of weight loads have been issued.  Rows are dealt to blocks round-robin,
     // so which rows a block owns does not depend on the count, and rows below
@@ -339,7 +339,7 @@ static int launch_inst(const MlpLaunch &a, int b0, int bcount)
     T *comb = a.combined ? static_cast<T *>(a.combined) + (size_t)b0 * a.ldc : nullptr;
     {
         ProfScope ps(ST_K_MLP_DECODE, a.stream);
-        ST_LAUNCH(ps, kern, dim3(a.G), dim3(TPB), lds, a.stream, x, bcount, a.H,
+        ST_LAUNCH(ps, kern, dim3(a.G), dim3(TPB), lds, a.stream, x, bcount, a.H, a.G,
                            static_cast<const T *>(a.gate), static_cast<const T *>(a.up),
                            static_cast<const T *>(a.down), a.n, a.n_dev, a.n_hint, comb, a.ldc, a.partials, a.act,
                            a.has_gate, gs_log2);
