@@ -560,7 +560,7 @@ __device__ __forceinline__ uint32_t pack_bits8(uint64_t ones)
 template <typename T, int RB, int TPB, int NB = 1, int NW = 1, int SPECN = RB / 2>
 __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     const uint8_t *__restrict__ new_mask, uint8_t *__restrict__ cur_mask2, int32_t *__restrict__ indices2,
-    int32_t *__restrict__ state, int I, int G, const T *__restrict__ x, int H, int B, int n_hint, int gs_log2,
+    int32_t *__restrict__ state, int I, int launch_word, const T *__restrict__ x, int H, int n_hint,
     T *__restrict__ combined, long ldc, float *__restrict__ partials, int act, int plan_bytes, FusedRows fr)
 {
     constexpr int VEC = Elem<T>::kVec;
@@ -578,9 +578,11 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     __shared__ PlanShared plan_shared;
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    // (what the first loads need comes first in the argument list, the number of blocks included: those arguments are
-    // in scalar registers when the wave starts, anything else -- the launch dimensions too -- arrives by a load)
+    // (what the first loads need comes first in the argument list, the number of blocks included: the first 14 dwords
+    // of the arguments are in scalar registers when the wave starts, anything else -- the launch dimensions too --
+    // arrives by a load that the first instructions would wait for.  Four small numbers share one of those dwords.)
     const int blk = blockIdx.x;
+    const int G = launch_word & 0xffff, gs_log2 = (launch_word >> 16) & 15, B = (launch_word >> 24) & 15;
     const int chunks = H / VEC;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
     const int GS = 1 << gs_log2, ngrp = TPB >> gs_log2, wpg = GS >> 6;
@@ -588,8 +590,8 @@ __global__ __launch_bounds__(TPB) void cache_sparse_decode_kernel(
     const bool valid = cc < chunks;
     const size_t coff = valid ? (size_t)cc * 16 : 0;
     const bool wave_live = __builtin_amdgcn_readfirstlane(cc & ~(kWave - 1)) < chunks;
-    const bool has_gate = fr.has_gate != 0;
-    const int row_bytes = fr.row_bytes;
+    const bool has_gate = ((launch_word >> 20) & 1) != 0;
+    const int row_bytes = H * (int)sizeof(T);
     const unsigned char *const pool_g = fr.pool_g, *const pool_u = fr.pool_u, *const pool_d = fr.pool_d;
     unsigned char *const act_g = fr.act_g, *const act_u = fr.act_u, *const act_d = fr.act_d;
     const int Q = (I + G - 1) / G;        // positions of this block: blk + G * q, q < Q (host: Q <= kSparseMaxQ)
@@ -1743,7 +1745,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
     static const bool fused_off = [] { const char *v = getenv("ST_CACHE_FUSED"); return v && atoi(v) == 0; }();
     // One kernel for one or two rows of x when a block owns at most kSparseMaxQ positions, the masks fit the
     // kernel's bitmaps and a row fits one pass of a thread group; everything else runs as two calls.
-    const bool fused = !fused_off && B <= 2 && aligned && I >= 8 && (I + G - 1) / G <= kSparseMaxQ &&
+    const bool fused = !fused_off && B <= 2 && aligned && I >= 8 && G <= 0xffff && (I + G - 1) / G <= kSparseMaxQ &&
                        I <= 32 * kSparseMaxW32 && I <= 8 * TPB * kSparseWords && chunks <= TPB && row_bytes % 16 == 0 &&
                        lds <= (size_t)(148 * 1024);
     if (!fused) {   // two launches: update, then the forward that reads the count on the device
@@ -1769,8 +1771,10 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
         auto launch = [&](auto kern, auto *xt, auto *ct) -> int {
             const int arc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), 148 * 1024);
             if (arc != ST_OK) return arc;
-            ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, mask, c->b.cur_mask, c->b.indices, c->b.state, I, G, xt,
-                      H, (int)B, hint, gs_log2, ct, (long)ldc, partials, act, (int)plan_bytes, fr);
+            // (blocks, log2 of the thread-group size, gated or not, rows of x: one argument, see the kernel)
+            const int launch_word = G | (gs_log2 << 16) | (fr.has_gate << 20) | ((int)B << 24);
+            ST_LAUNCH(ps, kern, dim3(G), dim3(TPB), lds, s, mask, c->b.cur_mask, c->b.indices, c->b.state, I,
+                      launch_word, xt, H, hint, ct, (long)ldc, partials, act, (int)plan_bytes, fr);
             return ST_OK;
         };
         int rc;

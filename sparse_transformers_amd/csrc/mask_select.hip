@@ -165,13 +165,15 @@ __device__ __forceinline__ int block_excl_count(int v, SelShared &sh, int tid)
 // row in index order.  KPT == 0: rows of any length, every pass reads the keys from LDS (`in_lds`) or the
 // scores again from memory.
 template <int KPT>
-__global__ __launch_bounds__(kSelThreads) void mask_select_kernel(const float *__restrict__ scores, int B, int I,
-                                                                  int method, long k_in, float z, int in_lds,
+__global__ __launch_bounds__(kSelThreads) void mask_select_kernel(const float *__restrict__ scores,
                                                                   uint8_t *__restrict__ mask,
+                                                                  uint8_t *__restrict__ rowmask,
                                                                   float *__restrict__ cutoff,
-                                                                  unsigned int *__restrict__ ticket,
-                                                                  uint8_t *__restrict__ rowmask, int ldm)
+                                                                  unsigned int *__restrict__ ticket, int B, int I,
+                                                                  int ldm, int method_word, long k_in, float z)
 {
+    // (pointers and sizes first: the first 14 dwords of the arguments are in scalar registers when the wave starts)
+    const int method = method_word & 0xff, in_lds = (method_word >> 8) & 1;
     constexpr int NR = KPT > 0 ? KPT : 1;
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ SelShared sh;
@@ -450,7 +452,7 @@ extern "C" int st_mask_select(const float *scores, int64_t B, int64_t I, int met
     }
     ProfScope ps(ST_K_MASK_SELECT, s);
     const dim3 grid((unsigned)B), block(kSelThreads);
-#define ST_SELECT_ARGS(in_lds) scores, (int)B, (int)I, method, (long)k, z, in_lds, mask, cutoff, ticket, rowmask, ldm
+#define ST_SELECT_ARGS(in_lds) scores, mask, rowmask, cutoff, ticket, (int)B, (int)I, ldm, method | ((in_lds) << 8), (long)k, z
     if (I <= 8 * kSelThreads)
         ST_LAUNCH(ps, (mask_select_kernel<8>), grid, block, (size_t)I * 4, s, ST_SELECT_ARGS(1));
     else if (I <= 16 * kSelThreads)

@@ -45,17 +45,23 @@ template <int RB, int CPT> struct RowBatch {
 // measures faster when all rows of a block fit in it).
 template <typename T, int NB, int RB, int CPT, int TPB, bool DB>
 __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
-    const T *__restrict__ x, int B, int H, int G, const T *__restrict__ gate, const T *__restrict__ up,
-    const T *__restrict__ down, int n_host, const int *__restrict__ n_dev, int n_hint, T *__restrict__ combined,
-    long ldc, float *__restrict__ partials, int act, int has_gate, int gs_log2)
+    const T *__restrict__ x, const T *__restrict__ gate, const T *__restrict__ up, const T *__restrict__ down,
+    const int *__restrict__ n_dev, int H, int launch_word, int n_spec, int n_host, T *__restrict__ combined,
+    long ldc, float *__restrict__ partials, int act)
 {
+    // (the first 14 dwords of the arguments are in scalar registers when the wave starts: everything the first loads
+    // need is among them -- the number of blocks, the thread-group size, the gate flag and the rows of x share one
+    // dword, and the host passes the row count to request ahead of the device's count, `n_spec`, ready-made; later
+    // arguments arrive by a load)
+    const int G = launch_word & 0xffff, gs_log2 = (launch_word >> 16) & 15, B = (launch_word >> 24) & 15;
+    const bool has_gate = ((launch_word >> 20) & 1) != 0;
     constexpr int VEC = Elem<T>::kVec;
     extern __shared__ __align__(16) unsigned char region[];  // group combine buffer
     __shared__ float red[TPB / kWave][RB][NB][2];             // per-wave partial (g,u)
     __shared__ float hs[TPB / kWave][RB][NB];                 // h of the rows being computed
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const int blk = blockIdx.x;  // G: the grid's size, passed as an argument so that it arrives preloaded
+    const int blk = blockIdx.x;
     // Active count: requested first, consumed only after the first two batches
     // of weight loads have been issued.  Rows are dealt to blocks round-robin,
     // so which rows a block owns does not depend on the count, and rows below
@@ -63,7 +69,6 @@ __global__ __launch_bounds__(TPB) void mlp_decode_kernel(
     // buffers hold I rows, so this is safe).
     ST_TL(0);
     const int nd_raw = n_dev ? *n_dev : n_host;
-    const int n_spec = n_dev ? (n_hint < n_host ? n_hint : n_host) : n_host;
     const int chunks = H / VEC;
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
 
@@ -337,12 +342,14 @@ static int launch_inst(const MlpLaunch &a, int b0, int bcount)
     }
     const T *x = static_cast<const T *>(a.x) + (size_t)b0 * a.H;
     T *comb = a.combined ? static_cast<T *>(a.combined) + (size_t)b0 * a.ldc : nullptr;
+    ST_REQUIRE(a.G <= 0xffff, "st_mlp_forward: %d blocks", a.G);
+    const int launch_word = a.G | (gs_log2 << 16) | ((a.has_gate ? 1 : 0) << 20) | (bcount << 24);
+    const int n_spec = a.n_dev ? (a.n_hint < a.n ? a.n_hint : a.n) : a.n;   // rows requested ahead of the device's count
     {
         ProfScope ps(ST_K_MLP_DECODE, a.stream);
-        ST_LAUNCH(ps, kern, dim3(a.G), dim3(TPB), lds, a.stream, x, bcount, a.H, a.G,
-                           static_cast<const T *>(a.gate), static_cast<const T *>(a.up),
-                           static_cast<const T *>(a.down), a.n, a.n_dev, a.n_hint, comb, a.ldc, a.partials, a.act,
-                           a.has_gate, gs_log2);
+        ST_LAUNCH(ps, kern, dim3(a.G), dim3(TPB), lds, a.stream, x, static_cast<const T *>(a.gate),
+                  static_cast<const T *>(a.up), static_cast<const T *>(a.down), a.n_dev, a.H, launch_word, n_spec,
+                  a.n, comb, a.ldc, a.partials, a.act);
     }
     ST_HIP(hipGetLastError());
     T *out = static_cast<T *>(a.out) + (size_t)b0 * a.H;

@@ -173,14 +173,16 @@ __device__ __forceinline__ int pf_swz(int row) { return (row >> 1) & 7; }
 // JN = 16-row tiles of gate and of up per wave: 2 (64 rows of each per block) or, to make more blocks out of
 // few rows, 1 (32 rows of each).
 template <typename T, bool HG, int BM, int NS, int KS, int JN>
-__global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__restrict__ X, int M, int H,
+__global__ __launch_bounds__(2 * BM * KS) void prefill_gateup_kernel(const T *__restrict__ X,
                                                                      const T *__restrict__ gate,
-                                                                     const T *__restrict__ up, int n_host,
-                                                                     const int *__restrict__ n_dev,
+                                                                     const T *__restrict__ up,
+                                                                     const int *__restrict__ n_dev, int M, int H,
+                                                                     int n_host, int jt, int mt,
                                                                      T *__restrict__ Hh, long ldh,
-                                                                     T *__restrict__ comb, long ldc, int act, int jt,
-                                                                     int mt)
+                                                                     T *__restrict__ comb, long ldc, int act)
 {
+    // (operands, sizes and the tile grid first: the first 14 dwords of the arguments are in scalar registers when the
+    // wave starts; what only the epilogue needs arrives by a load)
     constexpr int kThreads = 2 * BM;                     // per K group
     constexpr int kWR = 32 * JN;                         // rows of gate and of up per block
     constexpr int kRows = BM + (HG ? 2 : 1) * kWR;       // LDS rows of one buffer: x, gate, up
@@ -386,13 +388,13 @@ __device__ __forceinline__ void pf_load_to_lds(unsigned dst, unsigned off, const
 }
 
 template <typename T, bool HG>
-__global__ __launch_bounds__(kPwThreads) void prefill_gateup_wide_kernel(const T *__restrict__ X, int M, int H,
+__global__ __launch_bounds__(kPwThreads) void prefill_gateup_wide_kernel(const T *__restrict__ X,
                                                                          const T *__restrict__ gate,
-                                                                         const T *__restrict__ up, int n_host,
-                                                                         const int *__restrict__ n_dev,
+                                                                         const T *__restrict__ up,
+                                                                         const int *__restrict__ n_dev, int M, int H,
+                                                                         int n_host, int jt, int mt,
                                                                          T *__restrict__ Hh, long ldh,
-                                                                         T *__restrict__ comb, long ldc, int act,
-                                                                         int jt, int mt)
+                                                                         T *__restrict__ comb, long ldc, int act)
 {
     constexpr int kRows = kPwBM + (HG ? 2 : 1) * kPwWR;   // LDS rows of one buffer: x, gate, up
     constexpr int kBuf = kRows * kPfLd1;                  // 16-byte units per buffer
@@ -592,11 +594,11 @@ constexpr int kPfLdB = 18;   // Wd rows in LDS: 16 chunks + 2 of padding (288 by
 typedef short pf_v4i16_t __attribute__((ext_vector_type(4)));
 
 template <typename T>
-__global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__restrict__ Hh, long ldh, int M,
-                                                                     const T *__restrict__ Wd, int H, int n_host,
-                                                                     const int *__restrict__ n_dev,
-                                                                     T *__restrict__ Out, float *__restrict__ partial,
-                                                                     int split_k, int ct, int mt)
+__global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__restrict__ Hh,
+                                                                     const T *__restrict__ Wd,
+                                                                     const int *__restrict__ n_dev, long ldh, int M,
+                                                                     int H, int n_host, int split_k, int ct, int mt,
+                                                                     T *__restrict__ Out, float *__restrict__ partial)
 {
     constexpr int NS = 2;
     __shared__ uint4 lds[2 * kPfBM * kPfLd1 + 2 * kPfBK2 * kPfLdB];
@@ -742,12 +744,12 @@ __global__ __launch_bounds__(kPfThreads, 2) void prefill_down_kernel(const T *__
 __device__ __forceinline__ int pf_swz_b(int k) { return 2 * ((k & 3) | (((k >> 3) & 1) << 2)); }
 
 template <typename T>
-__global__ __launch_bounds__(kPwThreads) void prefill_down_wide_kernel(const T *__restrict__ Hh, long ldh, int M,
-                                                                       const T *__restrict__ Wd, int H, int n_host,
-                                                                       const int *__restrict__ n_dev,
+__global__ __launch_bounds__(kPwThreads) void prefill_down_wide_kernel(const T *__restrict__ Hh,
+                                                                       const T *__restrict__ Wd,
+                                                                       const int *__restrict__ n_dev, long ldh, int M,
+                                                                       int H, int n_host, int split_k, int ct, int mt,
                                                                        T *__restrict__ Out,
-                                                                       float *__restrict__ partial, int split_k,
-                                                                       int ct, int mt)
+                                                                       float *__restrict__ partial)
 {
     constexpr int kABuf = kPwBM * kPfLd1;             // 16-byte units of the Hh tile of a stage (32 KB)
     constexpr int kBuf = kABuf + kPfBK2 * 16;         // + 64 rows of Wd x 256 bytes (16 KB)
@@ -1047,9 +1049,9 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         const int mt = big ? (M + 255) / 256 : quarters ? (M + 63) / 64 : mt128;
         const int grid = (jt * mt + kXcds - 1) / kXcds * kXcds;
         auto go = [&](auto kern, int threads) -> int {
-            ST_LAUNCH(ps, kern, dim3(grid), dim3(threads), 0, stream, static_cast<const T *>(x), M, H,
-                      static_cast<const T *>(gate), static_cast<const T *>(up), n, n_dev, Hh, ldh,
-                      static_cast<T *>(comb), ldc, act, jt, mt);
+            ST_LAUNCH(ps, kern, dim3(grid), dim3(threads), 0, stream, static_cast<const T *>(x),
+                      static_cast<const T *>(gate), static_cast<const T *>(up), n_dev, M, H, n, jt, mt, Hh, ldh,
+                      static_cast<T *>(comb), ldc, act);
             return ST_OK;
         };
         int rc;
@@ -1066,13 +1068,13 @@ static int launch_prefill_t(const void *x, int M, int H, const void *gate, const
         if (wide_down) {
             const int ct = (H + kPfBN - 1) / kPfBN, mt = (M + kPwBM - 1) / kPwBM;
             const int grid = (ct * mt * split_k + kXcds - 1) / kXcds * kXcds;
-            ST_LAUNCH(ps, prefill_down_wide_kernel<T>, dim3(grid), dim3(kPwThreads), 0, stream, Hh, ldh, M,
-                      static_cast<const T *>(down), H, n, n_dev, static_cast<T *>(out), partial, split_k, ct, mt);
+            ST_LAUNCH(ps, prefill_down_wide_kernel<T>, dim3(grid), dim3(kPwThreads), 0, stream, Hh,
+                      static_cast<const T *>(down), n_dev, ldh, M, H, n, split_k, ct, mt, static_cast<T *>(out), partial);
         } else {
             const int ct = (H + kPfBN - 1) / kPfBN, mt = (M + kPfBM - 1) / kPfBM;
             const int grid = (ct * mt * split_k + kXcds - 1) / kXcds * kXcds;
-            ST_LAUNCH(ps, prefill_down_kernel<T>, dim3(grid), dim3(kPfThreads), 0, stream, Hh, ldh, M,
-                      static_cast<const T *>(down), H, n, n_dev, static_cast<T *>(out), partial, split_k, ct, mt);
+            ST_LAUNCH(ps, prefill_down_kernel<T>, dim3(grid), dim3(kPfThreads), 0, stream, Hh,
+                      static_cast<const T *>(down), n_dev, ldh, M, H, n, split_k, ct, mt, static_cast<T *>(out), partial);
         }
     }
     ST_HIP(hipGetLastError());

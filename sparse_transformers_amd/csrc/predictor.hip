@@ -92,12 +92,14 @@ constexpr int kPredUpBTile = 8;
 // passes); a wave owns RPW consecutive rows and issues the loads of all of them
 // before the rank-r intermediate is staged in LDS.
 template <typename T, int LPR, int RPW>
-__global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_kernel(const float *__restrict__ t, int B, int r,
-                                                                  const T *__restrict__ Bm, int I, float thr,
-                                                                  int cmp_ge, float *__restrict__ scores,
-                                                                  uint8_t *__restrict__ mask, int round_storage,
-                                                                  int accumulate)
+__global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_kernel(const float *__restrict__ t,
+                                                                  const T *__restrict__ Bm,
+                                                                  float *__restrict__ scores,
+                                                                  uint8_t *__restrict__ mask, int B, int r, int I,
+                                                                  float thr, int flags)
 {
+    // (13 dwords of arguments, all of them in scalar registers when the wave starts; the three switches share one)
+    const int cmp_ge = flags & 1, round_storage = (flags >> 1) & 1, accumulate = (flags >> 2) & 1;
     constexpr int VEC = Elem<T>::kVec;
     constexpr int RPI = kWave / LPR;                                          // rows per iteration
     constexpr int NIT = RPW / RPI > 0 ? RPW / RPI : 1;  // iterations per tile
@@ -196,12 +198,13 @@ __global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_kernel(const
 // strides, half the banks idle) and took 1.3 us per additional row of x at r = 256.  All NITER row loads of a
 // wave are issued before anything else.
 template <typename T, int LPR, int NITER>
-__global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_rows_kernel(const float *__restrict__ t, int B, int r,
-                                                                       const T *__restrict__ Bm, int I, float thr,
-                                                                       int cmp_ge, float *__restrict__ scores,
-                                                                       uint8_t *__restrict__ mask, int round_storage,
-                                                                       int accumulate)
+__global__ __launch_bounds__(kPredUpThreads) void predictor_up_mask_rows_kernel(const float *__restrict__ t,
+                                                                       const T *__restrict__ Bm,
+                                                                       float *__restrict__ scores,
+                                                                       uint8_t *__restrict__ mask, int B, int r, int I,
+                                                                       float thr, int flags)
 {
+    const int cmp_ge = flags & 1, round_storage = (flags >> 1) & 1, accumulate = (flags >> 2) & 1;   // (as above)
     constexpr int VEC = Elem<T>::kVec;
     constexpr int RPI = kWave / LPR;   // rows per iteration
     extern __shared__ __align__(16) unsigned char smem[];
@@ -282,7 +285,8 @@ static void launch_up_rpw(ProfScope &ps, const float *t_ws, int B, int r, const 
     const size_t lds = ((size_t)B * r * sizeof(float) + batch - 1) / batch * batch;
     constexpr int rows = RPW * (kPredUpThreads / kWave);
     ST_LAUNCH(ps, (predictor_up_mask_kernel<T, LPR, RPW>), dim3((I + rows - 1) / rows), dim3(kPredUpThreads), lds,
-              stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask, round_storage, accumulate);
+              stream, t_ws, static_cast<const T *>(Bm), scores, mask, B, r, I, thr,
+              (cmp_ge ? 1 : 0) | (round_storage ? 2 : 0) | (accumulate ? 4 : 0));
 }
 
 template <typename T, int LPR>
@@ -295,7 +299,8 @@ static void launch_up(ProfScope &ps, const float *t_ws, int B, int r, const void
         const size_t lds = ((size_t)B * r * sizeof(float) + batch - 1) / batch * batch;
         constexpr int rows = (kWave / LPR) * NITER * (kPredUpThreads / kWave);
         ST_LAUNCH(ps, (predictor_up_mask_rows_kernel<T, LPR, NITER>), dim3((I + rows - 1) / rows), dim3(kPredUpThreads),
-                  lds, stream, t_ws, B, r, static_cast<const T *>(Bm), I, thr, cmp_ge, scores, mask, round_storage, accumulate);
+                  lds, stream, t_ws, static_cast<const T *>(Bm), scores, mask, B, r, I, thr,
+                  (cmp_ge ? 1 : 0) | (round_storage ? 2 : 0) | (accumulate ? 4 : 0));
         return;
     }
     launch_up_rpw<T, LPR, pred_rows_per_wave(LPR)>(ps, t_ws, B, r, Bm, I, thr, cmp_ge, scores, mask, round_storage,
