@@ -1752,7 +1752,7 @@ extern "C" int st_cache_update_forward(st_cache *c, const uint8_t *mask, const v
         const int rc = st_cache_update_async(c, mask, stream);
         if (rc != ST_OK) return rc;
         return st_mlp_forward(x, B, c->H, c->b.gate_active, c->b.up_active, c->b.down_active, c->I,
-                              c->b.state + ST_STATE_N_ACTIVE, 0, out, combined, ldc, workspace, workspace_bytes, act,
+                              c->b.state + ST_STATE_N_ACTIVE, n_hint, out, combined, ldc, workspace, workspace_bytes, act,
                               c->dtype, c->has_gate, stream);
     }
     FusedRows fr;

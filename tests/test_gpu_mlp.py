@@ -139,6 +139,34 @@ def test_device_count_and_hint_paths():
     assert not out.any()                                       # empty active set -> zeros
 
 
+@pytest.mark.parametrize("B,H,dt", [(4, 3072, "float16"), (20, 2048, "bfloat16"), (6, 1536, "bfloat16")])
+def test_batch_device_count_and_hint_paths(B, H, dt):
+    """The batch kernels deal rows to blocks for the count the host expects before the device's count has arrived:
+    whatever that guess (absent, too low, exact, too high), the result carries the bits of a call with the exact host
+    count, and an empty set gives zeros."""
+    I, n = 4096, 1777
+    dtype = getattr(torch, dt)
+    g = torch.Generator().manual_seed(5)
+    gate = (torch.randn(I, H, generator=g) * 0.02).to(dtype).to(DEV)
+    up = (torch.randn(I, H, generator=g) * 0.02).to(dtype).to(DEV)
+    dn = (torch.randn(I, H, generator=g) * 0.02).to(dtype).to(DEV)
+    x = torch.randn(B, H, generator=g).to(dtype).to(DEV)
+    n_dev = torch.tensor([n], dtype=torch.int32, device=DEV)
+    ref = torch.empty(B, H, dtype=dtype, device=DEV)
+    mlp_forward_rows(x, gate, up, dn, n, None, ref, None, "silu", True)
+    want, _ = oracle.mlp_forward(x.float().cpu().numpy(), torch.cat([gate[:n], up[:n]]).float().cpu().numpy(),
+                                 dn[:n].float().cpu().numpy().T, "silu", True)
+    assert_close(ref.float().cpu().numpy(), want, dt, "host count")
+    for hint in (0, 1, 900, n - 1, n, n + 1, n + 700, I):
+        out = torch.full((B, H), float("nan"), dtype=dtype, device=DEV)
+        mlp_forward_rows(x, gate, up, dn, I, n_dev, out, None, "silu", True, n_hint=hint)
+        assert torch.equal(out, ref), f"hint {hint}"
+    n_dev.fill_(0)
+    out = torch.full((B, H), 1.0, dtype=dtype, device=DEV)
+    mlp_forward_rows(x, gate, up, dn, I, n_dev, out, None, "silu", True, n_hint=n)
+    assert not out.any()                                       # empty active set -> zeros
+
+
 def test_float64_device_count_and_empty_set():
     """Double precision with the count on the device: rows beyond it are ignored, the result carries the same bits
     as with the host's count (fixed summation order), and an empty set gives zeros."""
